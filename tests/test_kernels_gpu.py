@@ -1,0 +1,229 @@
+"""Each HIP kernel alone against its plain torch reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+from kernel_refs import PlainOps
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tokenizer_amd.kernels import get_ops
+    return get_ops()
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return PlainOps(torch.float64)
+
+
+def tol(dtype):
+    # float32: rounding of sums of a few hundred terms; bfloat16: one rounding of the output (2^-9 relative).
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=8e-3, atol=1e-3)
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=gen) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(ops, ref, dtype):
+    table = rand((1000, 200), dtype, 1)
+    ids = torch.tensor([0, 999, 5, 5, 17, 400, 123] * 5 + [1, 2], dtype=torch.int32).cuda()
+    out = torch.empty((ids.numel(), 200), dtype=torch.float32).cuda()
+    ops.embedding(ids, table, out)
+    want = torch.empty_like(out)
+    ref.embedding(ids, table, want)
+    assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [200, 896, 72])
+def test_add_rmsnorm(ops, ref, dtype, hidden):
+    residual = rand((33, hidden), torch.float32, 2, 3.0)
+    delta = rand((33, hidden), dtype, 3)
+    weight = rand((hidden,), torch.float32, 4) + 1
+    for use_delta in (True, False):
+        res_a, res_b = residual.clone(), residual.clone()
+        out_a = torch.empty((33, hidden), dtype=dtype).cuda()
+        out_b = torch.empty_like(out_a)
+        ops.add_rmsnorm(res_a, delta if use_delta else None, weight, 1e-5, out_a)
+        ref.add_rmsnorm(res_b, delta if use_delta else None, weight, 1e-5, out_b)
+        torch.testing.assert_close(res_a, res_b, rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(out_a.float(), out_b.float(), **tol(dtype))
+    rows = torch.tensor([32, 0, 7, 7], dtype=torch.int32).cuda()
+    res_a = residual.clone()
+    out_a = torch.empty((4, hidden), dtype=dtype).cuda()
+    out_b = torch.empty_like(out_a)
+    ops.add_rmsnorm(res_a, delta, weight, 1e-6, out_a, rows, store_residual=False)
+    ref.add_rmsnorm(residual.clone(), delta, weight, 1e-6, out_b, rows, store_residual=False)
+    assert torch.equal(res_a, residual), "a row subset must leave the residual alone"
+    torch.testing.assert_close(out_a.float(), out_b.float(), **tol(dtype))
+
+
+def test_rmsnorm_eps_matters(ops):
+    # Tiny inputs: the result is x / sqrt(eps) when mean(x^2) << eps, so a misplaced eps shows.
+    x = torch.full((1, 64), 1e-6).cuda()
+    w = torch.ones(64).cuda()
+    out = torch.empty((1, 64)).cuda()
+    ops.add_rmsnorm(x, None, w, 1e-4, out)
+    torch.testing.assert_close(out, torch.full((1, 64), 1e-6 / math.sqrt(1e-12 + 1e-4)).cuda(), rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_gate(ops, ref, dtype):
+    x = rand((19, 2 * 272), dtype, 5, 2.0)
+    out_a = torch.empty((19, 272), dtype=dtype).cuda()
+    out_b = torch.empty_like(out_a)
+    ops.silu_gate(x, out_a)
+    ref.silu_gate(x, out_b)
+    torch.testing.assert_close(out_a.float(), out_b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(6, 2, 48, 16), (3, 1, 32, 16), (4, 4, 128, 32)])
+def test_rope_store(ops, ref, dtype, geometry):
+    n_q, n_kv, d, page_size = geometry
+    n_tokens, n_pages, max_pos = 21, 9, 400
+    width = (n_q + 2 * n_kv) * d
+    qkv = rand((n_tokens, width), dtype, 6)
+    bias = rand((width,), torch.float32, 7)
+    positions = torch.randint(0, max_pos, (n_tokens,), generator=torch.Generator().manual_seed(8)).int().cuda()
+    inv = torch.tensor([1.0 / (10000.0 ** (i / d)) for i in range(0, d, 2)], dtype=torch.float64).float()
+    ang = torch.arange(max_pos).float()[:, None] * inv[None]
+    cos_sin = torch.cat([ang.cos(), ang.sin()], 1).cuda()
+    perm = torch.randperm(n_pages * page_size, generator=torch.Generator().manual_seed(9))[:n_tokens]
+    slots = perm.int().cuda()
+    slots[3] = -1
+    for use_bias, use_rot in ((True, True), (False, True), (False, False)):
+        a, b = qkv.clone(), qkv.clone()
+        ka = torch.zeros((n_pages, n_kv, page_size, d), dtype=dtype).cuda()
+        va, kb, vb = ka.clone(), ka.clone(), ka.clone()
+        args = (bias if use_bias else None, positions, cos_sin if use_rot else None, slots)
+        ops.rope_store(a, *args, ka, va, n_q, n_kv, d)
+        ref.rope_store(b, *args, kb, vb, n_q, n_kv, d)
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+        torch.testing.assert_close(ka.float(), kb.float(), **tol(dtype))
+        torch.testing.assert_close(va.float(), vb.float(), **tol(dtype))
+    # Without slots nothing is stored.
+    a = qkv.clone()
+    ops.rope_store(a, None, positions, cos_sin, None, None, None, n_q, n_kv, d)
+    b = qkv.clone()
+    ref.rope_store(b, None, positions, cos_sin, None, None, None, n_q, n_kv, d)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
+def make_paged_case(dtype, n_q, n_kv, d, page_size, lengths, q_lens, seed):
+    """Requests of the given lengths whose last q_lens tokens are queried; pages scattered at random."""
+    gen = torch.Generator().manual_seed(seed)
+    n_entries = len(lengths)
+    pages_each = [-(-n // page_size) for n in lengths]
+    n_pages = sum(pages_each) + 3
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    width = max(pages_each)
+    table = torch.full((n_entries, width), -1, dtype=torch.int32)
+    k_pages = torch.randn((n_pages, n_kv, page_size, d), generator=gen).to(dtype)
+    v_pages = torch.randn((n_pages, n_kv, page_size, d), generator=gen).to(dtype)
+    positions, entry_of_token = [], []
+    for e, (length, q_len) in enumerate(zip(lengths, q_lens)):
+        for i in range(pages_each[e]):
+            table[e, i] = order.pop()
+        positions += list(range(length - q_len, length))
+        entry_of_token += [e] * q_len
+    n_tokens = len(positions)
+    qkv = torch.randn((n_tokens, (n_q + 2 * n_kv) * d), generator=gen).to(dtype)
+    return (qkv.cuda(), k_pages.cuda(), v_pages.cuda(), torch.tensor(positions, dtype=torch.int32).cuda(),
+            torch.tensor(entry_of_token, dtype=torch.int32).cuda(), table.cuda())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(6, 3, 48, 16), (3, 1, 32, 16), (8, 2, 128, 32), (14, 2, 64, 16)])
+@pytest.mark.parametrize("window", [None, 37])
+def test_paged_attention(ops, ref, dtype, geometry, window):
+    n_q, n_kv, d, page_size = geometry
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        dtype, n_q, n_kv, d, page_size, lengths=[1, 300, 64, 17], q_lens=[1, 5, 64, 1], seed=11)
+    out_a = torch.empty((qkv.shape[0], n_q * d), dtype=dtype).cuda()
+    out_b = torch.empty_like(out_a)
+    scale = 1.0 / math.sqrt(d)
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
+    ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
+    torch.testing.assert_close(out_a.float(), out_b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key(ops, dtype):
+    # One key far back is made to dominate: the output must be its value row.
+    n_q, n_kv, d, page_size = 4, 2, 64, 16
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        dtype, n_q, n_kv, d, page_size, lengths=[700], q_lens=[1], seed=12)
+    target = 123
+    page, off = int(table[0, target // page_size]), target % page_size
+    q = qkv[0, :n_q * d].reshape(n_q, d).float()
+    for h in range(n_q):
+        k_pages[page, h // 2, off] = 0
+    k_pages[page, 0, off] = (q[0] * 40 / q[0].norm()).to(dtype)
+    qkv[0, d:2 * d] = qkv[0, :d]            # head 1 shares kv head 0 and looks the same way
+    k_pages[page, 1, off] = (q[2] * 40 / q[2].norm()).to(dtype)
+    qkv[0, 3 * d:4 * d] = qkv[0, 2 * d:3 * d]
+    out = torch.empty((1, n_q * d), dtype=dtype).cuda()
+    ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, None, 1.0)
+    got = out.reshape(n_q, d).float()
+    for h in range(n_q):
+        torch.testing.assert_close(got[h], v_pages[page, h // 2, off].float(), rtol=2e-2, atol=2e-2)
+    # With a window that ends just after the key, it is gone: position 699 sees keys >= 699 - w.
+    ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, 699 - target - 1, 1.0)
+    assert (out.reshape(n_q, d).float()[0] - v_pages[page, 0, off].float()).abs().max() > 0.1
+    ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, 699 - target, 1.0)
+    torch.testing.assert_close(out.reshape(n_q, d).float()[0], v_pages[page, 0, off].float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 100, 72), (37, 200, 136), (130, 260, 272), (300, 1000, 64), (64, 151, 896),
+                                   (8, 384, 96), (513, 130, 40)])
+def test_linear(ops, ref, dtype, shape):
+    m, n, k = shape
+    x = rand((m, k), dtype, 20)
+    w = rand((n, k), dtype, 21, 0.1)
+    bias = rand((n,), torch.float32, 22)
+    for use_bias in (True, False):
+        for out_dtype in ([torch.float32] if dtype == torch.float32 else [torch.bfloat16, torch.float32]):
+            got = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
+            want = ref.linear(x, w, bias if use_bias else None, out_dtype=torch.float64)
+            torch.testing.assert_close(got.double(), want, **tol(out_dtype))
+    # Rows of a wider buffer.
+    wide = rand((m, k + 24), dtype, 23)
+    got = ops.linear(wide[:, :k], w, None, out_dtype=torch.float32)
+    want = ref.linear(wide[:, :k], w, None, out_dtype=torch.float64)
+    torch.testing.assert_close(got.double(), want, **tol(torch.float32))
+
+
+def test_linear_float32_is_true_float32(ops):
+    # Inputs whose products need all 24 bits: a reduced-precision matrix mode would lose them.
+    k = 64
+    x = (1 + torch.arange(k, dtype=torch.float64) * 2.0 ** -20).float().reshape(1, k).cuda()
+    w = (1 - torch.arange(k, dtype=torch.float64) * 2.0 ** -21).float().reshape(1, k).cuda()
+    got = ops.linear(x, w, None)
+    want = (x.double() * w.double()).sum()
+    assert abs(float(got) - float(want)) < 1e-5 * float(want) * 0.01
+
+
+def test_argmax_first_maximum_wins(ops):
+    logits = torch.full((5, 3000), -1.0)
+    logits[0, 2999] = 3.0
+    logits[1, 7] = 2.0
+    logits[1, 2000] = 2.0          # tie: the lower index
+    logits[2, 1500] = 2.0
+    logits[2, 1499] = 2.0
+    logits[3] = 0.0                # all equal: index 0
+    logits[4] = float("-inf")      # a scan with `>` from -inf never moves: index 0
+    out = ops.argmax(logits.cuda()).cpu().tolist()
+    assert out == [2999, 7, 1499, 0, 0]
+    small = torch.tensor([[0.2, 1.5, 1.5, -3.0, 0.0]]).cuda()   # qwen-infer/src/sample.rs:191-192
+    assert ops.argmax(small).item() == 1

@@ -1,0 +1,44 @@
+"""Device memory of the cache: pages of keys and values per group, and per-request state slots."""
+from __future__ import annotations
+
+import torch
+
+from .manager import CacheManager
+
+_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+class CachePools:
+    """For group g: `pages[g]` of shape [layers in g, 2, num_pages, n_kv, page_size, d] (keys at 0, values
+    at 1) in the compute dtype.  For a layer with fixed-size state: `states[layer]` of shape
+    [max_requests, *state_shape]."""
+
+    def __init__(self, manager: CacheManager, needs, dtype: torch.dtype, device):
+        self.manager = manager
+        self.pages = []
+        for group in manager.groups:
+            need = group.need
+            self.pages.append(torch.zeros((len(group.layers), 2, manager.num_pages, need.n_kv_heads,
+                                           manager.page_size, need.head_dim), dtype=dtype, device=device))
+        self.states = {}
+        for layer, need in enumerate(needs):
+            if need.state_shape is not None:
+                self.states[layer] = torch.zeros((manager.max_requests, *need.state_shape),
+                                                 dtype=_STATE_DTYPES[need.state_dtype], device=device)
+
+    def layer_pages(self, layer: int):
+        """(keys, values) of one layer, each [num_pages, n_kv, page_size, d], or (None, None)."""
+        group = self.manager.group_of_layer[layer]
+        if group is None:
+            return None, None
+        index = self.manager.groups[group].layers.index(layer)
+        return self.pages[group][index, 0], self.pages[group][index, 1]
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.pages) + \
+            sum(t.numel() * t.element_size() for t in self.states.values())
+
+    def poison(self, value: float = float("nan")) -> None:
+        """Fill every page with a value that shows if a kernel reads what no request wrote."""
+        for tensor in self.pages:
+            tensor.fill_(value)

@@ -1,0 +1,90 @@
+// Embedding gather, residual-add + RMSNorm, gated activation.
+#include "common.h"
+
+// out[t, :] = table[ids[t], :] widened to float (the residual stream is float).
+template <typename T>
+__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  if (id < 0 || id >= vocab) id = 0;  // the host rejects such ids before the launch
+  const T* row = table + (size_t)id * hidden;
+  float* dst = out + (size_t)t * hidden;
+  for (int h = threadIdx.x; h < hidden; h += blockDim.x) dst[h] = ld(row + h);
+}
+
+// For output row i: r = rows ? rows[i] : i;  x = residual[r] (+ delta[r]);
+// if store_residual: residual[r] = x;  out[i] = x / sqrt(mean(x^2) + eps) * weight.
+// Sum of squares, root and scaling are float.
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                   const float* __restrict__ weight, T* __restrict__ out,
+                                   const int* __restrict__ rows, int hidden, float eps, int store_residual) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* res = residual + (size_t)r * hidden;
+  const T* del = delta ? delta + (size_t)r * hidden : nullptr;
+  float sq = 0.f;
+  for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+    float x = res[h];
+    if (del) x += ld(del + h);
+    sq += x * x;
+  }
+  const float total = block_sum(sq, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+  for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+    float x = res[h];
+    if (del) x += ld(del + h);
+    if (store_residual) res[h] = x;
+    st(dst + h, x * inv * weight[h]);
+  }
+}
+
+// out[t, j] = silu(in[t, j]) * in[t, inner + j], silu(z) = z * sigmoid(z), in float.
+template <typename T>
+__global__ void silu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, int inner, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inner;
+    const int j = (int)(idx - t * inner);
+    const float g = ld(in + t * 2 * inner + j);
+    const float u = ld(in + t * 2 * inner + inner + j);
+    st(out + idx, g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ta_embedding(const void* ids, const void* table, void* out, int n_tokens, int hidden,
+                            int vocab, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (dtype == DT_F32)
+    embedding_kernel<float><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab);
+  else
+    embedding_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_add_rmsnorm(void* residual, const void* delta, const void* weight, void* out,
+                              const void* rows, int n_rows, int hidden, float eps, int store_residual,
+                              int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (dtype == DT_F32)
+    add_rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)delta, (const float*)weight,
+                                                          (float*)out, (const int*)rows, hidden, eps, store_residual);
+  else
+    add_rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((float*)residual, (const bf16_t*)delta, (const float*)weight,
+                                                           (bf16_t*)out, (const int*)rows, hidden, eps, store_residual);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_silu_gate(const void* in, void* out, int n_tokens, int inner, int dtype, hipStream_t stream) {
+  const size_t total = (size_t)n_tokens * inner;
+  if (total == 0) return 0;
+  const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+  if (dtype == DT_F32)
+    silu_gate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, inner, total);
+  else
+    silu_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner, total);
+  return LAUNCH_STATUS();
+}

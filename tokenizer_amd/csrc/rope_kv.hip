@@ -1,0 +1,66 @@
+// Position encoding of queries and keys (half-split rotation) fused with the write of keys and
+// values into their pages.  One block per (token, head); heads are laid out q heads, k heads, v heads
+// in a row of the fused projection output.
+#include "common.h"
+
+// qkv: [n_tokens, row_stride], heads of size d.  bias (float, may be null) is added first.
+// cos_sin: [max_positions, d] float, cos of the d/2 angles then sin; null = no rotation.
+// slots: physical slot of each token (page * page_size + offset), or null = nothing is stored.
+// Pages: [n_pages, n_kv, page_size, d].
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
+                                  const int* __restrict__ positions, const float* __restrict__ cos_sin,
+                                  const int* __restrict__ slots, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                  int n_q, int n_kv, int d, int page_size) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;  // 0..n_q-1 q, then n_kv k heads, then n_kv v heads
+  T* x = qkv + (size_t)t * row_stride + (size_t)head * d;
+  const float* b = bias ? bias + (size_t)head * d : nullptr;
+  const int half = d / 2;
+  const bool is_v = head >= n_q + n_kv;
+  const bool is_k = !is_v && head >= n_q;
+  T* dst = nullptr;
+  if ((is_k || is_v) && slots) {
+    const int slot = slots[t];
+    if (slot >= 0) {
+      const int page = slot / page_size, off = slot - page * page_size;
+      const int kvh = is_k ? head - n_q : head - n_q - n_kv;
+      dst = (is_k ? k_pages : v_pages) + (((size_t)page * n_kv + kvh) * page_size + off) * d;
+    }
+  }
+  if (is_v || !cos_sin) {
+    if (!b && !dst) return;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+      float v = ld(x + i);
+      if (b) { v += b[i]; st(x + i, v); }
+      if (dst) st(dst + i, v);
+    }
+    return;
+  }
+  const float* cs = cos_sin + (size_t)positions[t] * d;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float x1 = ld(x + i), x2 = ld(x + half + i);
+    if (b) { x1 += b[i]; x2 += b[half + i]; }
+    const float c = cs[i], s = cs[half + i];
+    const float r1 = x1 * c - x2 * s;
+    const float r2 = x2 * c + x1 * s;
+    st(x + i, r1);
+    st(x + half + i, r2);
+    if (dst) { st(dst + i, r1); st(dst + half + i, r2); }
+  }
+}
+
+extern "C" int ta_rope_store(void* qkv, int row_stride, const void* bias, const void* positions,
+                             const void* cos_sin, const void* slots, void* k_pages, void* v_pages,
+                             int n_tokens, int n_q, int n_kv, int d, int page_size, int dtype,
+                             hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  dim3 grid(n_tokens, n_q + 2 * n_kv);
+  if (dtype == DT_F32)
+    rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, row_stride, (const float*)bias, (const int*)positions,
+        (const float*)cos_sin, (const int*)slots, (float*)k_pages, (float*)v_pages, n_q, n_kv, d, page_size);
+  else
+    rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, row_stride, (const float*)bias, (const int*)positions,
+        (const float*)cos_sin, (const int*)slots, (bf16_t*)k_pages, (bf16_t*)v_pages, n_q, n_kv, d, page_size);
+  return LAUNCH_STATUS();
+}

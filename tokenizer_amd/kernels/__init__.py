@@ -1,0 +1,250 @@
+"""Bindings of the hand-written HIP kernels (loaded through ctypes).
+
+There is no fallback: without a GPU and the built library `get_ops()` raises.
+Every wrapper checks on the host that its operands have the shapes, dtypes and
+layout its kernel and grid assume, and launches on torch's current stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import threading
+
+import torch
+
+from . import build as _build
+
+_F32, _BF16 = 0, 1
+_CODES = {torch.float32: _F32, torch.bfloat16: _BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
+
+
+def _ptr(tensor: torch.Tensor | None) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+
+
+def _need(cond: bool, message: str) -> None:
+    if not cond:
+        raise KernelError(message)
+
+
+def _dev(*tensors: torch.Tensor | None) -> None:
+    for tensor in tensors:
+        if tensor is not None:
+            _need(tensor.is_cuda, "kernel operands must live on the GPU")
+            _need(tensor.is_contiguous(), "kernel operands must be contiguous")
+
+
+class Ops:
+    """The kernel library.  One instance per process; see `get_ops()`."""
+
+    def __init__(self, path: str):
+        self.path = path
+        self.lib = ctypes.CDLL(path)
+        for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
+                     "ta_paged_attention_generic", "ta_gemm_f32", "ta_gemm_bf16", "ta_argmax"):
+            getattr(self.lib, name).restype = ctypes.c_int
+
+    @staticmethod
+    def _stream() -> ctypes.c_void_p:
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    @staticmethod
+    def _check(status: int, what: str) -> None:
+        if status != 0:
+            raise KernelError(f"{what} failed with status {status}"
+                              + (" (sizes the kernel does not take)" if status < 0 else " (HIP error)"))
+
+    # ------------------------------------------------------------------ embedding
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out[t] = table[ids[t]] as float32.  ids int32 [T]; table [V, H]; out float32 [T, H]."""
+        _dev(ids, table, out)
+        n, (vocab, hidden) = ids.numel(), table.shape
+        _need(ids.dtype == torch.int32 and ids.dim() == 1, "ids must be int32 [T]")
+        _need(out.dtype == torch.float32 and tuple(out.shape) == (n, hidden), "out must be float32 [T, H]")
+        self._check(self.lib.ta_embedding(_ptr(ids), _ptr(table), _ptr(out), n, hidden, vocab,
+                                          _code(table.dtype), self._stream()), "embedding")
+        return out
+
+    # ---------------------------------------------------------------------- norm
+    def add_rmsnorm(self, residual: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor,
+                    eps: float, out: torch.Tensor, rows: torch.Tensor | None = None,
+                    store_residual: bool = True) -> torch.Tensor:
+        """x = residual[r] (+ delta[r]); optionally residual[r] = x; out[i] = rmsnorm(x) * weight.
+
+        residual float32 [T, H]; delta [T, H] in out's dtype or None; weight float32 [H];
+        rows int32 [R] picks the rows (None: all, R = T); out [R, H].
+        """
+        _dev(residual, delta, weight, out, rows)
+        n_tokens, hidden = residual.shape
+        n_rows = n_tokens if rows is None else rows.numel()
+        _need(residual.dtype == torch.float32, "the residual stream is float32")
+        _need(weight.dtype == torch.float32 and weight.numel() == hidden, "norm weight must be float32 [H]")
+        _need(tuple(out.shape) == (n_rows, hidden), "norm output has the wrong shape")
+        if delta is not None:
+            _need(delta.shape == residual.shape and delta.dtype == out.dtype, "delta must match residual and out")
+        if rows is not None:
+            _need(rows.dtype == torch.int32, "rows must be int32")
+            _need(not store_residual, "a row subset never stores the residual")
+        self._check(self.lib.ta_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows),
+                                            n_rows, hidden, ctypes.c_float(eps), int(store_residual),
+                                            _code(out.dtype), self._stream()), "add_rmsnorm")
+        return out
+
+    # ------------------------------------------------------------- gated activation
+    def silu_gate(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out = silu(gate_up[:, :I]) * gate_up[:, I:].  gate_up [T, 2I]; out [T, I]."""
+        _dev(gate_up, out)
+        n_tokens, two_inner = gate_up.shape
+        _need(two_inner % 2 == 0 and tuple(out.shape) == (n_tokens, two_inner // 2) and out.dtype == gate_up.dtype,
+              "silu_gate shapes do not fit")
+        self._check(self.lib.ta_silu_gate(_ptr(gate_up), _ptr(out), n_tokens, two_inner // 2,
+                                          _code(out.dtype), self._stream()), "silu_gate")
+        return out
+
+    # ----------------------------------------------------------------------- rope
+    def rope_store(self, qkv: torch.Tensor, bias: torch.Tensor | None, positions: torch.Tensor,
+                   cos_sin: torch.Tensor | None, slots: torch.Tensor | None,
+                   k_pages: torch.Tensor | None, v_pages: torch.Tensor | None,
+                   n_q: int, n_kv: int, head_dim: int) -> None:
+        """Add bias, rotate q and k heads in place, store k and v heads into their pages.
+
+        qkv [T, (n_q + 2 n_kv) d]; bias float32 or None; positions int32 [T];
+        cos_sin float32 [P, d] (cos half, sin half) or None for no rotation;
+        slots int32 [T] (page * page_size + offset, negative = skip) or None;
+        pages [n_pages, n_kv, page_size, d].
+        """
+        _dev(qkv, bias, positions, cos_sin, slots, k_pages, v_pages)
+        n_tokens, width = qkv.shape
+        _need(width == (n_q + 2 * n_kv) * head_dim, "qkv width does not match the head counts")
+        _need(head_dim % 2 == 0, "head size must be even")
+        _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
+        page_size = 1
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.numel() == width, "bias must be float32 of the qkv width")
+        if cos_sin is not None:
+            _need(cos_sin.dtype == torch.float32 and cos_sin.shape[1] == head_dim, "cos_sin must be float32 [P, d]")
+        if slots is not None:
+            _need(slots.dtype == torch.int32 and slots.numel() == n_tokens, "slots must be int32 [T]")
+            _need(k_pages is not None and v_pages is not None, "slots without pages")
+            _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
+            _need(k_pages.dim() == 4 and k_pages.shape[1] == n_kv and k_pages.shape[3] == head_dim
+                  and v_pages.shape == k_pages.shape, "pages must be [n_pages, n_kv, page_size, d]")
+            page_size = k_pages.shape[2]
+        self._check(self.lib.ta_rope_store(_ptr(qkv), width, _ptr(bias), _ptr(positions), _ptr(cos_sin),
+                                           _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_tokens, n_q, n_kv,
+                                           head_dim, page_size, _code(qkv.dtype), self._stream()), "rope_store")
+
+    # ------------------------------------------------------------------ attention
+    def paged_attention(self, qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor,
+                        v_pages: torch.Tensor, positions: torch.Tensor, entry_of_token: torch.Tensor,
+                        block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
+                        window: int | None, scale: float, max_position: int | None = None) -> torch.Tensor:
+        """Causal attention of every token over the pages of its request.
+
+        qkv [T, >= n_q d] (query heads first); out [T, n_q d]; pages [n_pages, n_kv, page_size, d];
+        positions, entry_of_token int32 [T]; block_table int32 [E, P]; a token at position p sees keys
+        max(0, p - window)..p.  `max_position` (host) lets the wrapper check that the table is wide enough.
+        """
+        _dev(qkv, out, k_pages, v_pages, positions, entry_of_token, block_table)
+        n_tokens = qkv.shape[0]
+        _need(qkv.shape[1] >= n_q * head_dim, "qkv is narrower than the query heads")
+        _need(tuple(out.shape) == (n_tokens, n_q * head_dim) and out.dtype == qkv.dtype, "attention output shape")
+        _need(k_pages.dtype == qkv.dtype and k_pages.dim() == 4 and k_pages.shape[1] == n_kv
+              and k_pages.shape[3] == head_dim and v_pages.shape == k_pages.shape, "pages must be [n_pages, n_kv, page_size, d]")
+        _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
+        _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() == n_tokens, "entry_of_token must be int32 [T]")
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 [E, P]")
+        _need(n_kv > 0 and n_q % n_kv == 0, "query heads must be a multiple of kv heads")
+        _need(0 < head_dim <= 256, "head sizes up to 256 are supported")
+        page_size = k_pages.shape[2]
+        if max_position is not None:
+            _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
+        self._check(self.lib.ta_paged_attention_generic(
+            _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(positions),
+            _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], n_tokens, n_q, n_kv, head_dim,
+            page_size, -1 if window is None else int(window), ctypes.c_float(scale), _code(qkv.dtype),
+            self._stream()), "paged_attention")
+        return out
+
+    # --------------------------------------------------------------------- linear
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """out = x @ weight.T (+ bias).  x [M, K] (rows may be strided); weight [N, K]; bias float32 [N].
+
+        float32 operands run on plain multiply-adds; bfloat16 operands on the matrix cores with
+        float accumulation and a bfloat16 or float32 result.
+        """
+        _need(x.is_cuda and weight.is_cuda, "kernel operands must live on the GPU")
+        _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "linear shapes do not fit")
+        _need(x.stride(1) == 1 and weight.is_contiguous(), "linear operands must have contiguous rows")
+        _need(x.dtype == weight.dtype, "x and weight must share a dtype")
+        m, k = x.shape
+        n = weight.shape[0]
+        lda = x.stride(0) if m > 1 else k
+        if out_dtype is None:
+            out_dtype = x.dtype if out is None else out.dtype
+        if out is None:
+            out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        _need(tuple(out.shape) == (m, n) and out.is_contiguous() and out.dtype == out_dtype, "linear output shape")
+        if bias is not None:
+            _need(bias.is_cuda and bias.dtype == torch.float32 and bias.numel() == n, "bias must be float32 [N]")
+        if x.dtype == torch.float32:
+            _need(out_dtype == torch.float32, "float32 products give float32")
+            status = self.lib.ta_gemm_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
+                                          self._stream())
+        else:
+            _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
+            _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
+            _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+            status = self.lib.ta_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
+                                           _code(out_dtype), self._stream())
+        self._check(status, "linear")
+        return out
+
+    # ------------------------------------------------------------------- sampling
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """First maximum of each row.  logits float32 [B, V] -> int32 [B]."""
+        _dev(logits, out)
+        _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [B, V]")
+        if out is None:
+            out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+        _need(out.dtype == torch.int32 and out.numel() == logits.shape[0], "argmax output must be int32 [B]")
+        self._check(self.lib.ta_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
+                                       self._stream()), "argmax")
+        return out
+
+
+_OPS: Ops | None = None
+_LOCK = threading.Lock()
+
+
+def get_ops() -> Ops:
+    """The loaded kernel library; builds it on first use if no built library is found."""
+    global _OPS
+    if _OPS is not None:
+        return _OPS
+    with _LOCK:
+        if _OPS is None:
+            if not torch.cuda.is_available():
+                raise KernelError("tokenizer_amd runs on an AMD GPU through its HIP kernels; "
+                                  "no GPU is visible and there is no CPU path")
+            path = _build.find_library()
+            if path is None:
+                path = _build.build_library()
+            _OPS = Ops(path)
+    return _OPS
+
+
+def default_scale(head_dim: int) -> float:
+    return 1.0 / math.sqrt(head_dim)

@@ -1,0 +1,114 @@
+"""Compile the HIP sources under `csrc/` for gfx950 into one shared library.
+
+`hipcc` turns each `.hip` file into an object (in parallel), then links them.
+The library lands beside this package when that folder can be written, else in
+a per-user folder under the temporary directory.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import glob
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+
+PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SOURCE_DIR = os.path.join(PACKAGE_DIR, "csrc")
+LIB_NAME = "libtokenizer_amd_kernels.so"
+ARCH = "gfx950"
+# Packed float32 instructions are switched off for all device code.
+HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-Wno-unused-command-line-argument"]
+
+
+def _say(message: str) -> None:
+    print(f"[tokenizer_amd build] {message}", file=sys.stderr, flush=True)
+
+
+def hipcc_path() -> str:
+    for candidate in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if candidate and os.path.exists(candidate):
+            return candidate
+    raise RuntimeError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin); "
+                       "the HIP kernels cannot be built")
+
+
+def library_candidates() -> list[str]:
+    fallback = os.path.join(tempfile.gettempdir(), f"tokenizer_amd_{os.getuid()}")
+    return [os.path.join(PACKAGE_DIR, LIB_NAME), os.path.join(fallback, LIB_NAME)]
+
+
+def find_library() -> str | None:
+    for path in library_candidates():
+        if os.path.exists(path):
+            return path
+    return None
+
+
+def _writable_target() -> str:
+    for path in library_candidates():
+        folder = os.path.dirname(path)
+        try:
+            os.makedirs(folder, exist_ok=True)
+            probe = os.path.join(folder, f".write_probe_{os.getpid()}")
+            with open(probe, "w"):
+                pass
+            os.remove(probe)
+            return path
+        except OSError:
+            continue
+    raise RuntimeError("no writable folder for the kernel library")
+
+
+def _compile_one(hipcc: str, source: str, obj: str) -> tuple[str, float]:
+    started = time.time()
+    proc = subprocess.run([hipcc, *HIPCC_FLAGS, "-I", SOURCE_DIR, "-c", source, "-o", obj],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {os.path.basename(source)}:\n{proc.stderr[-4000:]}")
+    return os.path.basename(source), time.time() - started
+
+
+def build_library(verbose: bool = True) -> str:
+    """Compile every source and link the library; returns its path."""
+    hipcc = hipcc_path()
+    sources = sorted(glob.glob(os.path.join(SOURCE_DIR, "*.hip")))
+    if not sources:
+        raise RuntimeError(f"no HIP sources under {SOURCE_DIR}")
+    target = _writable_target()
+    env_home = os.environ.get("HOME")
+    if not env_home or not os.access(env_home, os.W_OK):
+        os.environ["HOME"] = tempfile.gettempdir()  # the compiler wants a place for its caches
+    started = time.time()
+    with tempfile.TemporaryDirectory(prefix="tokenizer_amd_obj_") as obj_dir:
+        if verbose:
+            _say(f"compiling {len(sources)} HIP sources for {ARCH} with {hipcc}")
+        objects = []
+        workers = max(1, min(len(sources), (os.cpu_count() or 2), 16))
+        with concurrent.futures.ThreadPoolExecutor(workers) as pool:
+            futures = []
+            for source in sources:
+                obj = os.path.join(obj_dir, os.path.basename(source) + ".o")
+                objects.append(obj)
+                futures.append(pool.submit(_compile_one, hipcc, source, obj))
+            for future in concurrent.futures.as_completed(futures):
+                name, seconds = future.result()
+                if verbose:
+                    _say(f"  {name} done in {seconds:.1f} s ({time.time() - started:.0f} s elapsed)")
+        partial = target + f".{os.getpid()}.tmp"
+        proc = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objects, "-o", partial],
+                              capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"linking the kernel library failed:\n{proc.stderr[-4000:]}")
+        os.replace(partial, target)
+    if verbose:
+        _say(f"built {target} in {time.time() - started:.1f} s")
+    return target
+
+
+if __name__ == "__main__":
+    build_library()

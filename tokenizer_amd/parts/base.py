@@ -1,0 +1,103 @@
+"""Interfaces of the parts a layer is put together from, and their registries.
+
+A part is built from its spec, the tensors it asked for and a `Runtime`
+(compute dtype, device, kernel library).  No part knows which model it is in.
+
+Interfaces
+----------
+Norm            tensor_specs(spec) -> {local name: TensorSpec}
+                apply(residual, delta, rows=None) -> normalised rows in the compute dtype.
+                `residual` is the float32 stream [T, H]; `delta` (or None) is added to it first and,
+                unless `rows` picks a subset, the sum is stored back.
+PositionEncoding
+                encode_and_store(qkv, geometry, ctx, cache, bias): adds the projection bias, encodes
+                the query and key heads in place and writes keys and values of this step into `cache`.
+Mixer           tensor_specs(spec), cache_need(spec) -> CacheNeed
+                forward(x [T, H], ctx: StepContext, cache: LayerCache) -> [T, H] in the compute dtype.
+FeedForward     tensor_specs(spec); forward(x [T, H], ctx) -> [T, H].
+Block           arranges two norms, a mixer and a feed-forward around the residual stream:
+                forward(residual, delta, ctx, cache) -> delta still to be added.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Callable
+
+import torch
+
+from .spec import CacheNeed, TensorSpec
+
+
+@dataclasses.dataclass
+class Runtime:
+    dtype: torch.dtype
+    device: torch.device
+    ops: Any                      # tokenizer_amd.kernels.Ops (or a stand-in with the same methods)
+
+
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: dict[str, type] = {}
+
+    def register(self, kind: str, cls: type | None = None, replace: bool = False):
+        def put(target: type) -> type:
+            if kind in self._items and not replace:
+                raise ValueError(f"{self.what} {kind!r} is already registered")
+            self._items[kind] = target
+            return target
+        return put if cls is None else put(cls)
+
+    def get(self, kind: str) -> type:
+        try:
+            return self._items[kind]
+        except KeyError:
+            raise KeyError(f"unknown {self.what} {kind!r}; registered: {', '.join(sorted(self._items))}") from None
+
+    def kinds(self) -> list[str]:
+        return sorted(self._items)
+
+
+NORMS = Registry("norm")
+POSITIONS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block")
+
+
+class Part:
+    """Common base: a part names its tensors and is built from them."""
+
+    @staticmethod
+    def tensor_specs(spec) -> dict[str, TensorSpec]:
+        return {}
+
+
+class Norm(Part):
+    def apply(self, residual: torch.Tensor, delta: torch.Tensor | None,
+              rows: torch.Tensor | None = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def encode_and_store(self, qkv, bias, n_q: int, n_kv: int, head_dim: int, ctx, cache) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    @staticmethod
+    def cache_need(spec) -> CacheNeed:
+        return CacheNeed()
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    def forward(self, residual: torch.Tensor, delta: torch.Tensor | None, ctx, cache) -> torch.Tensor:
+        raise NotImplementedError

@@ -1,0 +1,23 @@
+"""Arrangements of norms, mixer and feed-forward around the residual stream."""
+from __future__ import annotations
+
+from .base import BLOCKS, Block
+
+
+@BLOCKS.register("pre_norm")
+class PreNormBlock(Block):
+    """x + mixer(norm1(x)), then + feed_forward(norm2(.)) (qwen-infer/src/model.rs:615-622).
+
+    The residual stream is float32.  Each sub-layer's output is handed on as a pending `delta`
+    so that the add fuses into the next norm.
+    """
+
+    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+
+    def forward(self, residual, delta, ctx, cache):
+        normed = self.mixer_norm.apply(residual, delta)
+        mixed = self.mixer.forward(normed, ctx, cache)
+        normed = self.feed_forward_norm.apply(residual, mixed)
+        return self.feed_forward.forward(normed, ctx)

@@ -1,0 +1,84 @@
+"""A decoder put together from a `ModelSpec`: embedding, layers in schedule order, final norm, head."""
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Runtime
+from .spec import CacheNeed, ModelSpec, TensorSpec
+
+
+def _prefixed(prefix: str, specs: dict[str, TensorSpec]) -> dict[str, TensorSpec]:
+    return {f"{prefix}.{name}" if prefix else name: spec for name, spec in specs.items()}
+
+
+def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
+    """Every tensor name the model reads from the weight file, with its shape."""
+    out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size), std=spec.embedding_std)}
+    for layer in spec.layers:
+        out.update(_prefixed(layer.mixer_norm_prefix, NORMS.get(layer.mixer_norm.kind).tensor_specs(layer.mixer_norm)))
+        out.update(_prefixed(layer.mixer_prefix, MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer)))
+        out.update(_prefixed(layer.feed_forward_norm_prefix,
+                             NORMS.get(layer.feed_forward_norm.kind).tensor_specs(layer.feed_forward_norm)))
+        out.update(_prefixed(layer.feed_forward_prefix,
+                             FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward)))
+    out.update(_prefixed(spec.final_norm_prefix, NORMS.get(spec.final_norm.kind).tensor_specs(spec.final_norm)))
+    if not spec.tied_head:
+        out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
+    return out
+
+
+def cache_needs(spec: ModelSpec) -> list[CacheNeed]:
+    """What each layer's mixer asks of the cache manager, by layer index."""
+    return [MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) for layer in spec.layers]
+
+
+def _strip(prefix: str, tensors: dict[str, torch.Tensor]) -> dict[str, torch.Tensor]:
+    lead = prefix + "."
+    return {name[len(lead):]: value for name, value in tensors.items() if name.startswith(lead)}
+
+
+@dataclasses.dataclass
+class LayerCache:
+    """What one scheduled layer may touch of the cache in a step."""
+    group: int | None = None                # index into ctx.block_tables / ctx.slots
+    k_pages: torch.Tensor | None = None     # [n_pages, n_kv, page_size, d]
+    v_pages: torch.Tensor | None = None
+    state: torch.Tensor | None = None       # [n_slots, *state_shape]
+    writes: bool = True                     # False when the layer reads another layer's cache
+
+
+class DecoderModel:
+    """Weights and parts of one model.  It owns no cache: `forward` is handed the step's context
+    (token ids, positions, block tables) and one `LayerCache` per schedule entry."""
+
+    def __init__(self, spec: ModelSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
+        self.spec, self.runtime = spec, runtime
+        self.embedding = tensors[spec.embedding_name]
+        self.blocks = []
+        for layer in spec.layers:
+            mixer_norm = NORMS.get(layer.mixer_norm.kind)(layer.mixer_norm, _strip(layer.mixer_norm_prefix, tensors), runtime)
+            mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _strip(layer.mixer_prefix, tensors), runtime)
+            ff_norm = NORMS.get(layer.feed_forward_norm.kind)(layer.feed_forward_norm,
+                                                              _strip(layer.feed_forward_norm_prefix, tensors), runtime)
+            feed_forward = FEED_FORWARDS.get(layer.feed_forward.kind)(layer.feed_forward,
+                                                                     _strip(layer.feed_forward_prefix, tensors), runtime)
+            self.blocks.append(BLOCKS.get(layer.block)(mixer_norm, mixer, ff_norm, feed_forward))
+        self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)
+        self.head = self.embedding if spec.tied_head else tensors[spec.head_name]
+
+    def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
+        """Run the tokens of `ctx` through the schedule; float32 logits [len(want_rows), vocab]."""
+        ops = self.runtime.ops
+        residual = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.runtime.device)
+        ops.embedding(ctx.token_ids, self.embedding, residual)
+        delta = None
+        for entry, cache in zip(self.spec.schedule, layer_caches):
+            delta = self.blocks[entry.layer].forward(residual, delta, ctx, cache)
+        if ctx.want_rows.numel() == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.runtime.device)
+        # Only the wanted rows are normalised and multiplied with the head (the reference keeps
+        # the last row, qwen-infer/src/model.rs:1224-1242).
+        wanted = self.final_norm.apply(residual, delta, rows=ctx.want_rows)
+        return ops.linear(wanted, self.head, out_dtype=torch.float32)

@@ -1,0 +1,96 @@
+"""Weights by tensor name, checked against what the model's parts expect.
+
+The file is matched to the expectation in one pass and every problem is
+reported together: missing tensors, unexpected tensors and wrong shapes.
+Tensors are not renamed; a part that wants two matrices side by side joins
+them itself after loading (the reference keeps q, k, v and gate, up apart,
+qwen-infer/src/model.rs:263-276).
+"""
+from __future__ import annotations
+
+import os
+
+import torch
+
+from ..parts.spec import TensorSpec
+from .safetensors_io import SafetensorsError, SafetensorsFile
+
+
+class WeightError(ValueError):
+    """The weight file does not hold what the model needs."""
+
+    def __init__(self, path, missing=(), unexpected=(), wrong_shape=(), wrong_dtype=(), other=()):
+        self.path = path
+        self.missing = list(missing)
+        self.unexpected = list(unexpected)
+        self.wrong_shape = list(wrong_shape)   # (name, found, wanted)
+        self.wrong_dtype = list(wrong_dtype)   # (name, found)
+        self.other = list(other)
+        lines = [f"weights in {path} do not fit the model:"]
+        if self.missing:
+            lines.append(f"  missing ({len(self.missing)}): " + ", ".join(self.missing))
+        if self.unexpected:
+            lines.append(f"  unexpected ({len(self.unexpected)}): " + ", ".join(self.unexpected))
+        if self.wrong_shape:
+            lines.append(f"  wrong shape ({len(self.wrong_shape)}): " + ", ".join(
+                f"{n} is {list(f)}, wanted {list(w)}" for n, f, w in self.wrong_shape))
+        if self.wrong_dtype:
+            lines.append(f"  unusable dtype ({len(self.wrong_dtype)}): " + ", ".join(
+                f"{n} is {d}" for n, d in self.wrong_dtype))
+        lines.extend(f"  {msg}" for msg in self.other)
+        super().__init__("\n".join(lines))
+
+
+_FLOATS = (torch.bfloat16, torch.float16, torch.float32, torch.float64)
+_INTS = (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8)
+
+
+def stored_form(tensor: torch.Tensor, spec: TensorSpec, compute_dtype: torch.dtype) -> torch.Tensor:
+    """How a loaded tensor is kept: see `TensorSpec.role`.
+
+    Matrices feed the matrix products and are held in the compute dtype
+    (bfloat16 files stay bfloat16 in bfloat16 mode and are widened, exactly, in
+    float32 mode).  Vectors are widened to float32.  Integer tables become
+    int32.  "keep" leaves a tensor as stored, so one stored in 32-bit stays so.
+    """
+    if spec.role == "matrix":
+        return tensor.to(compute_dtype)
+    if spec.role == "vector":
+        return tensor.to(torch.float32)
+    if spec.role == "table":
+        return tensor.to(torch.int32)
+    return tensor
+
+
+def weight_path(folder: str) -> str:
+    return os.path.join(folder, "model.safetensors") if os.path.isdir(folder) else folder
+
+
+def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: torch.dtype,
+                 device: torch.device | str = "cpu") -> dict[str, torch.Tensor]:
+    """Load exactly the tensors in `expected`, or raise one `WeightError` naming every misfit."""
+    path = weight_path(folder)
+    try:
+        source = SafetensorsFile(path)
+    except SafetensorsError as err:
+        raise WeightError(path, other=[str(err)]) from None
+    names = set(source.names())
+    missing = sorted(set(expected) - names)
+    unexpected = sorted(names - set(expected))
+    wrong_shape, wrong_dtype = [], []
+    for name in sorted(names & set(expected)):
+        shape, dtype = source.info(name)
+        spec = expected[name]
+        if tuple(shape) != tuple(spec.shape):
+            wrong_shape.append((name, shape, spec.shape))
+        if spec.role in ("matrix", "vector") and dtype not in _FLOATS:
+            wrong_dtype.append((name, dtype))
+        if spec.role == "table" and dtype not in _INTS:
+            wrong_dtype.append((name, dtype))
+    if missing or unexpected or wrong_shape or wrong_dtype:
+        raise WeightError(path, missing, unexpected, wrong_shape, wrong_dtype)
+    out = {}
+    for name, spec in expected.items():
+        out[name] = stored_form(source.tensor(name), spec, compute_dtype).to(device).contiguous()
+    source.close()
+    return out

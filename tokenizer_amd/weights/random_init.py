@@ -1,0 +1,56 @@
+"""Random-weights mode: a model folder from a configuration and a seed.
+
+Every tensor is drawn from its own generator keyed by (seed, tensor name), so
+the values of a tensor do not depend on which other tensors exist.  Matrices,
+biases and the embedding are N(0, std) rounded to bfloat16 (the dtype model
+files are stored in); norm scales are 1.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+
+import torch
+
+from ..config.base import ModelConfig
+from ..parts.spec import TensorSpec
+from .safetensors_io import save_safetensors
+
+
+def _generator(seed: int, name: str) -> torch.Generator:
+    digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int.from_bytes(digest[:8], "little") & ((1 << 63) - 1))
+    return gen
+
+
+def random_tensor(name: str, spec: TensorSpec, seed: int) -> torch.Tensor:
+    if spec.role == "table":
+        return torch.zeros(spec.shape, dtype=torch.int32)
+    if spec.init == "ones":
+        return torch.ones(spec.shape, dtype=torch.bfloat16)
+    if spec.init == "zeros":
+        return torch.zeros(spec.shape, dtype=torch.bfloat16)
+    if spec.init != "normal":
+        raise ValueError(f"unknown init {spec.init!r} for {name}")
+    values = torch.empty(spec.shape, dtype=torch.float32)
+    values.normal_(0.0, spec.std, generator=_generator(seed, name))
+    return values.to(torch.bfloat16)
+
+
+def random_tensors(expected: dict[str, TensorSpec], seed: int) -> dict[str, torch.Tensor]:
+    return {name: random_tensor(name, spec, seed) for name, spec in expected.items()}
+
+
+def write_random_model(config: ModelConfig, seed: int, folder: str) -> str:
+    """Write config.json and model.safetensors for `config` with weights from `seed`."""
+    from ..config.registry import get_architecture
+    from ..parts.model import expected_tensors
+
+    spec = get_architecture(config.architecture).build_spec(config)
+    os.makedirs(folder, exist_ok=True)
+    config.save(folder)
+    save_safetensors(os.path.join(folder, "model.safetensors"),
+                     random_tensors(expected_tensors(spec), seed),
+                     metadata={"format": "pt", "seed": str(seed)})
+    return folder
