@@ -51,3 +51,100 @@ def test_whole_prompts(model_folders, oracle, name, dtype):
         close(got, oracle(name, ids), dtype)
         eng.end_request(seed)
     eng.cache.check_invariants()
+
+
+import trace_tools as tt
+
+LENGTHS = [1, 9, 40, 64, 100, 33, 77]
+
+
+def requests_for(name):
+    raw = TINY[name][0]
+    lens = [min(n, raw["max_position_embeddings"]) for n in LENGTHS]
+    return {f"r{i}": random_ids(raw["vocab_size"], n, 10 + i) for i, n in enumerate(lens)}
+
+
+def check_trace(model_folders, oracle, name, dtype, steps):
+    reqs = requests_for(name)
+    eng = engine_for(model_folders[name], dtype, max_tokens=tt.peak_tokens(steps), max_requests=4)
+    eng.pools.poison()          # a read of a slot no request wrote shows up as NaN
+    got = tt.run_in_process(eng, steps)
+    for rid, ids in reqs.items():
+        close(got[rid], oracle(name, ids), dtype)
+    eng.cache.check_invariants()
+    assert not eng.cache.requests
+    for group in eng.cache.groups:
+        assert group.allocator.all_refcounts_zero()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_last_32_tokens_one_by_one(model_folders, oracle, name, dtype):
+    check_trace(model_folders, oracle, name, dtype, tt.decode_tail(requests_for(name), 32))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_portions_of_changing_size(model_folders, oracle, name, dtype):
+    check_trace(model_folders, oracle, name, dtype, tt.portions(requests_for(name), 3))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+@pytest.mark.parametrize("seed", [4, 5])
+def test_mixed_batches_with_reused_pages(model_folders, oracle, name, dtype, seed):
+    steps = tt.mixed(requests_for(name), seed)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    check_trace(model_folders, oracle, name, dtype, steps)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_long_decoding(model_folders, oracle, name, dtype):
+    # Three tokens of prompt, then every further token alone up to the position limit of 256.
+    raw = TINY[name][0]
+    ids = random_ids(raw["vocab_size"], 256, 99)
+    steps = tt.decode_tail({"long": ids}, tail=253)
+    eng = engine_for(model_folders[name], dtype, max_tokens=256, max_requests=2)
+    eng.pools.poison()
+    got = tt.run_in_process(eng, steps)
+    close(got["long"], oracle(name, ids), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_first_tokens_of_a_sequence(model_folders, oracle, name, dtype):
+    # Position 0 alone, then position 1 alone, then two at once: the shortest contexts there are.
+    raw = TINY[name][0]
+    ids = random_ids(raw["vocab_size"], 4, 7)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": ids[:1], "want": [0]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": ids[1:2], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": ids[2:4], "want": [0, 1]}], "end": ["x"]}]
+    eng = engine_for(model_folders[name], dtype, max_tokens=64, max_requests=2)
+    eng.pools.poison()
+    got = tt.run_in_process(eng, steps)
+    close(got["x"], oracle(name, ids), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, oracle, tmp_path, dtype):
+    # The program itself, as a child process: mixed steps, wants on some places only, a step without wants.
+    name = "B"
+    reqs = requests_for(name)
+    steps = tt.mixed(reqs, 6)
+    for step in steps[::3]:
+        for entry in step["entries"]:
+            entry["want"] = entry["want"][-1:]
+    steps[1]["entries"][0]["want"] = []
+    vocab = TINY[name][0]["vocab_size"]
+    got = tt.run_program(model_folders[name], dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps), vocab)
+    # Rebuild which positions were asked for.
+    at = {rid: 0 for rid in reqs}
+    asked = {rid: [] for rid in reqs}
+    for step in steps:
+        for entry in step["entries"]:
+            asked[entry["id"]] += [at[entry["id"]] + w for w in entry["want"]]
+            at[entry["id"]] += len(entry["tokens"])
+    for rid, ids in reqs.items():
+        want = oracle(name, ids)[asked[rid]]
+        close(got[rid], want, dtype)
