@@ -1,0 +1,192 @@
+"""Decode and prefill throughput of the engine at Qwen2.5-0.5B sizes with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--dtype bfloat16]
+
+A step is one decode step of the whole batch.  The default run prefills 8 prompts of 2,048
+random ids and decodes from there; it also times a prefill of 2,048 tokens and decoding at
+batch 1 and 64, and prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Published peaks of MI355X.
+HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
+
+QWEN2_0_5B = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896,
+              "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864,
+              "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+              "max_position_embeddings": 32768, "sliding_window": 32768, "use_sliding_window": False,
+              "max_window_layers": 21, "hidden_act": "silu"}
+FULL_LAYERS = 24
+PROMPT_LEN = 2048
+CONTEXT_LEN = 4096
+
+
+def log(message: str) -> None:
+    print(f"[bench] {message}", file=sys.stderr, flush=True)
+
+
+def weight_bytes_per_step(model) -> int:
+    """Bytes of every weight a decode step reads once (the embedding table is read whole by the tied head)."""
+    import torch
+    seen, total = set(), 0
+    decoder = model.decoder
+    tensors = [decoder.head]
+    for block in decoder.blocks:
+        for part in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward):
+            tensors.extend(v for v in vars(part).values() if isinstance(v, torch.Tensor))
+    tensors.extend(v for v in vars(decoder.final_norm).values() if isinstance(v, torch.Tensor))
+    for tensor in tensors:
+        if tensor.data_ptr() not in seen:
+            seen.add(tensor.data_ptr())
+            total += tensor.numel() * tensor.element_size()
+    return total
+
+
+def kv_bytes_per_token(cfg, itemsize: int) -> int:
+    d = cfg.hidden_size // cfg.num_attention_heads
+    return cfg.num_hidden_layers * 2 * cfg.num_key_value_heads * d * itemsize
+
+
+def prefill_flops(cfg, tokens: int, logit_rows: int = 1) -> float:
+    d = cfg.hidden_size // cfg.num_attention_heads
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    linear = h * (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * d + cfg.num_attention_heads * d * h + 3 * h * i
+    flops = 2.0 * tokens * cfg.num_hidden_layers * linear
+    flops += cfg.num_hidden_layers * 4.0 * cfg.num_attention_heads * d * tokens * (tokens + 1) / 2
+    flops += 2.0 * h * cfg.vocab_size * logit_rows
+    return flops
+
+
+def make_prompts(batch: int, vocab: int, seed: int):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    return [[int(t) for t in rng.integers(0, vocab, size=PROMPT_LEN)] for _ in range(batch)]
+
+
+def run_decode(model, batch: int, steps: int, warmup: int):
+    """Prefill `batch` prompts, then time `steps` decode steps (greedy, ids picked on the device)."""
+    import torch
+    from tokenizer_amd.engine import Engine, StepEntry
+
+    page_size = 16
+    engine = Engine(model, num_pages=batch * (CONTEXT_LEN // page_size) + 8, page_size=page_size, max_requests=batch)
+    prompts = make_prompts(batch, model.vocab_size, seed=1)
+    last = []
+    for rid, prompt in enumerate(prompts):
+        engine.add_request(rid)
+        logits = engine.step([StepEntry(rid, prompt, [len(prompt) - 1])])
+        last.append(engine.argmax(logits)[0])
+
+    def decode_step(tokens):
+        logits = engine.step([StepEntry(rid, [tokens[rid]], [0]) for rid in range(batch)])
+        return engine.argmax(logits)
+
+    for _ in range(warmup):
+        last = decode_step(last)
+    torch.cuda.synchronize()
+    kv_start = engine.cache.seq_len(0)
+    started = time.perf_counter()
+    for _ in range(steps):
+        last = decode_step(last)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    kv_mean = kv_start + (steps - 1) / 2 + 1          # keys each step reads, averaged over the timed steps
+    for rid in range(batch):
+        engine.end_request(rid)
+    del engine
+    torch.cuda.empty_cache()
+    return elapsed, kv_mean
+
+
+def run_prefill(model, repeats: int = 3):
+    import torch
+    from tokenizer_amd.engine import Engine, StepEntry
+    engine = Engine(model, num_pages=PROMPT_LEN // 16 + 8, page_size=16, max_requests=1)
+    prompt = make_prompts(1, model.vocab_size, seed=2)[0]
+    best = None
+    for _ in range(repeats + 1):
+        engine.add_request("p")
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        logits = engine.step([StepEntry("p", prompt, [PROMPT_LEN - 1])])
+        engine.argmax(logits)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        engine.end_request("p")
+        best = elapsed if best is None else min(best, elapsed)
+    return best
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=128)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--layers", type=int, default=FULL_LAYERS)
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; runs with --gpus > 1 are not supported")
+        return 2
+
+    import torch
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import random_model
+
+    cfg = Qwen2Config.from_dict(dict(QWEN2_0_5B, num_hidden_layers=args.layers))
+    log(f"building random weights ({args.layers} layers, {args.dtype})")
+    model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    weights = weight_bytes_per_step(model)
+    kv_token = kv_bytes_per_token(cfg, itemsize)
+
+    log(f"decode at batch {args.batch}: {args.warmup} warmup + {args.steps} timed steps")
+    elapsed, kv_mean = run_decode(model, args.batch, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = args.batch * args.steps / elapsed
+    step_bytes = weights + args.batch * kv_mean * kv_token
+    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    record = {
+        "metric": "decode tokens/s (Qwen2.5-0.5B sizes, batch %d, context %d)" % (args.batch, CONTEXT_LEN),
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform random ids)",
+        "config": {"model": "qwen2.5-0.5b-sizes", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+                   "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch, "prompt_len": PROMPT_LEN,
+                   "seq_len": CONTEXT_LEN, "page_size": 16, "parallelism": "single-gpu"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBS, 4)},
+    }
+    if not args.no_points:
+        log("prefill of 2,048 tokens")
+        seconds = run_prefill(model)
+        flops = prefill_flops(cfg, PROMPT_LEN)
+        record["prefill"] = {"value": round(PROMPT_LEN / seconds, 1), "tokens": PROMPT_LEN, "ms": round(seconds * 1e3, 3),
+                             "frac": round(flops / seconds / (PEAK_TFLOPS[args.dtype] * 1e12), 5)}
+        points = {}
+        for batch, steps in ((1, args.steps), (64, max(16, args.steps // 4))):
+            log(f"decode at batch {batch}: {steps} timed steps")
+            e, _ = run_decode(model, batch, steps, min(args.warmup, 4))
+            points[f"decode_b{batch}"] = round(batch * steps / e, 1)
+        record["points"] = points
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,118 @@
+"""Configuration and registry."""
+import json
+
+import pytest
+
+from tiny_configs import TINY
+from tokenizer_amd.config import (ConfigError, Qwen2Config, load_config, register_architecture,
+                                  registered_architectures)
+from tokenizer_amd.config.base import ModelConfig
+from tokenizer_amd.models.qwen2 import qwen2_spec
+from tokenizer_amd.parts import cache_needs, expected_tensors
+
+
+def write(tmp_path, raw):
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    return str(tmp_path)
+
+
+def test_reads_the_architectures_own_keys(tmp_path):
+    raw = dict(TINY["B"][0], unknown_key=[1, 2, 3], torch_dtype="bfloat16")
+    cfg = load_config(write(tmp_path, raw))
+    assert isinstance(cfg, Qwen2Config)
+    assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads) == (3, 96, 3, 1)
+    assert cfg.derived_head_dim == 32 and cfg.rms_norm_eps == 1e-5 and cfg.rope_theta == 1e6
+    assert cfg.tie_word_embeddings is False
+
+
+def test_real_checkpoint_keys_parse(tmp_path):
+    # The config.json of Qwen2.5-0.5B as the reference's comments describe it (qwen-infer/src/model.rs:5-7,
+    # 1441-1444: flag off, max_window_layers 21).
+    raw = {"architectures": ["Qwen2ForCausalLM"], "hidden_act": "silu", "hidden_size": 896,
+           "intermediate_size": 4864, "max_position_embeddings": 32768, "max_window_layers": 21,
+           "num_attention_heads": 14, "num_hidden_layers": 24, "num_key_value_heads": 2, "rms_norm_eps": 1e-06,
+           "rope_theta": 1000000.0, "sliding_window": 32768, "tie_word_embeddings": True,
+           "use_sliding_window": False, "vocab_size": 151936, "bos_token_id": 151643}
+    cfg = load_config(write(tmp_path, raw))
+    assert cfg.derived_head_dim == 64
+    assert all(cfg.window_for_layer(i) is None for i in range(24))
+    spec = qwen2_spec(cfg)
+    names = expected_tensors(spec)
+    assert "lm_head.weight" not in names
+    assert names["model.layers.23.self_attn.k_proj.weight"].shape == (128, 896)
+    assert names["model.layers.0.mlp.down_proj.weight"].shape == (896, 4864)
+    assert sum(1 for n in names if n.endswith(".bias")) == 3 * 24
+
+
+def test_missing_keys_are_all_named(tmp_path):
+    raw = dict(TINY["A"][0])
+    del raw["rope_theta"], raw["rms_norm_eps"]
+    with pytest.raises(ConfigError) as err:
+        load_config(write(tmp_path, raw))
+    assert "rope_theta" in str(err.value) and "rms_norm_eps" in str(err.value)
+
+
+@pytest.mark.parametrize("change, word", [
+    ({"hidden_act": "gelu"}, "silu"),
+    ({"num_attention_heads": 5}, "heads"),
+    ({"num_key_value_heads": 3}, "kv heads"),
+    ({"num_hidden_layers": 0}, "num_hidden_layers"),
+    ({"vocab_size": "many"}, "vocab_size"),
+    ({"head_dim": 8}, "head_dim"),
+    ({"tie_word_embeddings": 1}, "tie_word_embeddings"),
+    ({"use_sliding_window": True, "sliding_window": None}, "sliding_window"),
+])
+def test_bad_values_are_refused(tmp_path, change, word):
+    with pytest.raises(ConfigError) as err:
+        load_config(write(tmp_path, dict(TINY["A"][0], **change)))
+    assert word in str(err.value)
+
+
+def test_unknown_architecture_lists_the_known_ones(tmp_path):
+    with pytest.raises(ConfigError) as err:
+        load_config(write(tmp_path, dict(TINY["A"][0], architectures=["LlamaForCausalLM"])))
+    assert "LlamaForCausalLM" in str(err.value) and "Qwen2ForCausalLM" in str(err.value)
+    raw = dict(TINY["A"][0])
+    del raw["architectures"]
+    with pytest.raises(ConfigError):
+        load_config(write(tmp_path, raw))
+
+
+def test_window_applies_from_max_window_layers_on(tmp_path):
+    # qwen-infer/src/model.rs:909-915 and the test at 1434-1445.
+    cfg = Qwen2Config.from_dict(TINY["C"][0])
+    assert [cfg.window_for_layer(i) for i in range(4)] == [None, 21, 21, 21]
+    off = Qwen2Config.from_dict(dict(TINY["C"][0], use_sliding_window=False))
+    assert [off.window_for_layer(i) for i in range(4)] == [None] * 4
+    needs = cache_needs(qwen2_spec(cfg))
+    assert [n.kind for n in needs] == ["full", "window", "window", "window"]
+    assert needs[1].window == 21 and needs[1].n_kv_heads == 5 and needs[1].head_dim == 16
+
+
+def test_every_size_in_the_spec_comes_from_the_config():
+    a, b = (qwen2_spec(Qwen2Config.from_dict(TINY[k][0])) for k in "AB")
+    assert (a.vocab_size, b.vocab_size) == (256, 384)
+    assert (len(a.layers), len(b.layers)) == (2, 3)
+    assert (a.layers[0].mixer.head_dim, b.layers[0].mixer.head_dim) == (16, 32)
+    assert (a.layers[0].mixer_norm.eps, b.layers[0].mixer_norm.eps) == (1e-6, 1e-5)
+    assert (a.layers[0].mixer.position.theta, b.layers[0].mixer.position.theta) == (1e4, 1e6)
+    assert (a.tied_head, b.tied_head) == (True, False)
+    assert "lm_head.weight" in expected_tensors(b) and "lm_head.weight" not in expected_tensors(a)
+    assert [e.layer for e in b.schedule] == [0, 1, 2]
+
+
+def test_a_new_architecture_registers_without_touching_the_package(tmp_path):
+    import dataclasses
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        width: int
+        depth: int = 1
+
+    name = "ToyForTestingTheRegistry"
+    if name not in registered_architectures():
+        register_architecture(name, ToyConfig, lambda cfg: ("spec", cfg.width))
+    cfg = load_config(write(tmp_path, {"architectures": [name], "width": 12}))
+    assert cfg.width == 12 and cfg.depth == 1 and cfg.architecture == name
+    with pytest.raises(ValueError):
+        register_architecture(name, ToyConfig, lambda cfg: None)

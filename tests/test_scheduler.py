@@ -1,0 +1,185 @@
+"""The scheduler's decisions, on a real engine driven by plain torch ops on the CPU
+(cases of qwen-server/src/engine.rs:1328-2529 that do not need a server)."""
+import pytest
+
+from cpu_engine import cpu_engine
+from tiny_configs import random_ids
+from tokenizer_amd.engine import (Failure, GenerateParams, Generated, QueueFull, Scheduler, SchedulerConfig,
+                                  StopReason, generate)
+
+
+def solo(folder, prompt, params):
+    return generate(cpu_engine(folder), prompt, params)
+
+
+def prompts(n, lengths, vocab=256):
+    return [random_ids(vocab, lengths[i % len(lengths)], 40 + i) for i in range(n)]
+
+
+def test_batched_equals_solo(model_folders):
+    folder = model_folders["A"]
+    engine = cpu_engine(folder, num_pages=64, max_requests=8)
+    sched = Scheduler(engine, SchedulerConfig(max_batch_size=8, num_blocks=64))
+    budgets = [5, 1, 4, 5, 2, 5, 3, 5]
+    ps = prompts(8, [1, 2, 3, 4, 5, 6, 17, 31])
+    ids = [sched.add_request(p, GenerateParams.greedy(n)) for p, n in zip(ps, budgets)]
+    results = sched.run()
+    for rid, prompt, n in zip(ids, ps, budgets):
+        want = solo(folder, prompt, GenerateParams.greedy(n))
+        assert isinstance(results[rid], Generated)
+        assert results[rid].tokens == want.tokens and results[rid].reason == StopReason.MaxTokens
+        assert results[rid].completion_tokens == n
+    assert sched.stats.requests_finished == 8 and sched.stats.max_running == 8
+    # The first iteration holds all eight prompts; later ones only single tokens of those still decoding.
+    assert sorted(engine.forwards[0]) == sorted(len(p) for p in ps)
+    assert all(set(step) == {1} for step in engine.forwards[1:])
+    assert [len(step) for step in engine.forwards[1:]] == [7, 6, 5, 4]
+    sched.assert_idle()
+
+
+def test_warm_requests_in_a_batch_draw_as_they_would_alone(model_folders):
+    folder = model_folders["A"]
+    sched = Scheduler(cpu_engine(folder), SchedulerConfig())
+    ps = prompts(3, [4, 9, 2])
+    params = [GenerateParams(max_tokens=12, temperature=1.3, top_p=0.95, seed=s) for s in (5, 6, 5)]
+    ids = [sched.add_request(p, q) for p, q in zip(ps, params)]
+    results = sched.run()
+    for rid, prompt, q in zip(ids, ps, params):
+        assert results[rid].tokens == solo(folder, prompt, q).tokens
+    sched.assert_idle()
+
+
+def test_token_budget_cuts_prompts_and_decoding_goes_first(model_folders):
+    folder = model_folders["A"]
+    engine = cpu_engine(folder, num_pages=64)
+    sched = Scheduler(engine, SchedulerConfig(max_num_batched_tokens=16, prefill_chunk=10))
+    long_a, long_b, short = random_ids(256, 37, 1), random_ids(256, 23, 2), random_ids(256, 3, 3)
+    first = sched.add_request(short, GenerateParams.greedy(6))
+    sched.step()                                         # the short one is through its prompt
+    a = sched.add_request(long_a, GenerateParams.greedy(3))
+    b = sched.add_request(long_b, GenerateParams.greedy(3))
+    results = sched.run()
+    assert all(sum(step) <= 16 for step in engine.forwards)
+    assert engine.forwards[0] == [3]
+    assert engine.forwards[1] == [1, 10, 5]              # the decoding token first, then portions in order of arrival
+    assert engine.forwards[2] == [1, 10, 5]
+    assert max(max(step) for step in engine.forwards) == 10
+    for rid, prompt, n in ((first, short, 6), (a, long_a, 3), (b, long_b, 3)):
+        assert results[rid].tokens == solo(folder, prompt, GenerateParams.greedy(n)).tokens
+    sched.assert_idle()
+
+
+def test_pages_run_out_the_newest_is_preempted_and_recomputed(model_folders):
+    # Pool of 3 pages, two 16-token prompts, 4 tokens each: both need a second page once they decode.
+    folder = model_folders["A"]
+    engine = cpu_engine(folder, num_pages=3, max_requests=4)
+    sched = Scheduler(engine, SchedulerConfig(num_blocks=3, prefix_cache=False))
+    ps = prompts(2, [16])
+    ids = [sched.add_request(p, GenerateParams.greedy(4)) for p in ps]
+    results = sched.run()
+    assert sched.stats.preemptions >= 1 and sched.stats.last_preempted_id == ids[1]
+    for rid, prompt in zip(ids, ps):
+        assert results[rid].tokens == solo(folder, prompt, GenerateParams.greedy(4)).tokens
+        assert results[rid].completion_tokens == 4
+    # The recomputation ran the prompt and the tokens sampled so far in one portion.
+    assert any(n > 16 for step in engine.forwards for n in step)
+    sched.assert_idle()
+
+
+def test_a_prompt_that_can_never_fit_fails_and_the_next_runs(model_folders):
+    folder = model_folders["A"]
+    sched = Scheduler(cpu_engine(folder, num_pages=1, max_requests=2), SchedulerConfig(num_blocks=1, prefix_cache=False))
+    big = sched.add_request(random_ids(256, 17, 1), GenerateParams.greedy(2))
+    small_prompt = random_ids(256, 5, 2)
+    small = sched.add_request(small_prompt, GenerateParams.greedy(2))
+    results = sched.run()
+    assert isinstance(results[big], Failure)
+    assert results[big].message == "kv pool has 1 blocks of 16; this sequence needs 2"
+    assert results[small].tokens == solo(folder, small_prompt, GenerateParams.greedy(2)).tokens
+    # One that fits its prompt but outgrows the whole pool while decoding fails the same way.
+    grow = sched.add_request(random_ids(256, 15, 3), GenerateParams.greedy(5))
+    results = sched.run()
+    assert isinstance(results[grow], Failure) and "needs 2" in results[grow].message
+    sched.assert_idle()
+
+
+def test_requests_that_cannot_be_accepted(model_folders):
+    sched = Scheduler(cpu_engine(model_folders["A"]), SchedulerConfig(max_waiting=2))
+    empty = sched.add_request([], GenerateParams.greedy(3))
+    assert sched.finished[empty].message == "prompt encoded to no tokens"
+    too_long = sched.add_request(random_ids(256, 100, 1), GenerateParams.greedy(29))     # max_position_embeddings 128
+    assert "exceeds max_position_embeddings 128" in sched.finished[too_long].message
+    bad = sched.add_request([1, 2], GenerateParams(temperature=-1.0))
+    assert "negative" in sched.finished[bad].message
+    sched.add_request([1], GenerateParams.greedy(1))
+    sched.add_request([2], GenerateParams.greedy(1))
+    with pytest.raises(QueueFull):
+        sched.add_request([3], GenerateParams.greedy(1))
+    sched.run()
+    sched.assert_idle()
+
+
+def test_admission_is_first_in_first_out(model_folders):
+    # The big request at the front waits for pages; the small one behind it must not overtake.
+    folder = model_folders["A"]
+    engine = cpu_engine(folder, num_pages=4, max_requests=4)
+    sched = Scheduler(engine, SchedulerConfig(num_blocks=4, prefix_cache=False))
+    running = sched.add_request(random_ids(256, 30, 1), GenerateParams.greedy(3))
+    sched.step()
+    big = sched.add_request(random_ids(256, 40, 2), GenerateParams.greedy(2))      # 3 pages, only 2 free
+    small = sched.add_request(random_ids(256, 4, 3), GenerateParams.greedy(2))
+    sched.step()
+    assert [seq.id for seq in sched.running] == [running] and [seq.id for seq in sched.waiting] == [big, small]
+    results = sched.run()
+    assert all(isinstance(results[r], Generated) for r in (running, big, small))
+    sched.assert_idle()
+
+
+def test_a_request_joins_while_others_run(model_folders):
+    folder = model_folders["A"]
+    sched = Scheduler(cpu_engine(folder), SchedulerConfig())
+    p1, p2 = random_ids(256, 7, 1), random_ids(256, 11, 2)
+    first = sched.add_request(p1, GenerateParams.greedy(8))
+    for _ in range(3):
+        sched.step()
+    second = sched.add_request(p2, GenerateParams.greedy(4))
+    results = sched.run()
+    assert results[first].tokens == solo(folder, p1, GenerateParams.greedy(8)).tokens
+    assert results[second].tokens == solo(folder, p2, GenerateParams.greedy(4)).tokens
+    sched.assert_idle()
+
+
+def test_shared_prefix_is_reused_and_gives_the_same_tokens(model_folders):
+    folder = model_folders["A"]
+    prefix = random_ids(256, 48, 9)
+    ps = [prefix + random_ids(256, 5 + i, 20 + i) for i in range(3)]
+
+    def run(prefix_cache):
+        engine = cpu_engine(folder, num_pages=32, prefix_cache=prefix_cache)
+        sched = Scheduler(engine, SchedulerConfig(max_batch_size=2, num_blocks=32, prefix_cache=prefix_cache))
+        ids = [sched.add_request(p, GenerateParams.greedy(4)) for p in ps]
+        results = sched.run()
+        sched.assert_idle()
+        return [results[i].tokens for i in ids], engine.forwards, sched.stats
+
+    with_cache, forwards_on, stats_on = run(True)
+    without, forwards_off, stats_off = run(False)
+    assert with_cache == without
+    for prompt, tokens in zip(ps, with_cache):
+        assert tokens == solo(folder, prompt, GenerateParams.greedy(4)).tokens
+    # The third request starts after the first has published its pages: it runs only its own tail.
+    assert sum(map(sum, forwards_on)) == sum(map(sum, forwards_off)) - 48
+    assert stats_on.peak_blocks <= stats_off.peak_blocks
+
+
+def test_cancel(model_folders):
+    sched = Scheduler(cpu_engine(model_folders["A"]), SchedulerConfig())
+    rid = sched.add_request([1, 2, 3], GenerateParams.greedy(10))
+    waiting = sched.add_request([4, 5], GenerateParams.greedy(10))
+    sched.step()
+    sched.step()
+    sched.cancel(rid)
+    assert sched.finished[rid].reason == StopReason.Cancelled and len(sched.finished[rid].tokens) == 2
+    sched.cancel(waiting)
+    sched.run()
+    sched.assert_idle()

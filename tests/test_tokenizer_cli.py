@@ -1,0 +1,89 @@
+"""The byte-level BPE read from tokenizer.json (vectors of src/qwen.rs:359-453 of the reference) and the
+command line's argument rules (qwen-infer/src/main.rs:76-148).  The reference's 314 real cases
+(tests/fixtures/qwen_cases.jsonl) need the real tokenizer.json, which is not available: parity unpinned."""
+import json
+
+import pytest
+
+from tokenizer_amd.cli import ArgError, parse_args
+from tokenizer_amd.tokenizer import Tokenizer, TokenizerError, UnknownToken, bytes_to_unicode_reverse
+
+
+def tiny_file(pattern="[\\s\\S]+"):
+    reverse = bytes_to_unicode_reverse()
+    of_byte = {byte: ch for ch, byte in reverse.items()}
+    vocab = {of_byte[b]: b for b in range(256)}
+    vocab["ab"] = 256            # the merge result has id 256, not the merge's rank 0
+    return {"added_tokens": [{"id": 300, "content": "<|endoftext|>", "normalized": False, "special": True}],
+            "normalizer": {"type": "NFC"},
+            "pre_tokenizer": {"type": "Sequence", "pretokenizers": [
+                {"type": "Split", "pattern": {"Regex": pattern}, "behavior": "Isolated", "invert": False},
+                {"type": "ByteLevel", "add_prefix_space": False, "use_regex": False}]},
+            "model": {"type": "BPE", "vocab": vocab, "merges": ["a b"]}}
+
+
+def test_bytes_to_unicode_maps_the_known_bytes():
+    reverse = bytes_to_unicode_reverse()
+    assert len(reverse) == 256 and len(set(reverse.values())) == 256
+    assert reverse["Ā"] == 0 and reverse["Ġ"] == ord(" ")
+    assert reverse["!"] == ord("!") and reverse["a"] == ord("a")
+
+
+def test_merges_by_rank_not_id_and_applies_nfc(tmp_path):
+    path = tmp_path / "tokenizer.json"
+    path.write_text(json.dumps(tiny_file()))
+    tok = Tokenizer.load_qwen(str(path))
+    assert tok.encode("ab") == [256]
+    assert tok.encode("ba") == [ord("b"), ord("a")]
+    assert tok.encode("aba") == [256, ord("a")]
+    assert tok.decode([256]) == "ab"
+    composed = tok.encode("é")
+    assert tok.encode("é") == composed and composed != [ord("e"), 0xCC, 0x81]
+    assert tok.decode(composed) == "é"
+    ids = tok.encode("a<|endoftext|>b")
+    assert ids == [ord("a"), 300, ord("b")] and tok.decode(ids) == "a<|endoftext|>b"
+    with pytest.raises(UnknownToken):
+        tok.decode([257])
+    assert tok.decode_bytes([0xC3]) == b"\xc3"       # bytes, not replaced characters
+
+
+def test_gaps_the_pattern_leaves_are_pieces_too():
+    tok = Tokenizer.from_json(tiny_file(pattern="a+"))
+    assert tok.encode("xaabx") == [ord("x"), ord("a"), ord("a"), ord("b"), ord("x")]
+    tok = Tokenizer.from_json(tiny_file(pattern="(?i:'s)|[^\\r\\n\\p{L}\\p{N}]?\\p{L}+|\\p{N}| ?[^\\s\\p{L}\\p{N}]+[\\r\\n]*|\\s*[\\r\\n]+|\\s+(?!\\S)|\\s+"))
+    assert tok.decode(tok.encode("ab  cab 12's")) == "ab  cab 12's"
+    assert tok.encode("ab ab")[:1] == [256]
+
+
+@pytest.mark.parametrize("change, word", [
+    (lambda f: f["added_tokens"][0].update(normalized=True), "normalized"),
+    (lambda f: f.update(normalizer={"type": "NFKC"}), "NFC"),
+    (lambda f: f.update(normalizer=None), "no normalizer"),
+    (lambda f: f["pre_tokenizer"]["pretokenizers"][0].update(behavior="Removed"), "Isolated"),
+    (lambda f: f["pre_tokenizer"]["pretokenizers"][1].update(use_regex=True), "use_regex"),
+    (lambda f: f["model"].update(type="Unigram"), "BPE"),
+    (lambda f: f["model"]["vocab"].pop("a"), "missing single-byte token 97"),
+    (lambda f: f["model"].update(merges=["a c", "a c"]), "not in the vocab"),
+    (lambda f: f["model"].update(merges=["ab"]), "no space"),
+])
+def test_files_of_another_kind_are_refused(change, word):
+    data = tiny_file()
+    change(data)
+    with pytest.raises(TokenizerError) as err:
+        Tokenizer.from_json(data)
+    assert word in str(err.value)
+
+
+def test_command_line_arguments():
+    args = parse_args(["--model", "m", "The capital of France is"])
+    assert (args["max_tokens"], args["temperature"], args["top_p"], args["seed"], args["stop"]) == (20, 0.0, 1.0, 0, [])
+    args = parse_args(["--max-tokens", "7", "--temperature", "0.5", "--top-p", "0.9", "--seed", "3",
+                       "--stop", "a", "--stop", "b", "--model", "m", "hi"])
+    assert (args["max_tokens"], args["temperature"], args["top_p"], args["seed"], args["stop"], args["prompt"]) == \
+        (7, 0.5, 0.9, 3, ["a", "b"], "hi")
+    for bad, word in ((["-x", "p"], "unknown argument -x"), (["a", "b"], "only one prompt"),
+                      (["--max-tokens"], "needs a value"), (["--max-tokens", "x", "p"], "--max-tokens x"),
+                      (["--seed", "1.5", "p"], "--seed wants an integer")):
+        with pytest.raises(ArgError) as err:
+            parse_args(bad)
+        assert word in str(err.value)

@@ -1,0 +1,70 @@
+"""Entry points in the manner of qwen-infer's library (qwen-infer/src/lib.rs:14-24, 116-130):
+`generate`, `generate_with`, `greedy_tokens`."""
+from __future__ import annotations
+
+import time
+
+from .generate import Control, GenerateParams, Generated, SampleCursor, Sampled, StopReason, _go_on, _no_bytes
+from .batch import StepEntry
+
+
+def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes=_no_bytes,
+                  on_chunk=_go_on) -> Generated:
+    """Prefill `prompt`, then sample up to `params.max_tokens` ids, one cached forward per id.
+
+    The forward after the last allowed sample is not run; `max_tokens == 0` still runs the prompt;
+    the chunk callback is probed once with "" after the prompt so that a caller who is gone
+    cancels before the first draw (qwen-infer/src/generate.rs:340-394).
+    """
+    if not prompt:
+        raise ValueError("prompt encoded to no tokens")
+    cursor = SampleCursor(params)
+    rid = ("generate", id(cursor))
+    engine.add_request(rid)
+    try:
+        started = time.perf_counter()
+        wants = [len(prompt) - 1] if params.max_tokens > 0 else []
+        logits = engine.step([StepEntry(rid, list(prompt), wants)])
+        if wants:
+            logits_row = _row(engine, logits, cursor)
+        prefill = time.perf_counter() - started
+        started = time.perf_counter()
+        if params.max_tokens == 0:
+            done = cursor.finish_without_sample(on_chunk)
+        elif on_chunk("") == Control.Stop:
+            done = Sampled([], "", [], StopReason.Cancelled, 0)
+        else:
+            while True:
+                outcome = _push(cursor, logits_row, token_bytes, on_chunk)
+                if isinstance(outcome, Sampled):
+                    done = outcome
+                    break
+                logits = engine.step([StepEntry(rid, [int(outcome)], [0])])
+                logits_row = _row(engine, logits, cursor)
+        decode = time.perf_counter() - started
+    finally:
+        engine.end_request(rid)
+    return Generated(done.tokens, done.text, done.chunks, done.reason, done.completion_tokens, prefill, decode)
+
+
+def _row(engine, logits, cursor):
+    """Greedy: the id picked on the device; warm: the logits row on the host."""
+    if cursor.is_greedy:
+        return engine.argmax(logits, [0])[0]
+    return engine.rows_to_host(logits, [0])[0]
+
+
+def _push(cursor, picked, token_bytes, on_chunk):
+    if cursor.is_greedy:
+        return cursor.push_token(picked, token_bytes, on_chunk)
+    return cursor.push_logits(picked, token_bytes, on_chunk)
+
+
+def generate(engine, prompt: list[int], params: GenerateParams, token_bytes=_no_bytes) -> Generated:
+    return generate_with(engine, prompt, params, token_bytes, _go_on)
+
+
+def greedy_tokens(engine, prompt: list[int], new_tokens: int) -> list[int]:
+    """Greedy ids through the cache (the reference's `greedy_tokens` recomputes everything each step;
+    the ids are the same)."""
+    return generate(engine, prompt, GenerateParams.greedy(new_tokens)).tokens

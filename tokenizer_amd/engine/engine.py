@@ -89,6 +89,19 @@ class Engine:
                                                 writes=entry.cache_of is None))
         self.steps = 0
 
+    @property
+    def max_positions(self) -> int:
+        return self.model.max_positions
+
+    # ------------------------------------------------------------------- sampling
+    def argmax(self, logits: torch.Tensor, rows: list[int] | None = None) -> list[int]:
+        """Greedy ids of the given rows of a step's logits, picked on the device."""
+        picked = self.model.runtime.ops.argmax(logits).cpu().tolist()
+        return picked if rows is None else [picked[row] for row in rows]
+
+    def rows_to_host(self, logits: torch.Tensor, rows: list[int]):
+        return logits[rows].float().cpu().numpy()
+
     # ------------------------------------------------------------------ requests
     def add_request(self, rid) -> None:
         self.cache.add_request(rid)
