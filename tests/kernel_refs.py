@@ -63,7 +63,7 @@ class PlainOps:
                     continue
                 page, off = divmod(slot, page_size)
                 k_pages[page, :, off, :] = stored[t, n_q:n_q + n_kv]
-                v_pages[page, :, off, :] = stored[t, n_q + n_kv:]
+                v_pages[page, :, :, off] = stored[t, n_q + n_kv:]       # values lie transposed in a page
 
     def paged_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                         n_q, n_kv, head_dim, window, scale, max_position=None):
@@ -78,7 +78,7 @@ class PlainOps:
             assert all(p >= 0 for p in pages), "attention reads a page that was given back"
             offs = [j % page_size for j in keys]
             k = k_pages[pages, :, offs, :].to(self.work)     # [keys, n_kv, d]
-            v = v_pages[pages, :, offs, :].to(self.work)
+            v = v_pages[pages, :, :, offs].to(self.work)      # [keys, n_kv, d]
             q = qkv[t, :n_q * head_dim].reshape(n_q, head_dim).to(self.work)
             k = k.repeat_interleave(group, dim=1)            # [keys, n_q, d]
             v = v.repeat_interleave(group, dim=1)

@@ -104,7 +104,9 @@ def test_rope_store(ops, ref, dtype, geometry):
     for use_bias, use_rot in ((True, True), (False, True), (False, False)):
         a, b = qkv.clone(), qkv.clone()
         ka = torch.zeros((n_pages, n_kv, page_size, d), dtype=dtype).cuda()
-        va, kb, vb = ka.clone(), ka.clone(), ka.clone()
+        kb = ka.clone()
+        va = torch.zeros((n_pages, n_kv, d, page_size), dtype=dtype).cuda()
+        vb = va.clone()
         args = (bias if use_bias else None, positions, cos_sin if use_rot else None, slots)
         ops.rope_store(a, *args, ka, va, n_q, n_kv, d)
         ref.rope_store(b, *args, kb, vb, n_q, n_kv, d)
@@ -129,36 +131,78 @@ def make_paged_case(dtype, n_q, n_kv, d, page_size, lengths, q_lens, seed):
     width = max(pages_each)
     table = torch.full((n_entries, width), -1, dtype=torch.int32)
     k_pages = torch.randn((n_pages, n_kv, page_size, d), generator=gen).to(dtype)
-    v_pages = torch.randn((n_pages, n_kv, page_size, d), generator=gen).to(dtype)
+    v_pages = torch.randn((n_pages, n_kv, d, page_size), generator=gen).to(dtype)
     positions, entry_of_token = [], []
+    used = torch.zeros(n_pages, page_size, dtype=torch.bool)
     for e, (length, q_len) in enumerate(zip(lengths, q_lens)):
         for i in range(pages_each[e]):
             table[e, i] = order.pop()
+            used[table[e, i], :max(0, min(page_size, length - i * page_size))] = True
         positions += list(range(length - q_len, length))
         entry_of_token += [e] * q_len
+    # Slots no request wrote hold NaN: a kernel that lets them into a sum shows it.
+    k_pages[~used[:, None, :, None].expand_as(k_pages)] = float("nan")
+    v_pages[~used[:, None, None, :].expand_as(v_pages)] = float("nan")
     n_tokens = len(positions)
     qkv = torch.randn((n_tokens, (n_q + 2 * n_kv) * d), generator=gen).to(dtype)
     return (qkv.cuda(), k_pages.cuda(), v_pages.cuda(), torch.tensor(positions, dtype=torch.int32).cuda(),
             torch.tensor(entry_of_token, dtype=torch.int32).cuda(), table.cuda())
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("geometry", [(6, 3, 48, 16), (3, 1, 32, 16), (8, 2, 128, 32), (14, 2, 64, 16)])
+# (dtype, fast): the generic kernel in both dtypes, the matrix-core kernels in bfloat16.
+ATTENTION_MODES = [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)]
+
+
+@pytest.fixture()
+def attention_mode(ops, request):
+    dtype, fast = request.param
+    before = ops.use_fast_attention
+    ops.use_fast_attention = fast
+    yield dtype
+    ops.use_fast_attention = before
+
+
+def attention_tol(dtype, fast):
+    # The matrix-core kernels round the probabilities to bfloat16 before the product with the values.
+    return dict(rtol=2e-2, atol=8e-3) if fast else tol(dtype)
+
+
+@pytest.mark.parametrize("attention_mode", ATTENTION_MODES, indirect=True)
+@pytest.mark.parametrize("geometry", [(6, 3, 48, 16), (3, 1, 32, 16), (8, 2, 128, 32), (14, 2, 64, 16),
+                                      (20, 1, 16, 16), (4, 4, 80, 48), (2, 1, 256, 16)])
 @pytest.mark.parametrize("window", [None, 37])
-def test_paged_attention(ops, ref, dtype, geometry, window):
+def test_paged_attention(ops, ref, attention_mode, geometry, window):
+    dtype = attention_mode
     n_q, n_kv, d, page_size = geometry
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         dtype, n_q, n_kv, d, page_size, lengths=[1, 300, 64, 17], q_lens=[1, 5, 64, 1], seed=11)
     out_a = torch.empty((qkv.shape[0], n_q * d), dtype=dtype).cuda()
     out_b = torch.empty_like(out_a)
     scale = 1.0 / math.sqrt(d)
-    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=int(positions.max()))
     ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
-    torch.testing.assert_close(out_a.float(), out_b.float(), **tol(dtype))
+    torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(dtype, ops.use_fast_attention))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_paged_attention_finds_one_far_key(ops, dtype):
+@pytest.mark.parametrize("window", [None, 1000])
+def test_decode_attention_long_contexts_and_many_splits(ops, ref, window):
+    # Batches of single tokens at long, unequal contexts: the key range is cut into many splits.
+    n_q, n_kv, d, page_size = 14, 2, 64, 16
+    for lengths in ([3000], [2049, 1, 777, 4096, 31, 32, 33, 2500]):
+        qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+            torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=[1] * len(lengths), seed=13)
+        out_a = torch.empty((qkv.shape[0], n_q * d), dtype=torch.bfloat16).cuda()
+        out_b = torch.empty_like(out_a)
+        ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window,
+                            0.125, max_position=max(lengths) - 1)
+        ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, 0.125)
+        torch.testing.assert_close(out_a.float(), out_b.float(), rtol=2e-2, atol=4e-3)
+
+
+@pytest.mark.parametrize("attention_mode", ATTENTION_MODES, indirect=True)
+def test_paged_attention_finds_one_far_key(ops, attention_mode):
+    dtype = attention_mode
     # One key far back is made to dominate: the output must be its value row.
     n_q, n_kv, d, page_size = 4, 2, 64, 16
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
@@ -176,12 +220,12 @@ def test_paged_attention_finds_one_far_key(ops, dtype):
     ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, None, 1.0)
     got = out.reshape(n_q, d).float()
     for h in range(n_q):
-        torch.testing.assert_close(got[h], v_pages[page, h // 2, off].float(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(got[h], v_pages[page, h // 2, :, off].float(), rtol=2e-2, atol=2e-2)
     # With a window that ends just after the key, it is gone: position 699 sees keys >= 699 - w.
     ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, 699 - target - 1, 1.0)
-    assert (out.reshape(n_q, d).float()[0] - v_pages[page, 0, off].float()).abs().max() > 0.1
+    assert (out.reshape(n_q, d).float()[0] - v_pages[page, 0, :, off].float()).abs().max() > 0.1
     ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, 699 - target, 1.0)
-    torch.testing.assert_close(out.reshape(n_q, d).float()[0], v_pages[page, 0, off].float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(out.reshape(n_q, d).float()[0], v_pages[page, 0, :, off].float(), rtol=2e-2, atol=2e-2)
 
 
 def linear_tol(out_dtype, x, w):

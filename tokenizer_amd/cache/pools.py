@@ -9,9 +9,10 @@ _STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": 
 
 
 class CachePools:
-    """For group g: `pages[g]` of shape [layers in g, 2, num_pages, n_kv, page_size, d] (keys at 0, values
-    at 1) in the compute dtype.  For a layer with fixed-size state: `states[layer]` of shape
-    [max_requests, *state_shape]."""
+    """For group g: `pages[g]` of shape [layers in g, 2, num_pages, n_kv, page_size * d] (keys at 0, values
+    at 1) in the compute dtype.  Inside a page keys are laid out [page_size, d] and values transposed,
+    [d, page_size] (the layout the matrix-core attention kernels read).  For a layer with fixed-size
+    state: `states[layer]` of shape [max_requests, *state_shape]."""
 
     def __init__(self, manager: CacheManager, needs, dtype: torch.dtype, device):
         self.manager = manager
@@ -19,7 +20,7 @@ class CachePools:
         for group in manager.groups:
             need = group.need
             self.pages.append(torch.zeros((len(group.layers), 2, manager.num_pages, need.n_kv_heads,
-                                           manager.page_size, need.head_dim), dtype=dtype, device=device))
+                                           manager.page_size * need.head_dim), dtype=dtype, device=device))
         self.states = {}
         for layer, need in enumerate(needs):
             if need.state_shape is not None:
@@ -27,12 +28,17 @@ class CachePools:
                                                  dtype=_STATE_DTYPES[need.state_dtype], device=device)
 
     def layer_pages(self, layer: int):
-        """(keys, values) of one layer, each [num_pages, n_kv, page_size, d], or (None, None)."""
+        """(keys [num_pages, n_kv, page_size, d], values [num_pages, n_kv, d, page_size]) of one layer,
+        or (None, None)."""
         group = self.manager.group_of_layer[layer]
         if group is None:
             return None, None
+        need = self.manager.groups[group].need
         index = self.manager.groups[group].layers.index(layer)
-        return self.pages[group][index, 0], self.pages[group][index, 1]
+        pages, page_size = self.pages[group], self.manager.page_size
+        shape = (self.manager.num_pages, need.n_kv_heads)
+        return (pages[index, 0].view(*shape, page_size, need.head_dim),
+                pages[index, 1].view(*shape, need.head_dim, page_size))
 
     def bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.pages) + \

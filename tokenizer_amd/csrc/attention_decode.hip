@@ -1,0 +1,239 @@
+// Attention of single query tokens over paged bfloat16 keys and values on the matrix cores, with the
+// key range of every token split over several workgroups (partial results are merged by a second kernel).
+//
+// One workgroup handles one (token, kv head, block of up to 16 query heads, split).  The query heads that
+// share a kv head form the N dimension of the 16x16x32 MFMA, so keys and values are read once for all of
+// them.  Both products are computed transposed, S^T = K Q^T and O^T = V^T P^T, which keeps the head index
+// in `lane % 16` for scores and outputs alike: the online-softmax rescaling needs no cross-lane traffic.
+// Values are stored transposed inside a page ([page, kv head, d, slot]), so that the eight keys a lane
+// contracts over are contiguous in memory.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+// D: head size (multiple of 16).  Pages: K [n_pages, n_kv, page_size, D], V^T [n_pages, n_kv, D, page_size],
+// page_size a multiple of 16.  rows: the token rows to serve (null: row i = item i).
+// Token at position p sees keys max(0, p - window)..p (window < 0: from 0).
+// Partials: part_o [n_items, n_q, splits, D] (unnormalised), part_ml [n_items, n_q, splits, 2] (max, sum);
+// with splits == 1 the result goes straight to `out` [n_tokens, n_q * D].
+template <int D, int DEC_WAVES>
+__global__ void __launch_bounds__(DEC_WAVES * WAVE)
+decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+                        const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
+                        const int* __restrict__ rows, const int* __restrict__ positions,
+                        const int* __restrict__ entry_of_token, const int* __restrict__ block_table,
+                        int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
+                        int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits) {
+  constexpr int KS = (D + 31) / 32;   // 32-wide steps over the head size for Q K^T
+  constexpr int DB = D / 16;          // 16-row blocks of O^T
+  __shared__ float acc_s[DEC_WAVES][D][17];
+  __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16];
+
+  const int split = blockIdx.x;
+  const int group = n_q / n_kv;
+  const int head_blocks = (group + 15) / 16;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int item = blockIdx.z;
+  const int t = rows ? rows[item] : item;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, g = lane >> 4;
+  const int heads_here = min(16, group - hb * 16);
+  const int head = kvh * group + hb * 16 + col;          // valid when col < heads_here
+  const int pos = positions[t];
+  const int* table = block_table + (size_t)entry_of_token[t] * table_stride;
+  const int lo = (window >= 0 && pos > window) ? pos - window : 0;
+  const int first = (lo / 32) * 32 + split * split_keys;  // first key of this split (a multiple of 32)
+  const int last = min(pos, first + split_keys - 1);
+
+  // Q^T fragments: lane holds head `col`, head-size elements ks*32 + 8g .. +7.
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = ks * 32 + 8 * g;
+    qf[ks] = zero8();
+    if (col < heads_here && d0 < D)
+      qf[ks] = *reinterpret_cast<const bf16x8*>(q + (size_t)t * q_stride + (size_t)head * D + d0);
+  }
+  floatx4 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) acc[db] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int kb = first + wave * 32; kb <= last; kb += DEC_WAVES * 32) {
+    float s[2][4];
+    size_t page_base[2];
+    bool active[2];
+    uint64_t keep[2];   // 16 bits of ones for every visible key of the lane's four: slots nobody wrote may hold anything
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+      const int k0 = kb + tile * 16;                       // 16 keys of one page
+      active[tile] = (k0 <= last) && (k0 + 15 >= lo);
+      page_base[tile] = 0;
+      floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
+      if (active[tile]) {
+        const int page = table[k0 / page_size];
+        page_base[tile] = ((size_t)page * n_kv + kvh) * page_size * D;   // same element count for K and V^T pages
+        const bf16_t* kr = k_pages + page_base[tile] + (size_t)((k0 % page_size) + col) * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d0 = ks * 32 + 8 * g;
+          bf16x8 kf = zero8();
+          if (d0 < D) kf = *reinterpret_cast<const bf16x8*>(kr + d0);
+          st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], st, 0, 0, 0);
+        }
+      }
+      keep[tile] = 0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = k0 + 4 * g + r;
+        const bool seen = active[tile] && key >= lo && key <= last;
+        s[tile][r] = seen ? st[r] * scale : -INFINITY;
+        if (seen) keep[tile] |= (uint64_t)0xffff << (16 * r);
+      }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                     fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m, mx);
+    if (m_new == -INFINITY) continue;                      // nothing visible yet (uniform over the head's lanes)
+    const float corr = __expf(m - m_new);
+    bf16x8 pf;
+    float psum = 0.f;
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = __expf(s[tile][r] - m_new);        // exp(-inf) = 0 for masked keys
+        psum += p;
+        pf[tile * 4 + r] = (__bf16)p;
+      }
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      // V^T fragment: row d = db*16 + col, slots 0..3 = keys 4g..4g+3 of tile 0, slots 4..7 of tile 1.
+      bf16x8 vf = zero8();
+#pragma unroll
+      for (int tile = 0; tile < 2; ++tile) {
+        if (active[tile]) {
+          const int k0 = kb + tile * 16;
+          const bf16_t* vr = vt_pages + page_base[tile] + (size_t)(db * 16 + col) * page_size + (k0 % page_size) + 4 * g;
+          union { uint64_t bits; bf16x4 v; } v4;
+          v4.bits = *reinterpret_cast<const uint64_t*>(vr) & keep[tile];   // 0 * NaN would poison the sum
+#pragma unroll
+          for (int r = 0; r < 4; ++r) vf[tile * 4 + r] = v4.v[r];
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[db][r] *= corr;
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[db], 0, 0, 0);
+    }
+  }
+  // Sum of the lane groups' partial denominators (the maximum is already common to them).
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc_s[wave][db * 16 + 4 * g + r][col] = acc[db][r];
+  if (g == 0) { m_s[wave][col] = m; l_s[wave][col] = l; }
+  __syncthreads();
+  // Merge the waves: thread (head h, element block) walks over D.
+  for (int idx = threadIdx.x; idx < 16 * D; idx += DEC_WAVES * WAVE) {
+    const int h = idx / D, d = idx % D;
+    if (h >= heads_here) continue;
+    float big = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) big = fmaxf(big, m_s[w][h]);
+    float o = 0.f, denom = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      const float wgt = (m_s[w][h] == -INFINITY) ? 0.f : __expf(m_s[w][h] - big);
+      o += acc_s[w][d][h] * wgt;
+      denom += l_s[w][h] * wgt;
+    }
+    const int hg = kvh * group + hb * 16 + h;
+    if (splits == 1) {
+      st(out + (size_t)t * n_q * D + (size_t)hg * D + d, o / denom);
+    } else {
+      const size_t p = ((size_t)item * n_q + hg) * splits + split;
+      part_o[p * D + d] = o;
+      if (d == 0) { part_ml[p * 2] = big; part_ml[p * 2 + 1] = denom; }
+    }
+  }
+}
+
+// out[t, head, :] = sum_s part_o[s] * exp(m_s - M) / sum_s l_s * exp(m_s - M).  One block per (item, head).
+__global__ void decode_attention_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                       const int* __restrict__ rows, bf16_t* __restrict__ out,
+                                       int n_q, int d, int splits) {
+  const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
+  const int t = rows ? rows[item] : item;
+  const size_t base = ((size_t)item * n_q + head) * splits;
+  float big = -INFINITY;
+  for (int s = 0; s < splits; ++s) big = fmaxf(big, part_ml[(base + s) * 2]);
+  float denom = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = part_ml[(base + s) * 2];
+    if (ms != -INFINITY) denom += part_ml[(base + s) * 2 + 1] * __expf(ms - big);
+  }
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = part_ml[(base + s) * 2];
+      if (ms != -INFINITY) o += part_o[(base + s) * d + i] * __expf(ms - big);
+    }
+    st(out + (size_t)t * n_q * d + (size_t)head * d + i, o / denom);
+  }
+}
+
+template <int D>
+static int launch_decode(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
+                         const void* rows, const void* positions, const void* entry_of_token,
+                         const void* block_table, int table_stride, void* part_o, void* part_ml, int n_items,
+                         int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
+                         hipStream_t stream) {
+  const int group = n_q / n_kv;
+  dim3 grid(splits, n_kv * ((group + 15) / 16), n_items);
+  constexpr int NW = D > 128 ? 2 : 4;   // keeps the merge buffer within 64 KB of LDS
+  decode_attention_kernel<D, NW><<<grid, NW * WAVE, 0, stream>>>(
+      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)rows,
+      (const int*)positions, (const int*)entry_of_token, (const int*)block_table, table_stride, (float*)part_o,
+      (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits);
+  int status = LAUNCH_STATUS();
+  if (status == 0 && splits > 1) {
+    decode_attention_merge<<<n_items * n_q, 64, 0, stream>>>((const float*)part_o, (const float*)part_ml,
+                                                             (const int*)rows, (bf16_t*)out, n_q, D, splits);
+    status = LAUNCH_STATUS();
+  }
+  return status;
+}
+
+// Returns -2 for a head size this kernel has no instance for (the caller then uses the generic kernel).
+extern "C" int ta_decode_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
+                                        const void* vt_pages, const void* rows, const void* positions,
+                                        const void* entry_of_token, const void* block_table, int table_stride,
+                                        void* part_o, void* part_ml, int n_items, int n_q, int n_kv, int d,
+                                        int page_size, int window, float scale, int split_keys, int splits,
+                                        hipStream_t stream) {
+  if (n_items <= 0) return 0;
+  if (n_kv <= 0 || n_q % n_kv || page_size % 16 || split_keys % 32 || splits < 1) return -1;
+#define CASE(DD) case DD: return launch_decode<DD>(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, \
+    block_table, table_stride, part_o, part_ml, n_items, n_q, n_kv, page_size, window, scale, split_keys, splits, stream);
+  switch (d) {
+    CASE(16) CASE(32) CASE(48) CASE(64) CASE(80) CASE(96) CASE(112) CASE(128) CASE(160) CASE(192) CASE(224) CASE(256)
+    default: return -2;
+  }
+#undef CASE
+}

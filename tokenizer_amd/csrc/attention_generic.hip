@@ -8,7 +8,8 @@
 
 // q: rows of `q_stride` elements, head h at h*d.  out: [n_tokens, n_q*d].
 // Token t at position p of entry e sees keys max(0, p-window)..p (window < 0: all from 0), whose
-// pages are block_table[e, key / page_size].  Pages: [n_pages, n_kv, page_size, d].
+// pages are block_table[e, key / page_size].  Key pages: [n_pages, n_kv, page_size, d]; value pages
+// are transposed inside a page: [n_pages, n_kv, d, page_size].
 template <typename T>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
 paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ out,
@@ -36,11 +37,12 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   for (int base = wave * WAVE; base < n_keys; base += ATT_WAVES * WAVE) {
     const int j = lo + base + lane;
     const bool valid = base + lane < n_keys;
-    int row = 0;
+    int row = 0, vbase = 0;   // key row, and start of this key's column in the value page
     float s = -INFINITY;
     if (valid) {
       const int page = table[j / page_size];
       row = (page * n_kv + kvh) * page_size + (j % page_size);
+      vbase = (page * n_kv + kvh) * page_size * d + (j % page_size);
       const T* kr = k_pages + (size_t)row * d;
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot += q_s[i] * ld(kr + i);
@@ -55,12 +57,11 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
     const int count = min(WAVE, n_keys - base);
     for (int jj = 0; jj < count; ++jj) {
       const float pj = __shfl(p, jj, WAVE);
-      const int vrow = __shfl(row, jj, WAVE);
-      const T* vr = v_pages + (size_t)vrow * d;
+      const T* vr = v_pages + (size_t)__shfl(vbase, jj, WAVE);
 #pragma unroll
       for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
         const int i = lane + r * WAVE;
-        if (i < d) acc[r] += pj * ld(vr + i);
+        if (i < d) acc[r] += pj * ld(vr + (size_t)i * page_size);
       }
     }
     m = m_new;

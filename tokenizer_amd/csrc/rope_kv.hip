@@ -6,7 +6,8 @@
 // qkv: [n_tokens, row_stride], heads of size d.  bias (float, may be null) is added first.
 // cos_sin: [max_positions, d] float, cos of the d/2 angles then sin; null = no rotation.
 // slots: physical slot of each token (page * page_size + offset), or null = nothing is stored.
-// Pages: [n_pages, n_kv, page_size, d].
+// Key pages: [n_pages, n_kv, page_size, d]; value pages are transposed inside a page,
+// [n_pages, n_kv, d, page_size], so that the keys a matrix-core lane contracts over lie side by side.
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
                                   const int* __restrict__ positions, const float* __restrict__ cos_sin,
@@ -20,12 +21,15 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
   const bool is_v = head >= n_q + n_kv;
   const bool is_k = !is_v && head >= n_q;
   T* dst = nullptr;
+  int dst_stride = 1;   // distance between consecutive elements of the head in the page
   if ((is_k || is_v) && slots) {
     const int slot = slots[t];
     if (slot >= 0) {
       const int page = slot / page_size, off = slot - page * page_size;
       const int kvh = is_k ? head - n_q : head - n_q - n_kv;
-      dst = (is_k ? k_pages : v_pages) + (((size_t)page * n_kv + kvh) * page_size + off) * d;
+      T* base = (is_k ? k_pages : v_pages) + ((size_t)page * n_kv + kvh) * page_size * d;
+      if (is_k) dst = base + (size_t)off * d;
+      else { dst = base + off; dst_stride = page_size; }
     }
   }
   if (is_v || !cos_sin) {
@@ -33,7 +37,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
     for (int i = threadIdx.x; i < d; i += blockDim.x) {
       float v = ld(x + i);
       if (b) { v += b[i]; st(x + i, v); }
-      if (dst) st(dst + i, v);
+      if (dst) st(dst + (size_t)i * dst_stride, v);
     }
     return;
   }

@@ -52,7 +52,8 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_gemm_f32", "ta_gemm_bf16", "ta_argmax"):
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16",
+                     "ta_argmax"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     @staticmethod
@@ -122,7 +123,7 @@ class Ops:
         qkv [T, (n_q + 2 n_kv) d]; bias float32 or None; positions int32 [T];
         cos_sin float32 [P, d] (cos half, sin half) or None for no rotation;
         slots int32 [T] (page * page_size + offset, negative = skip) or None;
-        pages [n_pages, n_kv, page_size, d].
+        key pages [n_pages, n_kv, page_size, d], value pages [n_pages, n_kv, d, page_size].
         """
         _dev(qkv, bias, positions, cos_sin, slots, k_pages, v_pages)
         n_tokens, width = qkv.shape
@@ -138,12 +139,20 @@ class Ops:
             _need(slots.dtype == torch.int32 and slots.numel() == n_tokens, "slots must be int32 [T]")
             _need(k_pages is not None and v_pages is not None, "slots without pages")
             _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
-            _need(k_pages.dim() == 4 and k_pages.shape[1] == n_kv and k_pages.shape[3] == head_dim
-                  and v_pages.shape == k_pages.shape, "pages must be [n_pages, n_kv, page_size, d]")
-            page_size = k_pages.shape[2]
+            page_size = self._page_size(k_pages, v_pages, n_kv, head_dim)
         self._check(self.lib.ta_rope_store(_ptr(qkv), width, _ptr(bias), _ptr(positions), _ptr(cos_sin),
                                            _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_tokens, n_q, n_kv,
                                            head_dim, page_size, _code(qkv.dtype), self._stream()), "rope_store")
+
+    @staticmethod
+    def _page_size(k_pages: torch.Tensor, v_pages: torch.Tensor, n_kv: int, head_dim: int) -> int:
+        _need(k_pages.dim() == 4 and k_pages.shape[1] == n_kv and k_pages.shape[3] == head_dim,
+              "key pages must be [n_pages, n_kv, page_size, d]")
+        page_size = k_pages.shape[2]
+        _need(tuple(v_pages.shape) == (k_pages.shape[0], n_kv, head_dim, page_size),
+              "value pages must be [n_pages, n_kv, d, page_size]")
+        _need(k_pages.numel() < 2 ** 31, "a layer's pages must hold fewer than 2^31 elements")
+        return page_size
 
     # ------------------------------------------------------------------ attention
     def paged_attention(self, qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor,
@@ -152,7 +161,8 @@ class Ops:
                         window: int | None, scale: float, max_position: int | None = None) -> torch.Tensor:
         """Causal attention of every token over the pages of its request.
 
-        qkv [T, >= n_q d] (query heads first); out [T, n_q d]; pages [n_pages, n_kv, page_size, d];
+        qkv [T, >= n_q d] (query heads first); out [T, n_q d]; key pages [n_pages, n_kv, page_size, d],
+        value pages [n_pages, n_kv, d, page_size];
         positions, entry_of_token int32 [T]; block_table int32 [E, P]; a token at position p sees keys
         max(0, p - window)..p.  `max_position` (host) lets the wrapper check that the table is wide enough.
         """
@@ -160,21 +170,51 @@ class Ops:
         n_tokens = qkv.shape[0]
         _need(qkv.shape[1] >= n_q * head_dim, "qkv is narrower than the query heads")
         _need(tuple(out.shape) == (n_tokens, n_q * head_dim) and out.dtype == qkv.dtype, "attention output shape")
-        _need(k_pages.dtype == qkv.dtype and k_pages.dim() == 4 and k_pages.shape[1] == n_kv
-              and k_pages.shape[3] == head_dim and v_pages.shape == k_pages.shape, "pages must be [n_pages, n_kv, page_size, d]")
+        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
+        page_size = self._page_size(k_pages, v_pages, n_kv, head_dim)
         _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
         _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() == n_tokens, "entry_of_token must be int32 [T]")
         _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 [E, P]")
         _need(n_kv > 0 and n_q % n_kv == 0, "query heads must be a multiple of kv heads")
         _need(0 < head_dim <= 256, "head sizes up to 256 are supported")
-        page_size = k_pages.shape[2]
         if max_position is not None:
             _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
+        if (qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
+                and qkv.shape[1] % 8 == 0 and self.use_fast_attention):
+            return self._decode_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
+                                          n_q, n_kv, head_dim, page_size, window, scale, max_position)
         self._check(self.lib.ta_paged_attention_generic(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(positions),
             _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], n_tokens, n_q, n_kv, head_dim,
             page_size, -1 if window is None else int(window), ctypes.c_float(scale), _code(qkv.dtype),
             self._stream()), "paged_attention")
+        return out
+
+    DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
+    use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
+    target_workgroups = 1024      # what the split of the key range aims at
+
+    def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
+                          n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None):
+        """Matrix-core attention of single tokens with the key range split over workgroups."""
+        n_items = qkv.shape[0] if rows is None else rows.numel()
+        max_keys = (block_table.shape[1] * page_size) if max_position is None else max_position + 1
+        if window is not None:
+            max_keys = min(max_keys, window + 32)
+        head_blocks = -(-(n_q // n_kv) // 16)
+        per_split = max(1, self.target_workgroups // max(1, n_items * n_kv * head_blocks))
+        split_keys = max(128, -(-max_keys // per_split))
+        split_keys = -(-split_keys // 32) * 32
+        splits = max(1, -(-(max_keys + 31) // split_keys))
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty((n_items, n_q, splits, head_dim), dtype=torch.float32, device=qkv.device)
+            part_ml = torch.empty((n_items, n_q, splits, 2), dtype=torch.float32, device=qkv.device)
+        self._check(self.lib.ta_decode_attention_bf16(
+            _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(rows), _ptr(positions),
+            _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], _ptr(part_o), _ptr(part_ml), n_items,
+            n_q, n_kv, head_dim, page_size, -1 if window is None else int(window), ctypes.c_float(scale),
+            split_keys, splits, self._stream()), "decode_attention")
         return out
 
     # --------------------------------------------------------------------- linear
