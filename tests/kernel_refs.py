@@ -99,6 +99,11 @@ class PlainOps:
             return out
         return y
 
+    def linear_silu_gate(self, x, weight, out=None):
+        inner = weight.shape[0] // 2
+        result = torch.empty((x.shape[0], inner), dtype=x.dtype, device=x.device) if out is None else out
+        return self.silu_gate(self.linear(x, weight), result)
+
     def argmax(self, logits, out=None):
         result = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device) if out is None else out
         for row in range(logits.shape[0]):

@@ -257,6 +257,38 @@ def test_linear(ops, ref, dtype, shape):
     torch.testing.assert_close(got.double(), want, **linear_tol(torch.float32, x, w))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 272, 96), (8, 4864, 896), (33, 130, 72), (64, 176, 80), (100, 128, 64)])
+def test_linear_silu_gate(ops, ref, dtype, shape):
+    m, inner, k = shape
+    x = rand((m, k), dtype, 30)
+    w = rand((2 * inner, k), dtype, 31, 0.1)
+    got = ops.linear_silu_gate(x, w)
+    want = torch.empty((m, inner), dtype=torch.float64).cuda()
+    gate_up = ref.linear(x, w, None, out_dtype=torch.float64)
+    ref.silu_gate(gate_up, want)
+    # Unfused, the products are rounded to the storage dtype before the activation; allow for that.
+    base = linear_tol(dtype, x, w)
+    torch.testing.assert_close(got.double(), want, rtol=2 * base["rtol"], atol=4 * base["atol"] + (2e-2 if dtype == torch.bfloat16 else 0))
+
+
+@pytest.mark.parametrize("shape", [(1, 1152, 896), (8, 896, 4864), (64, 151, 896), (17, 100, 40), (48, 3000, 264)])
+def test_skinny_rows_agree_with_the_tiled_kernel(ops, shape):
+    # The same product through the weight-streaming kernel and through the tiled one.
+    m, n, k = shape
+    x = rand((m, k), torch.bfloat16, 32)
+    w = rand((n, k), torch.bfloat16, 33, 0.1)
+    bias = rand((n,), torch.float32, 34)
+    skinny = ops.linear(x, w, bias, out_dtype=torch.float32)
+    before = ops.SKINNY_ROWS
+    try:
+        ops.SKINNY_ROWS = 0
+        tiled = ops.linear(x, w, bias, out_dtype=torch.float32)
+    finally:
+        ops.SKINNY_ROWS = before
+    torch.testing.assert_close(skinny, tiled, **linear_tol(torch.float32, x, w))
+
+
 def test_linear_float32_is_true_float32(ops):
     # Inputs that need 13 mantissa bits: a reduced-precision matrix mode (10 or 7 bits) would be off by
     # about 1e-2 here, float32 accumulation by less than 3e-4.

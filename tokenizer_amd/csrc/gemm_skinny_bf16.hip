@@ -1,0 +1,182 @@
+// C[M,N] = A[M,K] * W[N,K]^T (+ bias) for few rows (M <= 64): the decode-time product, bound by the
+// one pass over the weights.  Computed transposed on the matrix cores, C^T = W A^T: sixteen weight rows are
+// the M side of a 16x16x32 MFMA, up to four blocks of sixteen activation rows the N side, so every weight
+// element is loaded once, 16 bytes per lane.  The waves of a workgroup split K between them and add up
+// through LDS.  With GATED the kernel computes silu(A Wg^T) * (A Wu^T) for W = [Wg; Wu] in one pass.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p, bool ok) {
+  bf16x8 z;
+  if (ok) return *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+__device__ __forceinline__ void store4(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float* v) {
+  uint2 packed;
+  packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+  packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = packed;
+}
+__device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+__device__ __forceinline__ void store1(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
+
+// grid.x: tiles of 16 output columns (of N, or of N/2 with GATED).  NW waves per workgroup.
+template <int MB, int NW, bool GATED, typename OutT>
+__global__ void __launch_bounds__(NW * WAVE)
+skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
+                   const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K) {
+  constexpr int SETS = GATED ? 2 : 1;
+  __shared__ float red[NW][SETS * MB * 4][WAVE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, g = lane >> 4;
+  const int n_out = GATED ? N / 2 : N;
+  const int n0 = blockIdx.x * 16;
+  // Rows past the end are clamped, not masked: they only feed outputs that are never stored.
+  const int wrow = min(n0 + col, n_out - 1);
+  const bf16_t* w0 = W + (size_t)wrow * K + 8 * g;
+  const bf16_t* w1 = W + (size_t)(wrow + n_out) * K + 8 * g;     // the `up` rows when GATED
+  const bf16_t* a_row[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) a_row[mb] = A + (size_t)min(mb * 16 + col, M - 1) * lda + 8 * g;
+
+  floatx4 acc[SETS][MB];
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[s][mb] = (floatx4){0.f, 0.f, 0.f, 0.f};
+
+  const int full_steps = K / 32;
+  // Four steps at a time, all loads first, so that many are in flight per lane.
+  constexpr int UN = (SETS * MB > 4) ? 2 : 4;
+  int ks = wave;
+  for (; ks + (UN - 1) * NW < full_steps; ks += UN * NW) {
+    bf16x8 wf[UN][SETS], af[UN][MB];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int k = (ks + u * NW) * 32;
+      wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + k);
+      if (GATED) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + k);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) af[u][mb] = *reinterpret_cast<const bf16x8*>(a_row[mb] + k);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int s = 0; s < SETS; ++s)
+          acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][s], af[u][mb], acc[s][mb], 0, 0, 0);
+  }
+  for (; ks < full_steps; ks += NW) {
+    const int k = ks * 32;
+    bf16x8 wf[SETS];
+    wf[0] = *reinterpret_cast<const bf16x8*>(w0 + k);
+    if (GATED) wf[SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + k);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const bf16x8 af = *reinterpret_cast<const bf16x8*>(a_row[mb] + k);
+#pragma unroll
+      for (int s = 0; s < SETS; ++s)
+        acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af, acc[s][mb], 0, 0, 0);
+    }
+  }
+  if ((K & 31) && wave == full_steps % NW) {              // the tail of K (a multiple of 8), zero-filled
+    const int k = full_steps * 32;
+    const bool k_ok = k + 8 * g < K;
+    const bf16x8 wf0 = load8(w0 + k, k_ok);
+    bf16x8 wf1;
+    if (GATED) wf1 = load8(w1 + k, k_ok);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const bf16x8 af = load8(a_row[mb] + k, k_ok);
+      acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, af, acc[0][mb], 0, 0, 0);
+      if (GATED) acc[SETS - 1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, af, acc[SETS - 1][mb], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][(s * MB + mb) * 4 + r][lane] = acc[s][mb][r];
+  __syncthreads();
+  // Lane (col, g) of block mb holds C^T rows n0 + 4g + r (r = 0..3), column m = mb*16 + col.
+  for (int item = threadIdx.x; item < MB * WAVE; item += NW * WAVE) {
+    const int mb = item / WAVE, ln = item % WAVE;
+    const int m = mb * 16 + (ln & 15);
+    const int n = n0 + 4 * (ln >> 4);
+    if (m >= M || n >= n_out) continue;
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sum0 = 0.f, sum1 = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        sum0 += red[w][mb * 4 + r][ln];
+        if (GATED) sum1 += red[w][(MB + mb) * 4 + r][ln];
+      }
+      if (bias && n + r < n_out) sum0 += bias[n + r];
+      v[r] = GATED ? sum0 / (1.0f + __expf(-sum0)) * sum1 : sum0;
+    }
+    OutT* dst = C + (size_t)m * ldc + n;
+    if (n + 3 < n_out && (ldc & 3) == 0) {
+      store4(dst, v);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < n_out) store1(dst + r, v[r]);
+    }
+  }
+}
+
+template <int MB, int NW, bool GATED>
+static int launch_skinny(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
+                         int K, int out_dtype, hipStream_t stream) {
+  const int n_out = GATED ? N / 2 : N;
+  const int tiles = (n_out + 15) / 16;
+  if (out_dtype == DT_F32)
+    skinny_gemm_kernel<MB, NW, GATED, float><<<tiles, NW * WAVE, 0, stream>>>(
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (float*)C, ldc, M, N, K);
+  else
+    skinny_gemm_kernel<MB, NW, GATED, bf16_t><<<tiles, NW * WAVE, 0, stream>>>(
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)C, ldc, M, N, K);
+  return LAUNCH_STATUS();
+}
+
+template <int MB, bool GATED>
+static int pick_waves(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
+                      int K, int out_dtype, hipStream_t stream) {
+  // Few output tiles and a long K: more waves per tile, so that enough loads are in flight.
+  const int tiles = ((GATED ? N / 2 : N) + 15) / 16;
+  const int k_steps = (K + 31) / 32;
+  if (tiles >= 1024 || k_steps <= 8)
+    return launch_skinny<MB, 4, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+  if (tiles >= 256 || k_steps <= 32 || MB * (GATED ? 2 : 1) > 2)
+    return launch_skinny<MB, 8, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+  return launch_skinny<MB, 16, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+}
+
+// M <= 64; K, lda multiples of 8; pointers 16-byte aligned; with `gated` N is even and C is [M, N/2].
+extern "C" int ta_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* bias, void* C, int ldc,
+                                   int M, int N, int K, int out_dtype, int gated, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || (K & 7) || (lda & 7) || (gated && (N & 1))) return -1;
+  const int mb = (M + 15) / 16;
+#define GO(MBV) (gated ? pick_waves<MBV, true>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream) \
+                       : pick_waves<MBV, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream))
+  switch (mb) {
+    case 1: return GO(1);
+    case 2: return GO(2);
+    case 3: return GO(3);
+    default: return GO(4);
+  }
+#undef GO
+}

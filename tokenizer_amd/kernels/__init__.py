@@ -52,7 +52,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16",
                      "ta_argmax"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -247,10 +247,37 @@ class Ops:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-            status = self.lib.ta_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
-                                           _code(out_dtype), self._stream())
+            if m <= self.SKINNY_ROWS:
+                status = self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, m, n, k,
+                                                      _code(out_dtype), 0, self._stream())
+            else:
+                status = self.lib.ta_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
+                                               _code(out_dtype), self._stream())
         self._check(status, "linear")
         return out
+
+    SKINNY_ROWS = 64    # up to this many rows the weight-streaming kernel runs
+
+    def linear_silu_gate(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """out = silu(x @ Wg.T) * (x @ Wu.T) for weight = [Wg; Wu] of shape [2I, K]; out [M, I].
+
+        Few bfloat16 rows run in one kernel; otherwise the product and the gated activation are two."""
+        _need(weight.dim() == 2 and weight.shape[0] % 2 == 0, "the joined gate and up matrix has an even row count")
+        m, inner = x.shape[0], weight.shape[0] // 2
+        if out is None:
+            out = torch.empty((m, inner), dtype=x.dtype, device=x.device)
+        _need(tuple(out.shape) == (m, inner) and out.dtype == x.dtype and out.is_contiguous(), "gated output shape")
+        if x.dtype == torch.bfloat16 and m <= self.SKINNY_ROWS:
+            _need(x.is_cuda and weight.is_cuda and x.dim() == 2 and x.shape[1] == weight.shape[1], "linear shapes do not fit")
+            _need(x.stride(1) == 1 and weight.is_contiguous() and weight.dtype == torch.bfloat16, "linear operands")
+            k = x.shape[1]
+            lda = x.stride(0) if m > 1 else k
+            _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
+            _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+            self._check(self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), None, _ptr(out), inner, m, 2 * inner,
+                                                     k, _BF16, 1, self._stream()), "linear_silu_gate")
+            return out
+        return self.silu_gate(self.linear(x, weight), out)
 
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:

@@ -30,7 +30,4 @@ class GatedDense(FeedForward):
 
     def forward(self, x, ctx):
         ops = self.runtime.ops
-        gate_up = ops.linear(x, self.w_gate_up)
-        act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
-        ops.silu_gate(gate_up, act)
-        return ops.linear(act, self.w_down)
+        return ops.linear(ops.linear_silu_gate(x, self.w_gate_up), self.w_down)
