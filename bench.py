@@ -136,6 +136,7 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--layers", type=int, default=FULL_LAYERS)
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; runs with --gpus > 1 are not supported")
@@ -152,6 +153,10 @@ def main() -> int:
     weights = weight_bytes_per_step(model)
     kv_token = kv_bytes_per_token(cfg, itemsize)
 
+    if args.only_prefill:
+        seconds = run_prefill(model)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PROMPT_LEN}), flush=True)
+        return 0
     log(f"decode at batch {args.batch}: {args.warmup} warmup + {args.steps} timed steps")
     elapsed, kv_mean = run_decode(model, args.batch, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3

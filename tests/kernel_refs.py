@@ -66,7 +66,7 @@ class PlainOps:
                 v_pages[page, :, :, off] = stored[t, n_q + n_kv:]       # values lie transposed in a page
 
     def paged_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
-                        n_q, n_kv, head_dim, window, scale, max_position=None):
+                        n_q, n_kv, head_dim, window, scale, max_position=None, batch=None):
         page_size = k_pages.shape[2]
         group = n_q // n_kv
         for t in range(qkv.shape[0]):

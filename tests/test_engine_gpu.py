@@ -148,3 +148,40 @@ def test_trace_run_program(model_folders, oracle, tmp_path, dtype):
     for rid, ids in reqs.items():
         want = oracle(name, ids)[asked[rid]]
         close(got[rid], want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
+    # The same trace with and without graph replay: decode steps of changing batch size, with prompt
+    # portions (never captured) between them, each replay checked against the eager engine.
+    from tokenizer_amd.engine import StepEntry
+    name = "B"
+    vocab = TINY[name][0]["vocab_size"]
+    engines = [engine_for(model_folders[name], dtype, max_tokens=1024, max_requests=4, use_graphs=flag)
+               for flag in (True, False)]
+    assert engines[0].use_graphs and not engines[1].use_graphs
+    prompts = {rid: random_ids(vocab, n, 50 + rid) for rid, n in enumerate([37, 5, 64])}
+    for eng in engines:
+        for rid, ids in prompts.items():
+            eng.add_request(rid)
+    rng_tokens = random_ids(vocab, 400, 77)
+    plan = [[0], [0, 1], [0, 1, 2], "prefill", [0, 2], [1], [0, 1, 2], [0, 1, 2], "prefill", [2], [0, 1, 2]] * 3
+    at = 0
+    for action in plan:
+        if action == "prefill":
+            entries = [StepEntry(1, rng_tokens[at:at + 3], [2]), StepEntry(0, rng_tokens[at + 3:at + 4], [0])]
+            at += 4
+        else:
+            entries = [StepEntry(rid, [rng_tokens[at + i]], [0]) for i, rid in enumerate(action)]
+            at += len(action)
+        if action == [0]:
+            entries = [StepEntry(rid, e.tokens, e.want) if True else e for rid, e in zip(action, entries)]
+        got = []
+        for eng in engines:
+            if not all(eng.cache.seq_len(e.rid) for e in entries):          # first use: run the prompt
+                eng.step([StepEntry(e.rid, prompts[e.rid], []) for e in entries if not eng.cache.seq_len(e.rid)])
+            logits = eng.step(entries)
+            got.append((logits.float().cpu().clone(), eng.argmax(logits)))
+        torch.testing.assert_close(got[0][0], got[1][0], rtol=0, atol=0)
+        assert got[0][1] == got[1][1]
+    assert len(engines[0].graphs) >= 3

@@ -149,6 +149,23 @@ def make_paged_case(dtype, n_q, n_kv, d, page_size, lengths, q_lens, seed):
             torch.tensor(entry_of_token, dtype=torch.int32).cuda(), table.cuda())
 
 
+def make_batch(lengths, q_lens):
+    """What the engine's step context tells the attention kernels about a batch."""
+    import types
+    cu_q, first, tiles, rows = [0], [], [], []
+    for e, (length, q_len) in enumerate(zip(lengths, q_lens)):
+        first.append(length - q_len)
+        if q_len == 1:
+            rows.append(cu_q[-1])
+        else:
+            for offset in range(0, q_len, 16):
+                tiles += [e, offset]
+        cu_q.append(cu_q[-1] + q_len)
+    as_int = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
+    return types.SimpleNamespace(n_tokens=cu_q[-1], cu_q=as_int(cu_q), first_position=as_int(first),
+                                 q_tiles=as_int(tiles).reshape(-1, 2), decode_rows=as_int(rows))
+
+
 # (dtype, fast): the generic kernel in both dtypes, the matrix-core kernels in bfloat16.
 ATTENTION_MODES = [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)]
 
@@ -183,6 +200,29 @@ def test_paged_attention(ops, ref, attention_mode, geometry, window):
                         max_position=int(positions.max()))
     ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
     torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(dtype, ops.use_fast_attention))
+    if ops.use_fast_attention:
+        # With the batch described, prompt portions take the tiled kernel and single tokens the split one.
+        out_c = torch.full_like(out_a, float("nan"))
+        ops.paged_attention(qkv, out_c, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window,
+                            scale, max_position=int(positions.max()), batch=make_batch([1, 300, 64, 17], [1, 5, 64, 1]))
+        torch.testing.assert_close(out_c.float(), out_b.float(), **attention_tol(dtype, True))
+
+
+@pytest.mark.parametrize("geometry", [(14, 2, 64, 16), (12, 2, 128, 16), (3, 1, 32, 32), (5, 5, 16, 16)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, window):
+    # Portions that start in the middle of a page, end in the middle of a tile, and a long whole prompt.
+    n_q, n_kv, d, page_size = geometry
+    lengths, q_lens = [700, 333, 40, 16, 1000], [700, 50, 33, 16, 2]
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=17)
+    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+    out_b = torch.empty_like(out_a)
+    scale = 1.0 / math.sqrt(d)
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
+    torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
 
 
 @pytest.mark.parametrize("window", [None, 1000])

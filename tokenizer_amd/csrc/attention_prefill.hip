@@ -1,0 +1,231 @@
+// Causal (optionally windowed) attention of prompt portions over paged bfloat16 keys and values on the
+// matrix cores.  One wave owns a tile of 16 consecutive tokens of one request, one kv head and a block of
+// HG of the query heads that share it.  As in the decode kernel both products are computed transposed
+// (S^T = K Q^T, O^T = V^T P^T) with 16x16x32 MFMAs: the token index sits in `lane % 16` for scores and
+// outputs, keys and values are read 16 bytes per lane straight from the pages, each key tile once for all
+// HG heads.  Softmax runs online in float; probabilities are rounded to bfloat16 for the second product.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 pf_zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+// One step of the online softmax over 64 keys (four 16-key tiles, each inside one page) for the HG heads of
+// the wave.  FULL: every key of the block is visible to every token of the tile, so nothing is masked.
+// Scores stay unscaled; `c` = scale * log2(e) enters in exp2(s*c - m*c).
+template <int D, int HG, bool FULL>
+__device__ __forceinline__ void prefill_block(
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages, const int* __restrict__ table,
+    int kb, int kvh, int n_kv, int page_size, int col, int g, int heads_here, int my_pos, int my_lo, int lo, int hi,
+    float c, const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16], float (&m)[HG], float (&l)[HG]) {
+  constexpr int KS = (D + 31) / 32;
+  constexpr int DB = D / 16;
+  bf16x8 kf[4][KS];
+  union VFrag { uint2 half[2]; bf16x8 v; } vf[2][DB];
+  bool active[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int k0 = kb + t * 16;
+    active[t] = FULL || ((k0 <= hi) && (k0 + 15 >= lo));
+    if (active[t]) {
+      const int page = table[k0 / page_size];
+      const size_t base = ((size_t)page * n_kv + kvh) * page_size * D;
+      const bf16_t* kr = k_pages + base + (size_t)((k0 % page_size) + col) * D + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks * 32 + 8 * g < D) kf[t][ks] = *reinterpret_cast<const bf16x8*>(kr + ks * 32);
+        else kf[t][ks] = pf_zero8();
+      }
+      const bf16_t* vr = vt_pages + base + (size_t)col * page_size + (k0 % page_size) + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        uint2 v = *reinterpret_cast<const uint2*>(vr + (size_t)db * 16 * page_size);
+        if (!FULL) {                                   // slots past the last key may never have been written
+          const int left = hi - (k0 + 4 * g);          // keys of this lane that exist: 0..left
+          if (left < 3) {
+            if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
+            if (left < 2) v.y = 0; else v.y &= 0xffffu;
+          }
+        }
+        vf[t >> 1][db].half[t & 1] = v;
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kf[t][ks] = pf_zero8();
+#pragma unroll
+      for (int db = 0; db < DB; ++db) vf[t >> 1][db].half[t & 1] = make_uint2(0, 0);
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < HG; ++h) {
+    if (h >= heads_here) break;
+    float s[16];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][ks], qf[h][ks], st, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (FULL) {
+          s[t * 4 + r] = st[r];
+        } else {
+          const int key = kb + t * 16 + 4 * g + r;
+          s[t * 4 + r] = (active[t] && key <= my_pos && key >= my_lo) ? st[r] : -INFINITY;
+        }
+      }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(s[8], s[9]), fmaxf(s[10], s[11])), fmaxf(fmaxf(s[12], s[13]), fmaxf(s[14], s[15]))));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m[h], mx);
+    // A token that has seen no key yet keeps m = -inf; exp2 of (-inf) - (-inf) would be NaN.
+    const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
+    if (__any(m_new > m[h])) {                          // rescale only when some token's maximum moved
+      const float corr = __builtin_amdgcn_exp2f(m[h] * c - mc);   // m = -inf gives 0
+      l[h] *= corr;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[h][db][r] *= corr;
+      m[h] = m_new;
+    }
+    bf16x8 pf[2];
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[i], c, -mc));   // masked keys: exp2(-inf) = 0
+      psum += p;
+      pf[i >> 3][i & 7] = (__bf16)p;
+    }
+    l[h] += psum;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      acc[h][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[0][db].v, pf[0], acc[h][db], 0, 0, 0);
+      acc[h][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[1][db].v, pf[1], acc[h][db], 0, 0, 0);
+    }
+  }
+}
+
+// tiles: [n_tiles, 2] = (entry, offset of the tile's first token inside the entry's tokens).
+// cu_q[e]: first row of entry e; first_position[e]: position of that row.
+// K pages [n_pages, n_kv, page_size, D]; V^T pages [n_pages, n_kv, D, page_size]; page_size % 16 == 0.
+template <int D, int HG>
+__global__ void __launch_bounds__(WAVE)
+prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
+                         const int* __restrict__ tiles, const int* __restrict__ cu_q,
+                         const int* __restrict__ first_position, const int* __restrict__ block_table,
+                         int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
+  constexpr int KS = (D + 31) / 32;
+  constexpr int DB = D / 16;
+  const int lane = threadIdx.x;
+  const int col = lane & 15, g = lane >> 4;
+  const int group = n_q / n_kv;
+  const int head_blocks = (group + HG - 1) / HG;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int heads_here = min(HG, group - hb * HG);
+  const int head0 = kvh * group + hb * HG;
+  const int tile_index = gridDim.x - 1 - blockIdx.x;      // late tiles see the most keys: start them first
+  const int entry = tiles[2 * tile_index], offset = tiles[2 * tile_index + 1];
+  const int row0 = cu_q[entry] + offset;
+  const int n_valid = min(16, cu_q[entry + 1] - row0);
+  const int p0 = first_position[entry] + offset;          // position of the tile's first token
+  const int my_pos = p0 + min(col, n_valid - 1);          // padded columns repeat the last token
+  const int my_row = row0 + min(col, n_valid - 1);
+  const int hi = p0 + n_valid - 1;                         // last key any token of the tile sees
+  const int lo = (window >= 0 && p0 > window) ? p0 - window : 0;      // first key any token sees
+  const int lo_all = (window >= 0 && hi > window) ? hi - window : 0;  // first key every token sees
+  const int my_lo = (window >= 0 && my_pos > window) ? my_pos - window : 0;
+  const int* table = block_table + (size_t)entry * table_stride;
+
+  bf16x8 qf[HG][KS];
+#pragma unroll
+  for (int h = 0; h < HG; ++h)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + 8 * g;
+      qf[h][ks] = pf_zero8();
+      if (h < heads_here && d0 < D)
+        qf[h][ks] = *reinterpret_cast<const bf16x8*>(q + (size_t)my_row * q_stride + (size_t)(head0 + h) * D + d0);
+    }
+  floatx4 acc[HG][DB];
+  float m[HG], l[HG];
+#pragma unroll
+  for (int h = 0; h < HG; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[h][db] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int kb = (lo / 64) * 64; kb <= hi; kb += 64) {
+    if (kb >= lo_all && kb + 63 <= p0)
+      prefill_block<D, HG, true>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                 my_lo, lo, hi, scale_log2, qf, acc, m, l);
+    else
+      prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                  my_lo, lo, hi, scale_log2, qf, acc, m, l);
+  }
+#pragma unroll
+  for (int h = 0; h < HG; ++h) {
+    if (h >= heads_here) break;
+    float total = l[h];
+    total += __shfl_xor(total, 16, WAVE);
+    total += __shfl_xor(total, 32, WAVE);
+    if (col >= n_valid) continue;
+    const float inv = 1.0f / total;
+    bf16_t* dst = out + (size_t)my_row * n_q * D + (size_t)(head0 + h) * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      union { bf16x4 v; uint2 bits; } packed;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) packed.v[r] = (__bf16)(acc[h][db][r] * inv);
+      *reinterpret_cast<uint2*>(dst + db * 16 + 4 * g) = packed.bits;
+    }
+  }
+}
+
+template <int D, int HG>
+static int launch_prefill(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
+                          const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
+                          const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
+                          float scale, hipStream_t stream) {
+  const int group = n_q / n_kv;
+  dim3 grid(n_tiles, n_kv * ((group + HG - 1) / HG));
+  prefill_attention_kernel<D, HG><<<grid, WAVE, 0, stream>>>(
+      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
+      (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
+      window, scale * 1.4426950408889634f);
+  return LAUNCH_STATUS();
+}
+
+// Returns -2 for a head size without an instance (the caller then uses another kernel).
+extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
+                                         const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
+                                         const void* first_position, const void* block_table, int table_stride,
+                                         int n_q, int n_kv, int d, int page_size, int window, float scale,
+                                         int heads_per_wave, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
+  if (d == 64 && heads_per_wave == 1)
+    return launch_prefill<64, 1>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position,
+                                 block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
+#define CASE(DD, HG) case DD: return launch_prefill<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
+    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
+  switch (d) {
+    CASE(16, 4) CASE(32, 4) CASE(48, 2) CASE(64, 2) CASE(80, 2) CASE(96, 2) CASE(112, 2) CASE(128, 2)
+    CASE(160, 1) CASE(192, 1) CASE(224, 1) CASE(256, 1)
+    default: return -2;
+  }
+#undef CASE
+}

@@ -63,6 +63,42 @@ def random_model(config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:
     return Model(config, tensors, dtype, device, ops)
 
 
+class DecodeGraph:
+    """One captured HIP graph of a decode step: `n_entries` requests with one token each, contexts of up
+    to `bucket` tokens.  The batch's tables live in fixed buffers that are refilled before every replay;
+    the graph ends with the greedy pick, so ids are ready without a further launch."""
+
+    def __init__(self, engine: "Engine", entries: list[StepEntry], bucket: int):
+        self.bucket = bucket
+        self.width = bucket // engine.cache.page_size
+        device = engine.model.device
+        probe = build_context(entries, engine.cache, device, table_width=self.width)
+        size = sum(t.numel() for t in (probe.token_ids, probe.positions, probe.entry_of_token, probe.cu_q,
+                                       probe.first_position, probe.state_slots, probe.want_rows, probe.q_tiles,
+                                       probe.decode_rows))
+        size += sum(t.numel() for t in probe.slots) + sum(t.numel() for t in probe.block_tables)
+        self.host = torch.empty(size, dtype=torch.int32).pin_memory()
+        self.dev = torch.empty(size, dtype=torch.int32, device=device)
+        self.ctx = build_context(entries, engine.cache, device, table_width=self.width, into=(self.host, self.dev))
+        self.ctx.max_position = bucket - 1          # what the kernels' launch sizes are planned for
+        ops = engine.model.runtime.ops
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side):               # one eager run first, so that nothing is set up under capture
+            engine.model.decoder.forward(self.ctx, engine.layer_caches)
+        torch.cuda.current_stream(device).wait_stream(side)
+        torch.cuda.synchronize(device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=engine.graph_pool):
+            self.logits = engine.model.decoder.forward(self.ctx, engine.layer_caches)
+            self.ids = ops.argmax(self.logits)
+
+    def run(self, engine: "Engine", entries: list[StepEntry]) -> torch.Tensor:
+        build_context(entries, engine.cache, engine.model.device, table_width=self.width, into=(self.host, self.dev))
+        self.graph.replay()
+        return self.logits
+
+
 class Engine:
     """Owns the cache of one model and runs steps.
 
@@ -71,8 +107,10 @@ class Engine:
     entries and of each entry's `want`.
     """
 
+    GRAPH_BUCKET = 512      # decode graphs are captured per batch size and per this many tokens of context
+
     def __init__(self, model: Model, num_pages: int | None = None, page_size: int = 16, max_requests: int = 8,
-                 max_tokens: int | None = None, prefix_cache: bool = False):
+                 max_tokens: int | None = None, prefix_cache: bool = False, use_graphs: bool | None = None):
         if num_pages is None:
             if max_tokens is None:
                 raise ValueError("give num_pages or max_tokens")
@@ -88,6 +126,13 @@ class Engine:
                                                 v_pages=v_pages, state=self.pools.states.get(source),
                                                 writes=entry.cache_of is None))
         self.steps = 0
+        # Decode steps (one token per request, its logits wanted) replay a captured graph; the logits of a
+        # step stay valid until the next step.
+        self.use_graphs = (model.device.type == "cuda") if use_graphs is None else use_graphs
+        self.use_graphs = self.use_graphs and model.decoder.graph_safe
+        self.graphs: dict[tuple, DecodeGraph] = {}
+        self.graph_pool = torch.cuda.graph_pool_handle() if self.use_graphs else None
+        self._graph_result: DecodeGraph | None = None
 
     @property
     def max_positions(self) -> int:
@@ -96,11 +141,28 @@ class Engine:
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor, rows: list[int] | None = None) -> list[int]:
         """Greedy ids of the given rows of a step's logits, picked on the device."""
-        picked = self.model.runtime.ops.argmax(logits).cpu().tolist()
+        graph = self._graph_result
+        if graph is not None and logits is graph.logits:
+            picked = graph.ids.cpu().tolist()           # the graph already picked them
+        else:
+            picked = self.model.runtime.ops.argmax(logits).cpu().tolist()
         return picked if rows is None else [picked[row] for row in rows]
 
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):
         return logits[rows].float().cpu().numpy()
+
+    def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
+        longest = max(self.cache.seq_len(e.rid) for e in entries) + 1
+        bucket = -(-longest // self.GRAPH_BUCKET) * self.GRAPH_BUCKET
+        bucket = -(-bucket // self.cache.page_size) * self.cache.page_size
+        key = (len(entries), bucket)
+        graph = self.graphs.get(key)
+        if graph is None:
+            graph = DecodeGraph(self, entries, bucket)      # its first eager run and the capture write the same
+            self.graphs[key] = graph                         # keys and values the replay writes again
+        logits = graph.run(self, entries)
+        self._graph_result = graph
+        return logits
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid) -> None:
@@ -146,8 +208,12 @@ class Engine:
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         self.validate(entries)
         self.reserve(entries)
-        ctx = build_context(entries, self.cache, self.model.device)
-        logits = self.model.decoder.forward(ctx, self.layer_caches)
+        self._graph_result = None
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits = self._graph_step(entries)
+        else:
+            ctx = build_context(entries, self.cache, self.model.device)
+            logits = self.model.decoder.forward(ctx, self.layer_caches)
         for entry in entries:
             self.cache.advance(entry.rid, self.cache.seq_len(entry.rid) + len(entry.tokens))
         self.steps += 1

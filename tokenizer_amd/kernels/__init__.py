@@ -52,7 +52,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16",
                      "ta_argmax"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -158,13 +158,16 @@ class Ops:
     def paged_attention(self, qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor,
                         v_pages: torch.Tensor, positions: torch.Tensor, entry_of_token: torch.Tensor,
                         block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
-                        window: int | None, scale: float, max_position: int | None = None) -> torch.Tensor:
+                        window: int | None, scale: float, max_position: int | None = None,
+                        batch=None) -> torch.Tensor:
         """Causal attention of every token over the pages of its request.
 
         qkv [T, >= n_q d] (query heads first); out [T, n_q d]; key pages [n_pages, n_kv, page_size, d],
         value pages [n_pages, n_kv, d, page_size];
         positions, entry_of_token int32 [T]; block_table int32 [E, P]; a token at position p sees keys
         max(0, p - window)..p.  `max_position` (host) lets the wrapper check that the table is wide enough.
+        `batch` (a StepContext of the same tokens) lets bfloat16 batches run the tiled kernel on prompt
+        portions and the split kernel on single tokens; without it every token goes through the latter.
         """
         _dev(qkv, out, k_pages, v_pages, positions, entry_of_token, block_table)
         n_tokens = qkv.shape[0]
@@ -181,8 +184,20 @@ class Ops:
             _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
         if (qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
                 and qkv.shape[1] % 8 == 0 and self.use_fast_attention):
-            return self._decode_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
-                                          n_q, n_kv, head_dim, page_size, window, scale, max_position)
+            args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
+                    page_size, window, scale, max_position)
+            if batch is None or batch.q_tiles.numel() == 0:
+                return self._decode_attention(*args)
+            _need(batch.n_tokens == n_tokens and batch.cu_q.numel() == block_table.shape[0] + 1,
+                  "the batch description does not belong to these tokens")
+            self._check(self.lib.ta_prefill_attention_bf16(
+                _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(batch.q_tiles),
+                batch.q_tiles.shape[0], _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
+                block_table.shape[1], n_q, n_kv, head_dim, page_size, -1 if window is None else int(window),
+                ctypes.c_float(scale), self.prefill_heads_per_wave, self._stream()), "prefill_attention")
+            if batch.decode_rows.numel():
+                self._decode_attention(*args, rows=batch.decode_rows)
+            return out
         self._check(self.lib.ta_paged_attention_generic(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(positions),
             _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], n_tokens, n_q, n_kv, head_dim,
@@ -192,6 +207,7 @@ class Ops:
 
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
     use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
+    prefill_heads_per_wave = 0    # 0: the kernel's own choice for the head size
     target_workgroups = 1024      # what the split of the key range aims at
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
@@ -247,6 +263,13 @@ class Ops:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+            if (self.use_library_gemm and bias is None and out_dtype == torch.bfloat16 and m > self.SKINNY_ROWS
+                    and ((k >= 2048 and m >= 128) or m * n * k >= 2 ** 32)):
+                # Large plain products go to the vendor's library (hipBLASLt through torch), as the
+                # reference's engine uses a library for its matrix products; it is faster there than
+                # the tiled kernel of this package.
+                torch.matmul(x, weight.t(), out=out)
+                return out
             if m <= self.SKINNY_ROWS:
                 status = self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, m, n, k,
                                                       _code(out_dtype), 0, self._stream())
@@ -257,6 +280,7 @@ class Ops:
         return out
 
     SKINNY_ROWS = 64    # up to this many rows the weight-streaming kernel runs
+    use_library_gemm = True
 
     def linear_silu_gate(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """out = silu(x @ Wg.T) * (x @ Wu.T) for weight = [Wg; Wu] of shape [2I, K]; out [M, I].

@@ -20,6 +20,8 @@ class GQAttention(Mixer):
     key <= query and, with a window w, key + w >= query (model.rs:119-129).
     The three projection matrices are joined into one at load time so one product makes q, k and v.
     """
+    graph_safe = True
+
 
     def __init__(self, spec: MixerSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.spec, self.runtime = spec, runtime
@@ -36,6 +38,7 @@ class GQAttention(Mixer):
         self.window = spec.window
         position = spec.position or PositionSpec("none")
         self.position = POSITIONS.get(position.kind)(position, runtime)
+        self.graph_safe = bool(getattr(self.position, "graph_safe", False))
 
     @staticmethod
     def tensor_specs(spec: MixerSpec) -> dict[str, TensorSpec]:
@@ -62,5 +65,5 @@ class GQAttention(Mixer):
         mixed = torch.empty((x.shape[0], self.n_q * self.d), dtype=x.dtype, device=x.device)
         ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
                             ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
-                            self.scale, max_position=ctx.max_position)
+                            self.scale, max_position=ctx.max_position, batch=ctx)
         return ops.linear(mixed, self.w_o, self.b_o)

@@ -66,7 +66,13 @@ BLOCKS = Registry("block")
 
 
 class Part:
-    """Common base: a part names its tensors and is built from them."""
+    """Common base: a part names its tensors and is built from them.
+
+    `graph_safe` says that the part's forward only launches device work whose shape depends on the
+    batch's sizes, never on host-side values of the batch (positions, request ids): only then may a
+    decode step be captured once and replayed.  Parts are taken not to be unless they say so.
+    """
+    graph_safe = False
 
     @staticmethod
     def tensor_specs(spec) -> dict[str, TensorSpec]:
@@ -99,5 +105,7 @@ class FeedForward(Part):
 
 
 class Block:
+    graph_safe = False
+
     def forward(self, residual: torch.Tensor, delta: torch.Tensor | None, ctx, cache) -> torch.Tensor:
         raise NotImplementedError

@@ -11,6 +11,8 @@ class PreNormBlock(Block):
     The residual stream is float32.  Each sub-layer's output is handed on as a pending `delta`
     so that the add fuses into the next norm.
     """
+    graph_safe = True
+
 
     def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
         self.mixer_norm, self.mixer = mixer_norm, mixer

@@ -14,6 +14,8 @@ class GatedDense(FeedForward):
     gate and up are joined into one matrix at load time; the activation and the product with
     `up` run in float32 in one kernel.
     """
+    graph_safe = True
+
 
     def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         if spec.activation != "silu":

@@ -67,6 +67,10 @@ class DecoderModel:
             self.blocks.append(BLOCKS.get(layer.block)(mixer_norm, mixer, ff_norm, feed_forward))
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)
         self.head = self.embedding if spec.tied_head else tensors[spec.head_name]
+        parts = [self.final_norm] + [p for b in self.blocks for p in (b, b.mixer_norm, b.mixer, b.feed_forward_norm,
+                                                                      b.feed_forward) if hasattr(b, "mixer")]
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts) and \
+            all(hasattr(b, "mixer") for b in self.blocks)
 
     def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
         """Run the tokens of `ctx` through the schedule; float32 logits [len(want_rows), vocab]."""

@@ -10,6 +10,8 @@ from .spec import NormSpec, TensorSpec
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     """y = x / sqrt(mean(x^2) + eps) * weight (qwen-infer/src/model.rs:594-599), in float32."""
+    graph_safe = True
+
 
     def __init__(self, spec: NormSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.size, self.eps = spec.size, float(spec.eps)

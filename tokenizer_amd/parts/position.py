@@ -10,6 +10,8 @@ from .spec import PositionSpec
 @POSITIONS.register("none")
 class NoPosition(PositionEncoding):
     """No encoding: the projection bias is added and keys and values are stored as they are."""
+    graph_safe = True
+
 
     def __init__(self, spec: PositionSpec, runtime: Runtime):
         self.runtime = runtime
