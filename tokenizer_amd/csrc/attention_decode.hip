@@ -174,25 +174,33 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   }
 }
 
-// out[t, head, :] = sum_s part_o[s] * exp(m_s - M) / sum_s l_s * exp(m_s - M).  One block per (item, head).
-__global__ void decode_attention_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                       const int* __restrict__ rows, bf16_t* __restrict__ out,
-                                       int n_q, int d, int splits) {
+// out[t, head, :] = sum_s part_o[s] * exp(m_s - M) / sum_s l_s * exp(m_s - M).  One wave per (item, head):
+// the lanes first share out the splits (maximum and denominator), then the elements of the head.
+// A separate kernel on purpose: a last-arrival merge inside the first kernel needs device-wide fences,
+// which flush the L2 of every XCD and cost more than this launch.
+__global__ void __launch_bounds__(WAVE)
+decode_attention_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                       const int* __restrict__ rows, bf16_t* __restrict__ out, int n_q, int d, int splits) {
   const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
   const int t = rows ? rows[item] : item;
   const size_t base = ((size_t)item * n_q + head) * splits;
+  const int lane = threadIdx.x;
   float big = -INFINITY;
-  for (int s = 0; s < splits; ++s) big = fmaxf(big, part_ml[(base + s) * 2]);
+  for (int s = lane; s < splits; s += WAVE) big = fmaxf(big, part_ml[(base + s) * 2]);
+  big = wave_max(big);
   float denom = 0.f;
-  for (int s = 0; s < splits; ++s) {
+  for (int s = lane; s < splits; s += WAVE) {
     const float ms = part_ml[(base + s) * 2];
     if (ms != -INFINITY) denom += part_ml[(base + s) * 2 + 1] * __expf(ms - big);
   }
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  denom = wave_sum(denom);
+  for (int i = lane; i < d; i += WAVE) {
     float o = 0.f;
+#pragma unroll 4
     for (int s = 0; s < splits; ++s) {
-      const float ms = part_ml[(base + s) * 2];
-      if (ms != -INFINITY) o += part_o[(base + s) * d + i] * __expf(ms - big);
+      const float ms = part_ml[(base + s) * 2];                 // the same address for every lane: one load
+      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - big);
+      o += part_o[(base + s) * d + i] * w;
     }
     st(out + (size_t)t * n_q * d + (size_t)head * d + i, o / denom);
   }

@@ -311,8 +311,12 @@ class Ops:
         if out is None:
             out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
         _need(out.dtype == torch.int32 and out.numel() == logits.shape[0], "argmax output must be int32 [B]")
-        self._check(self.lib.ta_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
-                                       self._stream()), "argmax")
+        n_rows, vocab = logits.shape
+        chunks = max(1, min(256, vocab // 2048, 2048 // max(1, n_rows)))
+        partial_v = torch.empty((n_rows, chunks), dtype=torch.float32, device=logits.device)
+        partial_i = torch.empty((n_rows, chunks), dtype=torch.int32, device=logits.device)
+        self._check(self.lib.ta_argmax(_ptr(logits), _ptr(out), _ptr(partial_v), _ptr(partial_i), n_rows, vocab,
+                                       chunks, self._stream()), "argmax")
         return out
 
 
