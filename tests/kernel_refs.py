@@ -104,6 +104,43 @@ class PlainOps:
         result = torch.empty((x.shape[0], inner), dtype=x.dtype, device=x.device) if out is None else out
         return self.silu_gate(self.linear(x, weight), result)
 
+    # The fused decode products, as compositions of the ops above.
+    fuse_rows = 16
+
+    def can_fuse_decode(self, rows, dtype):
+        return 0 < rows <= self.fuse_rows
+
+    def fused_norm_qkv_rope(self, residual, norm_weight, eps, weight, bias, positions, cos_sin, slots,
+                            k_pages, v_pages, n_q, n_kv, head_dim):
+        x = torch.empty(residual.shape, dtype=weight.dtype, device=residual.device)
+        self.add_rmsnorm(residual.clone(), None, norm_weight, eps, x)
+        qkv = (x.to(self.work) @ weight.to(self.work).t())
+        if bias is not None:
+            qkv = qkv + bias.to(self.work)
+        # The fused kernel rotates the float accumulators and rounds once.
+        holder = qkv.to(self.work).clone()
+        work_k = None if slots is None else k_pages.to(self.work)
+        work_v = None if slots is None else v_pages.to(self.work)
+        PlainOps(self.work).rope_store(holder, None, positions, cos_sin, slots, work_k, work_v, n_q, n_kv, head_dim)
+        if slots is not None:
+            k_pages.copy_(work_k.to(k_pages.dtype))
+            v_pages.copy_(work_v.to(v_pages.dtype))
+        return holder[:, :n_q * head_dim].to(weight.dtype).contiguous()
+
+    def fused_norm_gated(self, residual, norm_weight, eps, weight):
+        x = torch.empty(residual.shape, dtype=weight.dtype, device=residual.device)
+        self.add_rmsnorm(residual.clone(), None, norm_weight, eps, x)
+        gate_up = x.to(self.work) @ weight.to(self.work).t()
+        inner = weight.shape[0] // 2
+        g, u = gate_up[:, :inner], gate_up[:, inner:]
+        return (g * torch.sigmoid(g) * u).to(weight.dtype)
+
+    def linear_add(self, x, weight, bias, residual):
+        y = x.to(self.work) @ weight.to(self.work).t()
+        if bias is not None:
+            y = y + bias.to(self.work)
+        residual.add_(y.to(torch.float32))
+
     def argmax(self, logits, out=None):
         result = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device) if out is None else out
         for row in range(logits.shape[0]):

@@ -329,6 +329,65 @@ def test_skinny_rows_agree_with_the_tiled_kernel(ops, shape):
     torch.testing.assert_close(skinny, tiled, **linear_tol(torch.float32, x, w))
 
 
+@pytest.mark.parametrize("geometry", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 16), (4, 4, 128, 520, 32), (20, 2, 96, 264, 16)])
+@pytest.mark.parametrize("rows", [1, 8, 16])
+def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
+    n_q, n_kv, d, hidden, page_size = geometry
+    n_pages, max_pos = 7, 300
+    gen = torch.Generator().manual_seed(40)
+    residual = rand((rows, hidden), torch.float32, 41, 2.0)
+    norm_w = rand((hidden,), torch.float32, 42) * 0.1 + 1
+    w = rand(((n_q + 2 * n_kv) * d, hidden), torch.bfloat16, 43, 0.05)
+    bias = rand(((n_q + 2 * n_kv) * d,), torch.float32, 44)
+    positions = torch.randint(0, max_pos, (rows,), generator=gen).int().cuda()
+    inv = torch.tensor([1.0 / (1e6 ** (i / d)) for i in range(0, d, 2)], dtype=torch.float64).float()
+    ang = torch.arange(max_pos).float()[:, None] * inv[None]
+    cos_sin = torch.cat([ang.cos(), ang.sin()], 1).cuda()
+    slots = torch.randperm(n_pages * page_size, generator=gen)[:rows].int().cuda()
+    if rows > 2:
+        slots[1] = -1
+    for use_bias, table, store in ((True, cos_sin, True), (False, cos_sin, True), (True, None, True), (True, cos_sin, False)):
+        ka = torch.zeros((n_pages, n_kv, page_size, d), dtype=torch.bfloat16).cuda()
+        va = torch.zeros((n_pages, n_kv, d, page_size), dtype=torch.bfloat16).cuda()
+        kb, vb = ka.clone(), va.clone()
+        args = (residual, norm_w, 1e-6, w, bias if use_bias else None, positions, table, slots if store else None)
+        before = residual.clone()
+        qa = ops.fused_norm_qkv_rope(*args, ka, va, n_q, n_kv, d)
+        qb = ref.fused_norm_qkv_rope(*args, kb, vb, n_q, n_kv, d)
+        assert torch.equal(residual, before)
+        # The norm's output is rounded to bfloat16 in both; what differs is the summation order.
+        tolerance = dict(rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(qa.float(), qb.float(), **tolerance)
+        torch.testing.assert_close(ka.float(), kb.float(), **tolerance)
+        torch.testing.assert_close(va.float(), vb.float(), **tolerance)
+        if not store:
+            assert float(ka.abs().max()) == 0 and float(va.abs().max()) == 0
+
+
+@pytest.mark.parametrize("shape", [(1, 4864, 896), (8, 272, 96), (16, 176, 80), (5, 136, 72)])
+def test_fused_norm_gated_and_linear_add(ops, ref, shape):
+    rows, inner, hidden = shape
+    residual = rand((rows, hidden), torch.float32, 50, 2.0)
+    norm_w = rand((hidden,), torch.float32, 51) * 0.1 + 1
+    w = rand((2 * inner, hidden), torch.bfloat16, 52, 0.1)
+    got = ops.fused_norm_gated(residual, norm_w, 1e-5, w)
+    want = ref.fused_norm_gated(residual, norm_w, 1e-5, w)
+    torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    # residual += act @ down.T + bias
+    down = rand((hidden, inner), torch.bfloat16, 53, 0.05)
+    bias = rand((hidden,), torch.float32, 54)
+    for use_bias in (True, False):
+        res_a, res_b = residual.clone(), residual.clone()
+        ops.linear_add(got, down, bias if use_bias else None, res_a)
+        ref.linear_add(got, down, bias if use_bias else None, res_b)
+        torch.testing.assert_close(res_a, res_b, **linear_tol(torch.float32, got, down))
+    wide = rand((rows, inner + 8), torch.bfloat16, 55)
+    res_a, res_b = residual.clone(), residual.clone()
+    ops.linear_add(wide[:, :inner], down, None, res_a)
+    ref.linear_add(wide[:, :inner], down, None, res_b)
+    torch.testing.assert_close(res_a, res_b, **linear_tol(torch.float32, wide[:, :inner], down))
+
+
 def test_linear_float32_is_true_float32(ops):
     # Inputs that need 13 mantissa bits: a reduced-precision matrix mode (10 or 7 bits) would be off by
     # about 1e-2 here, float32 accumulation by less than 3e-4.

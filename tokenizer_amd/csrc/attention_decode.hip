@@ -70,35 +70,52 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   float m = -INFINITY, l = 0.f;
 
   for (int kb = first + wave * 32; kb <= last; kb += DEC_WAVES * 32) {
-    float s[2][4];
-    size_t page_base[2];
+    // All loads of the block are issued first: keys, and values (whose addresses do not wait for the scores).
+    bf16x8 kf[2][KS];
+    union VFrag { uint2 half[2]; bf16x8 v; } vf[DB];
     bool active[2];
-    uint64_t keep[2];   // 16 bits of ones for every visible key of the lane's four: slots nobody wrote may hold anything
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile) {
       const int k0 = kb + tile * 16;                       // 16 keys of one page
       active[tile] = (k0 <= last) && (k0 + 15 >= lo);
-      page_base[tile] = 0;
-      floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
       if (active[tile]) {
         const int page = table[k0 / page_size];
-        page_base[tile] = ((size_t)page * n_kv + kvh) * page_size * D;   // same element count for K and V^T pages
-        const bf16_t* kr = k_pages + page_base[tile] + (size_t)((k0 % page_size) + col) * D;
+        const size_t base = ((size_t)page * n_kv + kvh) * page_size * D;   // same element count for K and V^T pages
+        const bf16_t* kr = k_pages + base + (size_t)((k0 % page_size) + col) * D + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const int d0 = ks * 32 + 8 * g;
-          bf16x8 kf = zero8();
-          if (d0 < D) kf = *reinterpret_cast<const bf16x8*>(kr + d0);
-          st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], st, 0, 0, 0);
+          if (ks * 32 + 8 * g < D) kf[tile][ks] = *reinterpret_cast<const bf16x8*>(kr + ks * 32);
+          else kf[tile][ks] = zero8();
         }
+        const bf16_t* vr = vt_pages + base + (size_t)col * page_size + (k0 % page_size) + 4 * g;
+        const int left = last - (k0 + 4 * g);              // keys of this lane that exist: 0..left
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          uint2 v = *reinterpret_cast<const uint2*>(vr + (size_t)db * 16 * page_size);
+          if (left < 3) {                                  // slots nobody wrote may hold anything: 0 * NaN would poison the sum
+            if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
+            if (left < 2) v.y = 0; else v.y &= 0xffffu;
+          }
+          vf[db].half[tile] = v;
+        }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kf[tile][ks] = zero8();
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vf[db].half[tile] = make_uint2(0, 0);
       }
-      keep[tile] = 0;
+    }
+    float s[2][4];
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+      floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tile][ks], qf[ks], st, 0, 0, 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int key = k0 + 4 * g + r;
-        const bool seen = active[tile] && key >= lo && key <= last;
-        s[tile][r] = seen ? st[r] * scale : -INFINITY;
-        if (seen) keep[tile] |= (uint64_t)0xffff << (16 * r);
+        const int key = kb + tile * 16 + 4 * g + r;
+        s[tile][r] = (active[tile] && key >= lo && key <= last) ? st[r] * scale : -INFINITY;
       }
     }
     float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
@@ -122,22 +139,9 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     m = m_new;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      // V^T fragment: row d = db*16 + col, slots 0..3 = keys 4g..4g+3 of tile 0, slots 4..7 of tile 1.
-      bf16x8 vf = zero8();
-#pragma unroll
-      for (int tile = 0; tile < 2; ++tile) {
-        if (active[tile]) {
-          const int k0 = kb + tile * 16;
-          const bf16_t* vr = vt_pages + page_base[tile] + (size_t)(db * 16 + col) * page_size + (k0 % page_size) + 4 * g;
-          union { uint64_t bits; bf16x4 v; } v4;
-          v4.bits = *reinterpret_cast<const uint64_t*>(vr) & keep[tile];   // 0 * NaN would poison the sum
-#pragma unroll
-          for (int r = 0; r < 4; ++r) vf[tile * 4 + r] = v4.v[r];
-        }
-      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[db][r] *= corr;
-      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[db], 0, 0, 0);
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db].v, pf, acc[db], 0, 0, 0);
     }
   }
   // Sum of the lane groups' partial denominators (the maximum is already common to them).

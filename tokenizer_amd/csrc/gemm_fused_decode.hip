@@ -1,0 +1,337 @@
+// Fused products for decode batches of up to 16 rows.  Each keeps the layout of the weight-streaming kernel
+// (C^T = W A^T on 16x16x32 MFMAs, the waves of a workgroup split K and add up through LDS) and folds the
+// neighbouring small kernels into its prologue or epilogue:
+//   NORM prologue   the rows are read from the float residual stream and RMS-normalised on the fly
+//   ROPE_STORE      q/k/v projection: bias, half-split rotation, keys and values written into their pages
+//   GATED           silu(gate) * up
+//   RESIDUAL        the product is added into the float residual stream in place
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+enum { EPI_ROPE_STORE = 0, EPI_GATED = 1, EPI_RESIDUAL = 2 };
+
+struct FusedArgs {
+  // input rows: bfloat16 activations, or (with the NORM prologue) the float residual with norm weight and eps
+  const bf16_t* a; int lda;
+  const float* residual_in; const float* norm_weight; float eps;
+  const bf16_t* w; const float* bias;
+  int m, n, k;
+  // EPI_GATED / plain output (bfloat16 [m, ldc])
+  bf16_t* out; int ldc;
+  // EPI_RESIDUAL
+  float* residual_out;
+  // EPI_ROPE_STORE
+  const int* positions; const float* cos_sin; const int* slots;
+  bf16_t* k_pages; bf16_t* v_pages; int n_q, n_kv, d, page_size;
+};
+
+__device__ __forceinline__ bf16x8 fz8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+template <int NW, int EPI, bool NORM>
+__global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs p) {
+  constexpr int SETS = (EPI == EPI_RESIDUAL) ? 1 : 2;
+  __shared__ float red[NW][SETS * 4][WAVE];
+  extern __shared__ __attribute__((aligned(16))) uint16_t a_s[];   // NORM: 16 normalised rows of K + 8 bfloat16
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, g = lane >> 4;
+  const int M = p.m, K = p.k;
+  const int tile = blockIdx.x;
+
+  // Which weight rows this workgroup owns: `row0` (+ `row1` for the second set).
+  int row0, row1 = 0;
+  bool paired = true;
+  int n_pair_tiles = 0;
+  if (EPI == EPI_ROPE_STORE) {
+    const int half = p.d / 2, per_half = half / 16;
+    n_pair_tiles = (p.n_q + p.n_kv) * per_half;
+    if (tile < n_pair_tiles) {
+      const int hd = tile / per_half, j = tile % per_half;
+      row0 = hd * p.d + j * 16;
+      row1 = row0 + half;
+    } else {
+      paired = false;
+      row0 = (p.n_q + p.n_kv) * p.d + (tile - n_pair_tiles) * 16;
+      row1 = row0;
+    }
+  } else if (EPI == EPI_GATED) {
+    row0 = tile * 16;
+    row1 = row0 + p.n / 2;
+  } else {
+    row0 = tile * 16;
+  }
+  const int n_limit = (EPI == EPI_GATED) ? p.n / 2 : p.n;
+  // Rows past the end are clamped: they only feed outputs that are never stored.
+  const bf16_t* w0 = p.w + (size_t)min(row0 + col, n_limit - 1) * K + 8 * g;
+  const bf16_t* w1 = p.w + (size_t)min(row1 + col, p.n - 1) * K + 8 * g;
+  const int a_m = min(col, M - 1);
+  const int full_steps = K / 32;
+  constexpr int UN = 4;
+  const int lds_stride = K + 8;
+
+  // Weight fragments come from HBM and take longest; the first batch is requested before the prologue.
+  // Step j of a wave's batch: steps come in pairs (128 contiguous bytes of a weight row, one cache line),
+  // pair q of the batch starting at pair `base` is pair base + q * NW.
+  auto step_of = [&](int base_pair, int u) { return (base_pair + (u >> 1) * NW) * 2 + (u & 1); };
+  bf16x8 wf[UN][SETS];
+  auto load_w = [&](int base_pair) {
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int step = min(step_of(base_pair, u), max(full_steps - 1, 0));   // clamped loads are not used
+      wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + step * 32);
+      if (SETS == 2) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + step * 32);
+    }
+  };
+  load_w(wave);
+
+  // What the epilogue needs besides the sums is requested now as well (wave 0 writes the results;
+  // lane (col, g) owns column m = col and rows 4g .. 4g+3 of the tile).
+  float pre_a[4] = {0.f, 0.f, 0.f, 0.f}, pre_b[4] = {0.f, 0.f, 0.f, 0.f};   // bias, or the old residual
+  float pre_cos[4] = {1.f, 1.f, 1.f, 1.f}, pre_sin[4] = {0.f, 0.f, 0.f, 0.f};
+  int pre_slot = -1;
+  if (wave == 0 && col < M) {
+    if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = row0 + 4 * g + r;
+        if (n < p.n) pre_a[r] = p.residual_out[(size_t)col * p.n + n] + (p.bias ? p.bias[n] : 0.f);
+      }
+    } else if (EPI == EPI_ROPE_STORE) {
+      pre_slot = p.slots ? p.slots[col] : -1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (p.bias) { pre_a[r] = p.bias[row0 + 4 * g + r]; pre_b[r] = p.bias[row1 + 4 * g + r]; }
+        if (paired && p.cos_sin) {
+          const float* cs = p.cos_sin + (size_t)p.positions[col] * p.d;
+          const int i = row0 % p.d + 4 * g + r;
+          pre_cos[r] = cs[i];
+          pre_sin[r] = cs[p.d / 2 + i];
+        }
+      }
+    }
+  }
+
+  if (NORM) {
+    // Each row once: 1 / sqrt(mean(x^2) + eps), then x * that * weight rounded to bfloat16 into LDS.
+    for (int m = wave; m < M; m += NW) {
+      const float* x = p.residual_in + (size_t)m * K;
+      uint16_t* dst = a_s + (size_t)m * lds_stride;
+      if (K <= 4 * WAVE * 4) {
+        // The row fits in four float4 per lane: read it (and the norm weight) once and keep it in registers.
+        float4 v[4], gw[4];
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int k = (i * WAVE + lane) * 4;
+          v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+          gw[i] = v[i];
+          if (k < K) {
+            v[i] = *reinterpret_cast<const float4*>(x + k);          // K is a multiple of 8
+            gw[i] = *reinterpret_cast<const float4*>(p.norm_weight + k);
+          }
+          sq += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+        }
+        sq = wave_sum(sq);
+        const float inv = 1.0f / sqrtf(sq / (float)K + p.eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int k = (i * WAVE + lane) * 4;
+          if (k >= K) continue;
+          union { bf16x4 v; uint2 bits; } packed;
+          packed.v[0] = (__bf16)(v[i].x * inv * gw[i].x); packed.v[1] = (__bf16)(v[i].y * inv * gw[i].y);
+          packed.v[2] = (__bf16)(v[i].z * inv * gw[i].z); packed.v[3] = (__bf16)(v[i].w * inv * gw[i].w);
+          *reinterpret_cast<uint2*>(dst + k) = packed.bits;
+        }
+        continue;
+      }
+      float sq = 0.f;
+      for (int k = lane * 4; k < K; k += WAVE * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(x + k);
+        sq += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      }
+      sq = wave_sum(sq);
+      const float inv = 1.0f / sqrtf(sq / (float)K + p.eps);
+      for (int k = lane * 4; k < K; k += WAVE * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(x + k);
+        const float4 gw = *reinterpret_cast<const float4*>(p.norm_weight + k);
+        union { bf16x4 v; uint2 bits; } packed;
+        packed.v[0] = (__bf16)(v.x * inv * gw.x); packed.v[1] = (__bf16)(v.y * inv * gw.y);
+        packed.v[2] = (__bf16)(v.z * inv * gw.z); packed.v[3] = (__bf16)(v.w * inv * gw.w);
+        *reinterpret_cast<uint2*>(dst + k) = packed.bits;
+      }
+    }
+    __syncthreads();
+  }
+  const bf16_t* ar = NORM ? nullptr : p.a + (size_t)a_m * p.lda + 8 * g;
+  const uint16_t* as_row = a_s + (size_t)a_m * lds_stride + 8 * g;
+  auto load_a = [&](int k) -> bf16x8 {
+    if (NORM) return *reinterpret_cast<const bf16x8*>(as_row + k);
+    return *reinterpret_cast<const bf16x8*>(ar + k);
+  };
+
+  floatx4 acc[SETS];
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) acc[s] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  // Batches of UN steps; the next batch's weights are requested before the current one is multiplied.
+  for (int pair = wave; pair * 2 < full_steps; pair += (UN / 2) * NW) {
+    bf16x8 wc[UN][SETS], af[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      wc[u][0] = wf[u][0];
+      if (SETS == 2) wc[u][SETS - 1] = wf[u][SETS - 1];
+      af[u] = load_a(min(step_of(pair, u), full_steps - 1) * 32);
+    }
+    if ((pair + (UN / 2) * NW) * 2 < full_steps) load_w(pair + (UN / 2) * NW);
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      if (step_of(pair, u) >= full_steps) continue;
+#pragma unroll
+      for (int s = 0; s < SETS; ++s)
+        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][s], af[u], acc[s], 0, 0, 0);
+    }
+  }
+  if ((K & 31) && wave == 0) {                             // tail of K (a multiple of 8): zero-filled
+    const int k = full_steps * 32;
+    const bool ok = k + 8 * g < K;
+    const bf16x8 af = ok ? load_a(k) : fz8();
+    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w0 + k) : fz8(), af, acc[0], 0, 0, 0);
+    if (SETS == 2)
+      acc[SETS - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w1 + k) : fz8(), af, acc[SETS - 1], 0, 0, 0);
+  }
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][s * 4 + r][lane] = acc[s][r];
+  __syncthreads();
+  if (threadIdx.x >= WAVE) return;
+  // Lane (col, g): output column m = col, rows 4g .. 4g+3 of the tile.
+  const int m = col;
+  if (m >= M) return;
+  float v0[4], v1[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      s0 += red[w][r][lane];
+      if (SETS == 2) s1 += red[w][4 + r][lane];
+    }
+    v0[r] = s0;
+    v1[r] = s1;
+  }
+  if (EPI == EPI_RESIDUAL) {
+    const int n = row0 + 4 * g;
+    float* dst = p.residual_out + (size_t)m * p.n + n;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n + r < p.n) dst[r] = pre_a[r] + v0[r];            // old residual (+ bias) was fetched at the start
+  } else if (EPI == EPI_GATED) {
+    const int n = row0 + 4 * g;
+    bf16_t* dst = p.out + (size_t)m * p.ldc + n;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n + r < n_limit) st(dst + r, v0[r] / (1.0f + __expf(-v0[r])) * v1[r]);
+  } else {
+    const int d = p.d, half = d / 2;
+    const int slot = pre_slot;
+    const int page = slot >= 0 ? slot / p.page_size : 0, off = slot >= 0 ? slot % p.page_size : 0;
+    if (paired) {
+      const int hd = row0 / d, i = row0 % d + 4 * g;            // element i (< half) of head hd, and i + half
+      float r1[4], r2[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float x1 = v0[r] + pre_a[r], x2 = v1[r] + pre_b[r];
+        r1[r] = x1 * pre_cos[r] - x2 * pre_sin[r];              // cos 1, sin 0 without a rotation
+        r2[r] = x2 * pre_cos[r] + x1 * pre_sin[r];
+      }
+      bf16_t* dst = nullptr;
+      if (hd < p.n_q) dst = p.out + (size_t)m * p.ldc + (size_t)hd * d + i;
+      else if (slot >= 0) dst = p.k_pages + (((size_t)page * p.n_kv + (hd - p.n_q)) * p.page_size + off) * d + i;
+      if (dst) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { st(dst + r, r1[r]); st(dst + half + r, r2[r]); }
+      }
+    } else if (slot >= 0) {
+      const int e = row0 - (p.n_q + p.n_kv) * d + 4 * g;        // element of the joined value heads
+      const int kvh = e / d, dd = e % d;
+      bf16_t* dst = p.v_pages + (((size_t)page * p.n_kv + kvh) * d + dd) * p.page_size + off;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) st(dst + (size_t)r * p.page_size, v0[r] + pre_a[r]);
+    }
+  }
+}
+
+template <int NW, int EPI, bool NORM>
+static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
+  size_t lds = NORM ? (size_t)16 * (args.k + 8) * sizeof(uint16_t) : 0;
+  if (lds > 48 * 1024) {
+    // More dynamic LDS than the default limit: ask for it (the device has 160 KB per compute unit).
+    if (lds > 140 * 1024) return -1;
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) return (int)err;
+  }
+  fused_decode_kernel<NW, EPI, NORM><<<tiles, NW * WAVE, lds, stream>>>(args);
+  return LAUNCH_STATUS();
+}
+
+template <int EPI, bool NORM>
+static int launch_fused(const FusedArgs& args, int tiles, hipStream_t stream) {
+  const int k_steps = (args.k + 31) / 32;
+  if (tiles >= 1024 || k_steps <= 8) return launch_one<4, EPI, NORM>(args, tiles, stream);
+  if (tiles >= 256 || k_steps <= 32 || NORM) return launch_one<8, EPI, NORM>(args, tiles, stream);
+  if constexpr (!NORM) return launch_one<16, EPI, false>(args, tiles, stream);
+  return -1;
+}
+
+// q/k/v projection of up to 16 rows read from the float residual (normalised on the fly): bias, rotation,
+// q into `q_out` [m, n_q * d], keys and values into their pages (slots null or negative: not stored).
+extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_weight, float eps, const void* w,
+                                      const void* bias, void* q_out, const void* positions, const void* cos_sin,
+                                      const void* slots, void* k_pages, void* v_pages, int m, int k, int n_q,
+                                      int n_kv, int d, int page_size, hipStream_t stream) {
+  if (m <= 0) return 0;
+  if (m > 16 || (k & 7) || (d & 31)) return -1;
+  FusedArgs a = {};
+  a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
+  a.w = (const bf16_t*)w; a.bias = (const float*)bias; a.m = m; a.n = (n_q + 2 * n_kv) * d; a.k = k;
+  a.out = (bf16_t*)q_out; a.ldc = n_q * d;
+  a.positions = (const int*)positions; a.cos_sin = (const float*)cos_sin; a.slots = (const int*)slots;
+  a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
+  const int tiles = (n_q + n_kv) * (d / 32) + n_kv * d / 16;
+  return launch_fused<EPI_ROPE_STORE, true>(a, tiles, stream);
+}
+
+// out [m, n/2] = silu(x Wg^T) * (x Wu^T), x = the normalised residual rows, W = [Wg; Wu] of shape [n, k].
+extern "C" int ta_fused_norm_gated(const void* residual, const void* norm_weight, float eps, const void* w,
+                                   void* out, int m, int n, int k, hipStream_t stream) {
+  if (m <= 0) return 0;
+  if (m > 16 || (k & 7) || (n & 1)) return -1;
+  FusedArgs a = {};
+  a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
+  a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
+  return launch_fused<EPI_GATED, true>(a, (n / 2 + 15) / 16, stream);
+}
+
+// residual [m, n] += x W^T (+ bias), x bfloat16 [m, k] with row stride lda.  `waves` (4, 8, 16; 0 = the
+// launcher's choice) lets a caller pick how many waves share a tile's K.
+extern "C" int ta_fused_linear_residual(const void* x, int lda, const void* w, const void* bias, void* residual,
+                                        int m, int n, int k, int waves, hipStream_t stream) {
+  if (m <= 0) return 0;
+  if (m > 16 || (k & 7) || (lda & 7)) return -1;
+  FusedArgs a = {};
+  a.a = (const bf16_t*)x; a.lda = lda; a.w = (const bf16_t*)w; a.bias = (const float*)bias;
+  a.m = m; a.n = n; a.k = k; a.residual_out = (float*)residual;
+  const int tiles = (n + 15) / 16;
+  if (waves == 4) return launch_one<4, EPI_RESIDUAL, false>(a, tiles, stream);
+  if (waves == 8) return launch_one<8, EPI_RESIDUAL, false>(a, tiles, stream);
+  if (waves == 16) return launch_one<16, EPI_RESIDUAL, false>(a, tiles, stream);
+  return launch_fused<EPI_RESIDUAL, false>(a, tiles, stream);
+}

@@ -52,7 +52,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual",
                      "ta_argmax"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -302,6 +302,73 @@ class Ops:
                                                      k, _BF16, 1, self._stream()), "linear_silu_gate")
             return out
         return self.silu_gate(self.linear(x, weight), out)
+
+    # ------------------------------------------------------- fused decode products
+    FUSED_ROWS = 16
+    use_fused_decode = True
+    linear_add_waves = 0      # 0: the launcher picks how many waves share a tile's K
+
+    def can_fuse_decode(self, rows: int, dtype: torch.dtype) -> bool:
+        """Batches of few bfloat16 rows can run the products that take the norm, the rotation with the
+        cache write, the gated activation and the residual add into the same kernel."""
+        return self.use_fused_decode and dtype == torch.bfloat16 and 0 < rows <= self.FUSED_ROWS
+
+    def fused_norm_qkv_rope(self, residual, norm_weight, eps, weight, bias, positions, cos_sin, slots,
+                            k_pages, v_pages, n_q: int, n_kv: int, head_dim: int) -> torch.Tensor:
+        """q, k, v = rmsnorm(residual) @ weight.T + bias; q and k rotated; k and v stored into their pages
+        (when `slots` is given); returns q [M, n_q * d] in bfloat16.  residual float32 [M, K]."""
+        _dev(residual, norm_weight, weight, bias, positions, cos_sin, slots, k_pages, v_pages)
+        m, k = residual.shape
+        _need(residual.dtype == torch.float32 and norm_weight.dtype == torch.float32 and norm_weight.numel() == k,
+              "the residual and the norm weight are float32")
+        _need(weight.dtype == torch.bfloat16 and tuple(weight.shape) == ((n_q + 2 * n_kv) * head_dim, k),
+              "the joined q/k/v matrix has the wrong shape")
+        _need(m <= self.FUSED_ROWS and k % 8 == 0 and head_dim % 32 == 0, "sizes the fused projection does not take")
+        _need(positions.dtype == torch.int32 and positions.numel() == m, "positions must be int32 [M]")
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.numel() == weight.shape[0], "bias must be float32")
+        if cos_sin is not None:
+            _need(cos_sin.dtype == torch.float32 and cos_sin.shape[1] == head_dim, "cos_sin must be float32 [P, d]")
+        page_size = 1
+        if slots is not None:
+            _need(slots.dtype == torch.int32 and slots.numel() == m, "slots must be int32 [M]")
+            _need(k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16, "pages must be bfloat16")
+            page_size = self._page_size(k_pages, v_pages, n_kv, head_dim)
+        q = torch.empty((m, n_q * head_dim), dtype=torch.bfloat16, device=residual.device)
+        self._check(self.lib.ta_fused_norm_qkv_rope(
+            _ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(weight), _ptr(bias), _ptr(q), _ptr(positions),
+            _ptr(cos_sin), _ptr(slots), _ptr(k_pages if slots is not None else None),
+            _ptr(v_pages if slots is not None else None), m, k, n_q, n_kv, head_dim, page_size, self._stream()),
+            "fused_norm_qkv_rope")
+        return q
+
+    def fused_norm_gated(self, residual, norm_weight, eps, weight) -> torch.Tensor:
+        """silu(x @ Wg.T) * (x @ Wu.T) with x = rmsnorm(residual), weight = [Wg; Wu]; bfloat16 [M, I]."""
+        _dev(residual, norm_weight, weight)
+        m, k = residual.shape
+        _need(residual.dtype == torch.float32 and norm_weight.dtype == torch.float32 and norm_weight.numel() == k,
+              "the residual and the norm weight are float32")
+        _need(weight.dtype == torch.bfloat16 and weight.shape[1] == k and weight.shape[0] % 2 == 0, "gate/up matrix shape")
+        _need(m <= self.FUSED_ROWS and k % 8 == 0, "sizes the fused product does not take")
+        out = torch.empty((m, weight.shape[0] // 2), dtype=torch.bfloat16, device=residual.device)
+        self._check(self.lib.ta_fused_norm_gated(_ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(weight),
+                                                 _ptr(out), m, weight.shape[0], k, self._stream()), "fused_norm_gated")
+        return out
+
+    def linear_add(self, x, weight, bias, residual) -> None:
+        """residual += x @ weight.T (+ bias), in place, in float32.  x bfloat16 [M, K], M <= 16."""
+        _dev(weight, bias, residual)
+        _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.dtype == torch.bfloat16, "x must be bfloat16 rows")
+        m, k = x.shape
+        n = weight.shape[0]
+        lda = x.stride(0) if m > 1 else k
+        _need(weight.dtype == torch.bfloat16 and weight.shape[1] == k, "weight shape")
+        _need(residual.dtype == torch.float32 and tuple(residual.shape) == (m, n), "the residual must be float32 [M, N]")
+        _need(m <= self.FUSED_ROWS and k % 8 == 0 and lda % 8 == 0 and x.data_ptr() % 16 == 0, "sizes not taken")
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.numel() == n, "bias must be float32 [N]")
+        self._check(self.lib.ta_fused_linear_residual(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(residual), m, n, k,
+                                                      self.linear_add_waves, self._stream()), "linear_add")
 
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:

@@ -6,6 +6,8 @@ import math
 import torch
 
 from .base import MIXERS, POSITIONS, Mixer, Runtime
+from .norm import RMSNorm
+from .position import NoPosition, RotaryHalfSplit
 from .spec import CacheNeed, MixerSpec, PositionSpec, TensorSpec
 
 
@@ -57,6 +59,25 @@ class GQAttention(Mixer):
     def cache_need(spec: MixerSpec) -> CacheNeed:
         kind = "full" if spec.window is None else "window"
         return CacheNeed(kind=kind, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window)
+
+    def forward_normed(self, residual, delta, norm, ctx, cache):
+        """Decode batches of few bfloat16 rows: norm + q/k/v product + bias + rotation + cache write in one
+        kernel, attention, then the output product added straight into the residual stream."""
+        ops = self.runtime.ops
+        fused = (delta is None and type(norm) is RMSNorm and type(self.position) in (NoPosition, RotaryHalfSplit)
+                 and self.d % 32 == 0 and cache.group is not None
+                 and getattr(ops, "can_fuse_decode", lambda rows, dtype: False)(residual.shape[0], self.runtime.dtype))
+        if not fused:
+            return super().forward_normed(residual, delta, norm, ctx, cache)
+        q = ops.fused_norm_qkv_rope(residual, norm.weight, norm.eps, self.w_qkv, self.b_qkv, ctx.positions,
+                                    self.position.table(), ctx.slots[cache.group] if cache.writes else None,
+                                    cache.k_pages, cache.v_pages, self.n_q, self.n_kv, self.d)
+        mixed = torch.empty((q.shape[0], self.n_q * self.d), dtype=q.dtype, device=q.device)
+        ops.paged_attention(q, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
+                            ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
+                            self.scale, max_position=ctx.max_position, batch=ctx)
+        ops.linear_add(mixed, self.w_o, self.b_o, residual)
+        return None
 
     def forward(self, x, ctx, cache):
         ops = self.runtime.ops

@@ -14,7 +14,9 @@ PositionEncoding
                 the query and key heads in place and writes keys and values of this step into `cache`.
 Mixer           tensor_specs(spec), cache_need(spec) -> CacheNeed
                 forward(x [T, H], ctx: StepContext, cache: LayerCache) -> [T, H] in the compute dtype.
-FeedForward     tensor_specs(spec); forward(x [T, H], ctx) -> [T, H].
+                Optional: forward_normed(residual, delta, norm, ctx, cache) to fold the norm before it and the
+                residual add after it into its own kernels (returns None when it added its output itself).
+FeedForward     tensor_specs(spec); forward(x [T, H], ctx) -> [T, H]; optional forward_normed likewise.
 Block           arranges two norms, a mixer and a feed-forward around the residual stream:
                 forward(residual, delta, ctx, cache) -> delta still to be added.
 """
@@ -98,10 +100,20 @@ class Mixer(Part):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_normed(self, residual, delta, norm: Norm, ctx, cache):
+        """The sub-layer from the residual stream on: add `delta`, normalise, mix.  Returns the output still
+        to be added to the stream, or None if the part added it itself.  A part may override this to fold
+        the norm and the add into its own kernels; this default keeps them apart."""
+        return self.forward(norm.apply(residual, delta), ctx, cache)
+
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         raise NotImplementedError
+
+    def forward_normed(self, residual, delta, norm: Norm, ctx):
+        """As `Mixer.forward_normed`, for the feed-forward."""
+        return self.forward(norm.apply(residual, delta), ctx)
 
 
 class Block:

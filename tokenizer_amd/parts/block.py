@@ -9,7 +9,7 @@ class PreNormBlock(Block):
     """x + mixer(norm1(x)), then + feed_forward(norm2(.)) (qwen-infer/src/model.rs:615-622).
 
     The residual stream is float32.  Each sub-layer's output is handed on as a pending `delta`
-    so that the add fuses into the next norm.
+    so that the add fuses into the next norm; a part that added its output itself hands on None.
     """
     graph_safe = True
 
@@ -19,7 +19,5 @@ class PreNormBlock(Block):
         self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
 
     def forward(self, residual, delta, ctx, cache):
-        normed = self.mixer_norm.apply(residual, delta)
-        mixed = self.mixer.forward(normed, ctx, cache)
-        normed = self.feed_forward_norm.apply(residual, mixed)
-        return self.feed_forward.forward(normed, ctx)
+        mixed = self.mixer.forward_normed(residual, delta, self.mixer_norm, ctx, cache)
+        return self.feed_forward.forward_normed(residual, mixed, self.feed_forward_norm, ctx)

@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from .base import FEED_FORWARDS, FeedForward, Runtime
+from .norm import RMSNorm
 from .spec import FeedForwardSpec, TensorSpec
 
 
@@ -29,6 +30,18 @@ class GatedDense(FeedForward):
         return {"gate_proj.weight": TensorSpec((spec.intermediate_size, spec.hidden_size)),
                 "up_proj.weight": TensorSpec((spec.intermediate_size, spec.hidden_size)),
                 "down_proj.weight": TensorSpec((spec.hidden_size, spec.intermediate_size))}
+
+    def forward_normed(self, residual, delta, norm, ctx):
+        """Decode batches of few bfloat16 rows: norm + gate/up product + activation in one kernel, then the
+        down product added straight into the residual stream."""
+        ops = self.runtime.ops
+        fused = (delta is None and type(norm) is RMSNorm
+                 and getattr(ops, "can_fuse_decode", lambda rows, dtype: False)(residual.shape[0], self.runtime.dtype))
+        if not fused:
+            return super().forward_normed(residual, delta, norm, ctx)
+        act = ops.fused_norm_gated(residual, norm.weight, norm.eps, self.w_gate_up)
+        ops.linear_add(act, self.w_down, None, residual)
+        return None
 
     def forward(self, x, ctx):
         ops = self.runtime.ops
