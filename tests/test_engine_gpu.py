@@ -31,11 +31,12 @@ def engine_for(folder, dtype, **kw):
     return Engine(load_model(folder, dtype), **kw)
 
 
-def close(got, want, dtype):
+def close(got, want, dtype, tolerance=None):
     got = got.float().cpu()
     err = float((got - want).abs().max())
     scale = float(want.abs().max())
-    assert err <= TOL[dtype] * max(scale, 1.0), f"max abs error {err} against logits up to {scale}"
+    bound = (TOL[dtype] if tolerance is None else tolerance) * max(scale, 1.0)
+    assert err <= bound, f"max abs error {err} against logits up to {scale}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -185,3 +186,72 @@ def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
         torch.testing.assert_close(got[0][0], got[1][0], rtol=0, atol=0)
         assert got[0][1] == got[1][1]
     assert len(engines[0].graphs) >= 3
+
+
+def sharpened(folder, out_folder, factor):
+    """A copy of a model folder whose query and key projections are scaled up: attention becomes nearly
+    one-hot, so a wrong key, page or window edge changes the logits by far more than any rounding."""
+    import shutil
+    from safetensors.torch import load_file
+    from tokenizer_amd.weights import save_safetensors
+    shutil.copytree(folder, out_folder)
+    tensors = {k: v.clone() for k, v in load_file(folder + "/model.safetensors").items()}   # not views of a mapped file
+    for name in tensors:
+        if "q_proj" in name or "k_proj" in name:
+            tensors[name] = (tensors[name].float() * factor).to(torch.bfloat16)
+    save_safetensors(out_folder + "/model.safetensors", tensors)
+    return out_folder
+
+
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_peaked_attention_over_hundreds_of_keys(model_folders, tmp_path, name):
+    # float32 only: with weights like these bfloat16 rounding alone moves the nearly one-hot choices.
+    folder = sharpened(model_folders[name], str(tmp_path / "sharp"), 24.0)
+    cfg, tensors = plain.load_folder(folder)
+    _, tensors64 = plain.load_folder(folder, torch.float64)
+    vocab, limit = cfg["vocab_size"], cfg["max_position_embeddings"]
+    reqs = {f"r{i}": random_ids(vocab, min(n, limit), 90 + i) for i, n in enumerate([250, 97, 33, 180])}
+    exact = {rid: plain.all_logits(cfg, tensors64, ids).float() for rid, ids in reqs.items()}
+    want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
+    # Scores are 24^2 times larger here and carry that much more float32 rounding into the softmax, in any
+    # implementation.  So the yardstick is the plain float32 implementation's own distance from a float64
+    # run: the engine may be a few times that, no more.  A wrong key moves these logits by more than 0.05.
+    plain_error = max(float((want[r] - exact[r]).abs().max()) for r in reqs)
+    for steps in (tt.mixed(reqs, 8), tt.decode_tail(reqs, 32)):
+        eng = engine_for(folder, "float32", max_tokens=tt.peak_tokens(steps), max_requests=4)
+        eng.pools.poison()
+        got = tt.run_in_process(eng, steps)
+        for rid in reqs:
+            err = float((got[rid] - exact[rid]).abs().max())
+            assert err <= 4 * plain_error + 2e-5, f"engine off by {err}, plain float32 by {plain_error}"
+    # The sharpening matters: the same engine run on the original weights is far from these logits.
+    eng = engine_for(model_folders[name], "float32", max_tokens=1024, max_requests=4)
+    other = tt.run_in_process(eng, tt.whole(reqs))
+    assert max(float((other[r] - want[r]).abs().max()) for r in reqs) > 0.05
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_points(model_folders, tmp_path, dtype):
+    import subprocess
+    import sys
+    from tokenizer_amd.engine import GenerateParams, generate, greedy_tokens
+    name = "B"
+    cfg, tensors = plain.load_folder(model_folders[name])
+    prompt = random_ids(cfg["vocab_size"], 11, 5)
+    want = plain.greedy_generate(cfg, tensors, prompt, 8)
+    eng = engine_for(model_folders[name], dtype, num_pages=8, max_requests=2)
+    out = generate(eng, prompt, GenerateParams.greedy(8))
+    if dtype == "float32":
+        assert out.tokens == want and greedy_tokens(eng, prompt, 8) == want
+    assert out.completion_tokens == 8 and out.reason.value == "MaxTokens" and out.prefill > 0 and out.decode > 0
+    # The command line: ids in, ids out (the folder has no tokenizer.json), the reference's lines on stderr.
+    root = tt.ROOT
+    run = subprocess.run([sys.executable, f"{root}/bin/qwen-infer", "--model", model_folders[name], "--dtype", dtype,
+                          "--max-tokens", "8", "--token-ids", " ".join(map(str, prompt))],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert f"prompt ids ({len(prompt)}): {prompt}" in run.stderr
+    assert "max_tokens 8 temperature 0.0 top_p 1.0 seed 0 eos []" in run.stderr
+    assert f"generated ids: {out.tokens}" in run.stderr and "stop: MaxTokens" in run.stderr
+    assert "tok/s (8 tokens, KV cache, total" in run.stderr
+    assert run.stdout.split() == [str(t) for t in out.tokens]

@@ -1,0 +1,337 @@
+"""Each part of a layer alone against the plain implementation, and parts defined here, outside the package:
+a mixer with state of its own, a model whose layers have different mixers, a schedule that runs a layer twice
+on one cache."""
+import dataclasses
+import math
+
+import pytest
+import torch
+
+from plain import qwen2_plain as plain
+from tiny_configs import random_ids
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: dict(rtol=1e-4, atol=2e-5), torch.bfloat16: dict(rtol=3e-2, atol=3e-2)}
+
+
+def close(got, want, dtype):
+    """float32: elementwise.  bfloat16: every rounding is 2^-9 relative to the values around it, and a few of
+    them pile up, so the bound is relative to the largest value of the result (2 %), not to each element."""
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, **TOL[dtype])
+    else:
+        err, scale = float((got - want).abs().max()), float(want.abs().max())
+        assert err <= 2e-2 * scale, f"max abs error {err} against values up to {scale}"
+
+
+def runtime(dtype):
+    from tokenizer_amd.kernels import get_ops
+    from tokenizer_amd.parts import Runtime
+    return Runtime(dtype, torch.device("cuda:0"), get_ops())
+
+
+def context_for(needs, lengths, dtype, page_size=16, chunks=None):
+    """A cache manager, pools and the step context of whole sequences of the given lengths."""
+    from tokenizer_amd.cache import CacheManager, CachePools
+    from tokenizer_amd.engine.batch import StepEntry, build_context
+    manager = CacheManager(needs, num_pages=sum(-(-n // page_size) for n in lengths) + 2, page_size=page_size,
+                           max_requests=len(lengths))
+    pools = CachePools(manager, needs, dtype, "cuda:0")
+    pools.poison()
+    entries = []
+    for rid, n in enumerate(lengths):
+        manager.add_request(rid)
+        assert manager.reserve(rid, n)
+        entries.append(StepEntry(rid, [0] * n, []))
+    return manager, pools, build_context(entries, manager, "cuda:0")
+
+
+def rand(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from tokenizer_amd.parts import NORMS, NormSpec
+    spec = NormSpec("rmsnorm", 72, 3e-5)
+    weight = rand((72,), 1) * 0.1 + 1
+    norm = NORMS.get("rmsnorm")(spec, {"weight": weight.cuda()}, runtime(dtype))
+    residual, delta = rand((9, 72), 2, 3.0), rand((9, 72), 3).to(dtype)
+    res = residual.cuda().clone()
+    out = norm.apply(res, delta.cuda())
+    want_res = residual + delta.float()
+    torch.testing.assert_close(res.cpu(), want_res, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(out.float().cpu(), plain.rms_norm(want_res, weight, 3e-5), **TOL[dtype])
+    rows = torch.tensor([8, 2], dtype=torch.int32).cuda()
+    out = norm.apply(res, None, rows=rows)
+    torch.testing.assert_close(out.float().cpu(), plain.rms_norm(want_res[[8, 2]], weight, 3e-5), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_position_part_rotates_and_stores(dtype):
+    from tokenizer_amd.parts import POSITIONS, CacheNeed, LayerCache, PositionSpec
+    n_q, n_kv, d = 3, 1, 32
+    need = CacheNeed("full", n_kv, d)
+    manager, pools, ctx = context_for([need], [21, 5], dtype)
+    k_pages, v_pages = pools.layer_pages(0)
+    cache = LayerCache(group=0, k_pages=k_pages, v_pages=v_pages)
+    rope = POSITIONS.get("rope_half_split")(PositionSpec("rope_half_split", d, 1e6, 64), runtime(dtype))
+    qkv = rand((26, (n_q + 2 * n_kv) * d), 4).to(dtype)
+    work = qkv.cuda().clone()
+    rope.encode_and_store(work, None, n_q, n_kv, d, ctx, cache)
+    cos, sin = plain.rope_tables(1e6, d, 64)
+    positions = list(range(21)) + list(range(5))
+    heads = qkv.float().reshape(26, n_q + 2 * n_kv, d).transpose(0, 1)
+    want = plain.apply_rope(heads[:n_q + n_kv], cos[positions], sin[positions])
+    got = work.float().cpu().reshape(26, n_q + 2 * n_kv, d).transpose(0, 1)
+    torch.testing.assert_close(got[:n_q + n_kv], want, **TOL[dtype])
+    torch.testing.assert_close(got[n_q + n_kv:], heads[n_q + n_kv:], rtol=0, atol=0)     # values are not rotated
+    # Request 0's token 17 sits in its second page at offset 1: keys row-wise, values transposed.
+    page = manager.table(0, 0)[1]
+    torch.testing.assert_close(k_pages[page, 0, 1].float().cpu(), want[n_q, 17], **TOL[dtype])
+    torch.testing.assert_close(v_pages[page, 0, :, 1].float().cpu(), heads[n_q + n_kv, 17], rtol=0, atol=0)
+    # "none" leaves the heads as they are and still stores them.
+    none = POSITIONS.get("none")(PositionSpec("none"), runtime(dtype))
+    work = qkv.cuda().clone()
+    none.encode_and_store(work, None, n_q, n_kv, d, ctx, cache)
+    torch.testing.assert_close(work.float().cpu(), qkv.float(), rtol=0, atol=0)
+    torch.testing.assert_close(k_pages[page, 0, 1].float().cpu(), heads[n_q, 17], rtol=0, atol=0)
+
+
+def attention_tensors(n_q, n_kv, d, hidden, seed):
+    names = {"q_proj.weight": (n_q * d, hidden), "k_proj.weight": (n_kv * d, hidden), "v_proj.weight": (n_kv * d, hidden),
+             "o_proj.weight": (hidden, n_q * d), "q_proj.bias": (n_q * d,), "k_proj.bias": (n_kv * d,),
+             "v_proj.bias": (n_kv * d,)}
+    return {name: rand(shape, seed + i, 0.2).to(torch.bfloat16).float() for i, (name, shape) in enumerate(names.items())}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("geometry", [(6, 2, 16, 40, None), (4, 4, 32, 72, 9), (14, 2, 64, 96, None)])
+def test_attention_mixer_alone(dtype, geometry):
+    from tokenizer_amd.parts import MIXERS, LayerCache, MixerSpec, PositionSpec
+    n_q, n_kv, d, hidden, window = geometry
+    spec = MixerSpec("gqa_attention", hidden, n_q, n_kv, d, qkv_bias=True, window=window,
+                     position=PositionSpec("rope_half_split", d, 10000.0, 128))
+    mixer_cls = MIXERS.get("gqa_attention")
+    tensors = attention_tensors(n_q, n_kv, d, hidden, 10)
+    assert set(mixer_cls.tensor_specs(spec)) == set(tensors)
+    assert {k: v.shape for k, v in mixer_cls.tensor_specs(spec).items()} == {k: tuple(v.shape) for k, v in tensors.items()}
+    need = mixer_cls.cache_need(spec)
+    assert need.kind == ("window" if window else "full") and (need.n_kv_heads, need.head_dim) == (n_kv, d)
+    held = {k: (v.to(dtype) if v.dim() == 2 else v).cuda() for k, v in tensors.items()}
+    mixer = mixer_cls(spec, held, runtime(dtype))
+    lengths = [37, 16, 3]
+    manager, pools, ctx = context_for([need], lengths, dtype)
+    k_pages, v_pages = pools.layer_pages(0)
+    x = rand((sum(lengths), hidden), 20).to(dtype)
+    out = mixer.forward(x.cuda(), ctx, LayerCache(group=0, k_pages=k_pages, v_pages=v_pages)).float().cpu()
+    cos, sin = plain.rope_tables(10000.0, d, 128)
+    named = {f"a.{k}": v for k, v in tensors.items()}
+    at = 0
+    for n in lengths:
+        want = plain.self_attention(x[at:at + n].float(), named, "a", n_q, n_kv, d, cos, sin, list(range(n)), window)
+        close(out[at:at + n], want, dtype)
+        at += n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows", [5, 130])
+def test_feed_forward_alone(dtype, rows):
+    from tokenizer_amd.parts import FEED_FORWARDS, FeedForwardSpec
+    spec = FeedForwardSpec("gated_dense", 72, 136, "silu")
+    tensors = {"gate_proj.weight": rand((136, 72), 1, 0.2), "up_proj.weight": rand((136, 72), 2, 0.2),
+               "down_proj.weight": rand((72, 136), 3, 0.2)}
+    tensors = {k: v.to(torch.bfloat16).float() for k, v in tensors.items()}
+    part = FEED_FORWARDS.get("gated_dense")(spec, {k: v.to(dtype).cuda() for k, v in tensors.items()}, runtime(dtype))
+    x = rand((rows, 72), 4).to(dtype)
+    out = part.forward(x.cuda(), None).float().cpu()
+    want = plain.mlp(x.float(), {f"m.{k}": v for k, v in tensors.items()}, "m")
+    close(out, want, dtype)
+    with pytest.raises(ValueError):
+        FEED_FORWARDS.get("gated_dense")(FeedForwardSpec("gated_dense", 72, 136, "gelu"), {}, runtime(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_alone(dtype):
+    # One pre-norm block with its own sizes: norm, attention, add, norm, feed-forward, add (the last add is
+    # left to the next norm, so the block hands back the stream and what is still to be added).
+    from tokenizer_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, FeedForwardSpec, LayerCache, MixerSpec,
+                                     NormSpec, PositionSpec)
+    n_q, n_kv, d, hidden, inner = 3, 1, 32, 96, 136
+    rt = runtime(dtype)
+    cfg = {"rms_norm_eps": 2e-5, "num_attention_heads": n_q, "num_key_value_heads": n_kv, "hidden_size": hidden}
+    t = {f"model.layers.0.self_attn.{k}": v for k, v in attention_tensors(n_q, n_kv, d, hidden, 30).items()}
+    for name, shape, seed in (("mlp.gate_proj.weight", (inner, hidden), 40), ("mlp.up_proj.weight", (inner, hidden), 41),
+                              ("mlp.down_proj.weight", (hidden, inner), 42)):
+        t[f"model.layers.0.{name}"] = rand(shape, seed, 0.1).to(torch.bfloat16).float()
+    t["model.layers.0.input_layernorm.weight"] = rand((hidden,), 43) * 0.1 + 1
+    t["model.layers.0.post_attention_layernorm.weight"] = rand((hidden,), 44) * 0.1 + 1
+
+    def held(prefix):
+        return {k[len(prefix) + 1:]: (v.to(dtype) if v.dim() == 2 else v.float()).cuda() for k, v in t.items()
+                if k.startswith(prefix + ".")}
+    mixer_spec = MixerSpec("gqa_attention", hidden, n_q, n_kv, d, qkv_bias=True,
+                           position=PositionSpec("rope_half_split", d, 10000.0, 64))
+    norm_spec = NormSpec("rmsnorm", hidden, 2e-5)
+    block = BLOCKS.get("pre_norm")(
+        NORMS.get("rmsnorm")(norm_spec, held("model.layers.0.input_layernorm"), rt),
+        MIXERS.get("gqa_attention")(mixer_spec, held("model.layers.0.self_attn"), rt),
+        NORMS.get("rmsnorm")(norm_spec, held("model.layers.0.post_attention_layernorm"), rt),
+        FEED_FORWARDS.get("gated_dense")(FeedForwardSpec("gated_dense", hidden, inner), held("model.layers.0.mlp"), rt))
+    for lengths in ([29, 7], [1, 1, 1]):           # the second batch is small enough for the fused decode kernels
+        need = MIXERS.get("gqa_attention").cache_need(mixer_spec)
+        manager, pools, ctx = context_for([need], lengths, dtype)
+        k_pages, v_pages = pools.layer_pages(0)
+        x = rand((sum(lengths), hidden), 45)
+        residual = x.cuda().clone()
+        delta = block.forward(residual, None, ctx, LayerCache(group=0, k_pages=k_pages, v_pages=v_pages))
+        got = residual.cpu() + (0 if delta is None else delta.float().cpu())
+        cos, sin = plain.rope_tables(10000.0, d, 64)
+        at = 0
+        for n in lengths:
+            want = plain.decoder_layer(x[at:at + n], cfg, t, 0, cos, sin, list(range(n)))
+            close(got[at:at + n], want, dtype)
+            at += n
+
+
+# ------------------------------------------------------------------------------------------------
+# Parts and an architecture defined here, not in the package.
+def register_toys():
+    from tokenizer_amd.config import get_architecture, register_architecture, registered_architectures
+    from tokenizer_amd.config.base import ModelConfig
+    if "ToyMixedForCausalLM" in registered_architectures():
+        return get_architecture("ToyMixedForCausalLM").config_class
+    from tokenizer_amd.parts import (MIXERS, CacheNeed, FeedForwardSpec, LayerSpec, Mixer, MixerSpec, ModelSpec,
+                                     NormSpec, PositionSpec, ScheduleEntry, TensorSpec)
+
+    if "running_mean" not in MIXERS.kinds():
+        @MIXERS.register("running_mean")
+        class RunningMean(Mixer):
+            """y_t = W * mean(x_0 .. x_t): the sum so far is the request's state, one slot of fixed size."""
+
+            def __init__(self, spec, tensors, rt):
+                self.hidden, self.rt, self.w = spec.hidden_size, rt, tensors["mix.weight"]
+
+            @staticmethod
+            def tensor_specs(spec):
+                return {"mix.weight": TensorSpec((spec.hidden_size, spec.hidden_size), std=0.1)}
+
+            @staticmethod
+            def cache_need(spec):
+                return CacheNeed(kind="none", state_shape=(spec.hidden_size,), state_dtype="float32")
+
+            def forward(self, x, ctx, cache):
+                means = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+                for info in ctx.entries:
+                    rows = slice(info.q_start, info.q_start + info.q_len)
+                    state = cache.state[info.slot]
+                    if info.position == 0:
+                        state.zero_()                      # a new request starts from nothing, whoever had the slot
+                    sums = torch.cumsum(x[rows].float(), dim=0) + state
+                    counts = torch.arange(info.position + 1, info.position + info.q_len + 1, device=x.device)
+                    means[rows] = sums / counts[:, None]
+                    state.copy_(sums[-1])
+                return self.rt.ops.linear(means.to(x.dtype), self.w)
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        vocab_size: int
+        hidden_size: int
+        heads: int
+        inner: int
+        twice: bool = False
+
+    def toy_spec(cfg):
+        d = cfg.hidden_size // cfg.heads
+        norm = NormSpec("rmsnorm", cfg.hidden_size, 1e-5)
+        ff = FeedForwardSpec("gated_dense", cfg.hidden_size, cfg.inner, "silu")
+        mixers = [MixerSpec("running_mean", cfg.hidden_size),
+                  MixerSpec("gqa_attention", cfg.hidden_size, cfg.heads, cfg.heads, d, qkv_bias=False,
+                            position=PositionSpec("rope_half_split", d, 10000.0, 256))]
+        layers = tuple(LayerSpec("pre_norm", m, ff, norm, norm, f"l.{i}.mix", f"l.{i}.ff", f"l.{i}.n1", f"l.{i}.n2")
+                       for i, m in enumerate(mixers))
+        # `twice`: the attention layer runs a second time and then reads the keys and values of its first run.
+        schedule = (ScheduleEntry(0), ScheduleEntry(1)) + ((ScheduleEntry(1, cache_of=1),) if cfg.twice else ())
+        return ModelSpec("ToyMixedForCausalLM", cfg.vocab_size, cfg.hidden_size, 256, "emb.weight", layers, schedule,
+                         norm, "final", tied_head=True, head_name="head.weight")
+
+    register_architecture("ToyMixedForCausalLM", ToyConfig, toy_spec)
+    return ToyConfig
+
+
+def toy_plain_logits(tensors, ids, heads, twice):
+    """The toy model on whole sequences with the plain parts."""
+    t = {k: v.float() for k, v in tensors.items()}
+    hidden = t["emb.weight"].shape[1]
+    d = hidden // heads
+    x = t["emb.weight"][ids]
+    n = len(ids)
+
+    def ff(x, i):
+        h = plain.rms_norm(x, t[f"l.{i}.n2.weight"], 1e-5)
+        return x + plain.mlp(h, {f"m.{k.split('.ff.')[1]}": v for k, v in t.items() if f"l.{i}.ff." in k}, "m")
+
+    h = plain.rms_norm(x, t["l.0.n1.weight"], 1e-5)
+    means = torch.cumsum(h, 0) / torch.arange(1, n + 1)[:, None]
+    x = ff(x + means @ t["l.0.mix.mix.weight"].t(), 0)
+    cos, sin = plain.rope_tables(10000.0, d, 256)
+    pos = list(range(n))
+
+    def heads_of(h, name, rotate):
+        v = (h @ t[f"l.1.mix.{name}.weight"].t()).reshape(n, heads, d).transpose(0, 1)
+        return plain.apply_rope(v, cos[pos], sin[pos]) if rotate else v
+
+    mask = plain.attention_mask(pos, pos, None)
+    h = plain.rms_norm(x, t["l.1.n1.weight"], 1e-5)
+    k, v = heads_of(h, "k_proj", True), heads_of(h, "v_proj", False)
+    mixed = plain.attend(heads_of(h, "q_proj", True), k, v, mask).transpose(0, 1).reshape(n, hidden)
+    x = ff(x + mixed @ t["l.1.mix.o_proj.weight"].t(), 1)
+    if twice:
+        h = plain.rms_norm(x, t["l.1.n1.weight"], 1e-5)
+        mixed = plain.attend(heads_of(h, "q_proj", True), k, v, mask).transpose(0, 1).reshape(n, hidden)   # first run's k, v
+        x = ff(x + mixed @ t["l.1.mix.o_proj.weight"].t(), 1)
+    return plain.rms_norm(x, t["final.weight"], 1e-5) @ t["emb.weight"].t()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("twice", [False, True])
+def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype, twice):
+    import trace_tools as tt
+    import tokenizer_amd as ta
+    from safetensors.torch import load_file
+    from tokenizer_amd.engine import Engine, Scheduler, SchedulerConfig, GenerateParams, load_model
+
+    config_cls = register_toys()
+    cfg = config_cls.from_dict({"vocab_size": 96, "hidden_size": 64, "heads": 2, "inner": 88, "twice": twice})
+    folder = ta.write_random_model(cfg, 3, str(tmp_path / "toy"))
+    tensors = load_file(folder + "/model.safetensors")
+    assert "l.0.mix.mix.weight" in tensors and "l.1.mix.q_proj.weight" in tensors and "l.1.mix.q_proj.bias" not in tensors
+    model = load_model(folder, dtype)
+    assert [n.kind for n in model.cache_needs] == ["none", "full"] and model.cache_needs[0].state_shape == (64,)
+    assert not model.decoder.graph_safe           # the toy mixer loops over requests on the host
+    requests = {f"r{i}": random_ids(96, n, 60 + i) for i, n in enumerate([1, 23, 64, 40, 9])}
+    steps = tt.mixed(requests, 7, max_live=3)
+    engine = Engine(model, max_tokens=tt.peak_tokens(steps), max_requests=3)
+    assert len(engine.cache.groups) == 1 and engine.cache.state_layers == [0]
+    engine.pools.poison()
+    got = tt.run_in_process(engine, steps)
+    for rid, ids in requests.items():
+        want = toy_plain_logits(tensors, ids, 2, twice)
+        err = float((got[rid] - want).abs().max())
+        assert err <= (2e-5 if dtype == "float32" else 4e-2) * max(1.0, float(want.abs().max())), (rid, err)
+    engine.cache.check_invariants()
+    # The scheduler, preemption included, works on it unchanged: few pages, outputs equal to running alone.
+    small = Engine(model, num_pages=5, max_requests=3)
+    sched = Scheduler(small, SchedulerConfig(num_blocks=5, prefix_cache=False, max_batch_size=3))
+    prompts = [random_ids(96, n, 80 + n) for n in (30, 28, 14)]
+    rids = [sched.add_request(p, GenerateParams.greedy(6)) for p in prompts]
+    results = sched.run()
+    assert sched.stats.preemptions >= 1
+    if dtype == "float32":
+        for rid, prompt in zip(rids, prompts):
+            ids = list(prompt)
+            for _ in range(6):
+                ids.append(plain.greedy_token(toy_plain_logits(tensors, ids, 2, twice)[-1]))
+            assert results[rid].tokens == ids[len(prompt):]
+    sched.assert_idle()
