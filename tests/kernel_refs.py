@@ -141,6 +141,14 @@ class PlainOps:
             y = y + bias.to(self.work)
         residual.add_(y.to(torch.float32))
 
+    def sample(self, logits, temperature, top_p, uniform, out=None):
+        from plain import qwen2_plain as plain
+        result = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device) if out is None else out
+        for row in range(logits.shape[0]):
+            result[row] = plain.sample_token(logits[row].float().cpu().numpy(), float(temperature[row]),
+                                             float(top_p[row]), float(uniform[row]))
+        return result
+
     def argmax(self, logits, out=None):
         result = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device) if out is None else out
         for row in range(logits.shape[0]):

@@ -255,3 +255,26 @@ def test_greedy_generation_through_the_entry_points(model_folders, tmp_path, dty
     assert f"generated ids: {out.tokens}" in run.stderr and "stop: MaxTokens" in run.stderr
     assert "tok/s (8 tokens, KV cache, total" in run.stderr
     assert run.stdout.split() == [str(t) for t in out.tokens]
+
+
+def test_warm_requests_draw_on_the_device_as_they_would_alone(model_folders):
+    # Temperature and nucleus draws in a batch of the scheduler equal the same requests run one by one:
+    # the uniform numbers are the request's own, and the sampling kernel sees only that request's row.
+    from tokenizer_amd.engine import GenerateParams, Scheduler, SchedulerConfig, generate
+    name = "A"
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [random_ids(vocab, n, 70 + n) for n in (4, 9, 2, 17)]
+    params = [GenerateParams(max_tokens=10, temperature=t, top_p=p, seed=s)
+              for t, p, s in ((1.3, 0.95, 5), (0.7, 1.0, 6), (1.3, 0.5, 5), (0.0, 1.0, 1))]
+    eng = engine_for(model_folders[name], "float32", num_pages=32, max_requests=4)
+    sched = Scheduler(eng, SchedulerConfig(num_blocks=32, max_batch_size=4))
+    rids = [sched.add_request(p, q) for p, q in zip(prompts, params)]
+    results = sched.run()
+    solo = engine_for(model_folders[name], "float32", num_pages=32, max_requests=1)
+    for rid, prompt, q in zip(rids, prompts, params):
+        assert results[rid].tokens == generate(solo, prompt, q).tokens
+    assert len({tuple(results[r].tokens) for r in rids}) == 4
+    again = generate(solo, prompts[0], params[0]).tokens
+    other = generate(solo, prompts[0], GenerateParams(max_tokens=10, temperature=1.3, top_p=0.95, seed=6)).tokens
+    assert again == results[rids[0]].tokens and other != again
+    sched.assert_idle()

@@ -4,8 +4,23 @@ from __future__ import annotations
 
 import time
 
-from .generate import Control, GenerateParams, Generated, SampleCursor, Sampled, StopReason, _go_on, _no_bytes
 from .batch import StepEntry
+from .generate import Control, GenerateParams, Generated, SampleCursor, Sampled, StopReason, _go_on, _no_bytes
+
+
+def _next(engine, cursor: SampleCursor, logits, token_bytes, on_chunk):
+    """Pick the next id on the device (greedy, or a warm draw with the cursor's next uniform number) and hand
+    it to the cursor; an engine without a device sampler gets the logits row drawn on the host."""
+    if cursor.exhausted:
+        return cursor.push_token(0, token_bytes, on_chunk)        # finishes, nothing is drawn
+    if cursor.is_greedy:
+        token = engine.argmax(logits, [0])[0]
+    elif hasattr(engine, "sample"):
+        token = engine.sample(logits, [0], [cursor.params.temperature], [cursor.params.top_p],
+                              [cursor.next_uniform()])[0]
+    else:
+        return cursor.push_logits(engine.rows_to_host(logits, [0])[0], token_bytes, on_chunk)
+    return cursor.push_token(token, token_bytes, on_chunk)
 
 
 def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes=_no_bytes,
@@ -23,10 +38,9 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
     engine.add_request(rid)
     try:
         started = time.perf_counter()
-        wants = [len(prompt) - 1] if params.max_tokens > 0 else []
-        logits = engine.step([StepEntry(rid, list(prompt), wants)])
-        if wants:
-            logits_row = _row(engine, logits, cursor)
+        logits = engine.step([StepEntry(rid, list(prompt), [len(prompt) - 1] if params.max_tokens > 0 else [])])
+        if params.max_tokens > 0:
+            engine.argmax(logits, [0])                 # waits for the prompt's forward, so the clock is honest
         prefill = time.perf_counter() - started
         started = time.perf_counter()
         if params.max_tokens == 0:
@@ -35,29 +49,15 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
             done = Sampled([], "", [], StopReason.Cancelled, 0)
         else:
             while True:
-                outcome = _push(cursor, logits_row, token_bytes, on_chunk)
+                outcome = _next(engine, cursor, logits, token_bytes, on_chunk)
                 if isinstance(outcome, Sampled):
                     done = outcome
                     break
                 logits = engine.step([StepEntry(rid, [int(outcome)], [0])])
-                logits_row = _row(engine, logits, cursor)
         decode = time.perf_counter() - started
     finally:
         engine.end_request(rid)
     return Generated(done.tokens, done.text, done.chunks, done.reason, done.completion_tokens, prefill, decode)
-
-
-def _row(engine, logits, cursor):
-    """Greedy: the id picked on the device; warm: the logits row on the host."""
-    if cursor.is_greedy:
-        return engine.argmax(logits, [0])[0]
-    return engine.rows_to_host(logits, [0])[0]
-
-
-def _push(cursor, picked, token_bytes, on_chunk):
-    if cursor.is_greedy:
-        return cursor.push_token(picked, token_bytes, on_chunk)
-    return cursor.push_logits(picked, token_bytes, on_chunk)
 
 
 def generate(engine, prompt: list[int], params: GenerateParams, token_bytes=_no_bytes) -> Generated:

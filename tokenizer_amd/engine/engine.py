@@ -148,6 +148,17 @@ class Engine:
             picked = self.model.runtime.ops.argmax(logits).cpu().tolist()
         return picked if rows is None else [picked[row] for row in rows]
 
+    def sample(self, logits: torch.Tensor, rows: list[int], temperature: list[float], top_p: list[float],
+               uniform: list[float]) -> list[int]:
+        """Temperature / nucleus draws for the given rows of a step's logits, on the device; one uniform
+        number per row (from the request's own generator)."""
+        device = logits.device
+        picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=device)]
+        as_tensor = lambda values: torch.tensor(values, dtype=torch.float32, device=device)
+        ids = self.model.runtime.ops.sample(picked.contiguous(), as_tensor(temperature), as_tensor(top_p),
+                                            as_tensor(uniform))
+        return [int(v) for v in ids.cpu().tolist()]
+
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):
         return logits[rows].float().cpu().numpy()
 

@@ -91,7 +91,8 @@ class Scheduler:
     """Admits requests, cuts prompts into portions, decodes, finishes and frees.
 
     `engine` needs: `.cache` (a CacheManager), `.step(entries) -> logits`, `.argmax(logits, rows) ->
-    list[int]`, `.rows_to_host(logits, rows) -> float32 array`, `.max_positions`.
+    list[int]`, `.max_positions`, and for warm requests `.sample(logits, rows, temperature, top_p, uniform)
+    -> list[int]` or, without it, `.rows_to_host(logits, rows) -> float32 array` (drawn on the host then).
     """
 
     def __init__(self, engine, config: SchedulerConfig | None = None):
@@ -244,7 +245,17 @@ class Scheduler:
         if greedy_rows:
             for row, token in zip(greedy_rows, self.engine.argmax(logits, greedy_rows)):
                 picked[row] = int(token)
-        warm_logits = self.engine.rows_to_host(logits, warm_rows) if warm_rows else None
+        warm_logits = None
+        if warm_rows and hasattr(self.engine, "sample"):
+            # Drawn on the device: each request brings its own uniform number, so a draw does not depend on
+            # who else is in the batch.
+            cursors = [wanting[row].cursor for row in warm_rows]
+            tokens = self.engine.sample(logits, warm_rows, [c.params.temperature for c in cursors],
+                                        [c.params.top_p for c in cursors], [c.next_uniform() for c in cursors])
+            for row, token in zip(warm_rows, tokens):
+                picked[row] = int(token)
+        elif warm_rows:
+            warm_logits = self.engine.rows_to_host(logits, warm_rows)
         elapsed = time.perf_counter() - started
         self.stats.steps += 1
         self.stats.tokens_forwarded += sum(count for _, count in planned)

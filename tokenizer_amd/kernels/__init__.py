@@ -53,7 +53,7 @@ class Ops:
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual",
-                     "ta_argmax"):
+                     "ta_argmax", "ta_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     @staticmethod
@@ -384,6 +384,24 @@ class Ops:
         partial_i = torch.empty((n_rows, chunks), dtype=torch.int32, device=logits.device)
         self._check(self.lib.ta_argmax(_ptr(logits), _ptr(out), _ptr(partial_v), _ptr(partial_i), n_rows, vocab,
                                        chunks, self._stream()), "argmax")
+        return out
+
+
+    def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniform: torch.Tensor,
+               out: torch.Tensor | None = None) -> torch.Tensor:
+        """Temperature / nucleus draw per row with the reference's rules (tokens by falling logit, lower
+        index first among equals; the shortest prefix reaching top_p; the uniform number walks its mass).
+        logits float32 [B, V]; temperature (> 0), top_p, uniform: float32 [B]; returns int32 [B]."""
+        _dev(logits, temperature, top_p, uniform, out)
+        _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [B, V]")
+        n_rows = logits.shape[0]
+        for name, t in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
+            _need(t.dtype == torch.float32 and t.numel() == n_rows, f"{name} must be float32 [B]")
+        if out is None:
+            out = torch.empty(n_rows, dtype=torch.int32, device=logits.device)
+        _need(out.dtype == torch.int32 and out.numel() == n_rows, "sample output must be int32 [B]")
+        self._check(self.lib.ta_sample(_ptr(logits), _ptr(temperature), _ptr(top_p), _ptr(uniform), _ptr(out),
+                                       n_rows, logits.shape[1], self._stream()), "sample")
         return out
 
 
