@@ -278,3 +278,42 @@ def test_warm_requests_draw_on_the_device_as_they_would_alone(model_folders):
     other = generate(solo, prompts[0], GenerateParams(max_tokens=10, temperature=1.3, top_p=0.95, seed=6)).tokens
     assert again == results[rids[0]].tokens and other != again
     sched.assert_idle()
+
+
+REAL_SIZES = {
+    # Layer sizes of the three model sizes the benchmarks name, cut to two layers and a small vocabulary.
+    "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864),
+    "1.5b": dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960),
+    "7b": dict(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944),
+}
+
+
+@pytest.mark.parametrize("size", list(REAL_SIZES))
+def test_layers_of_real_sizes(tmp_path, size):
+    # The kernels at the widths, head sizes and group sizes of the real models: prompts in portions, decode
+    # steps alone and in a batch (fused and unfused kernels, captured graphs), against the plain implementation.
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    raw = dict(TINY["A"][0], num_hidden_layers=2, vocab_size=1000, max_position_embeddings=512,
+               tie_word_embeddings=(size != "7b"), **REAL_SIZES[size])
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 11, str(tmp_path / size))
+    cfg, tensors = plain.load_folder(folder)
+    reqs = {f"r{i}": random_ids(1000, n, 20 + i) for i, n in enumerate([150, 47, 80])}
+    want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (tt.mixed(reqs, 2), tt.decode_tail(reqs, 24)):
+            eng = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=4)
+            eng.pools.poison()
+            got = tt.run_in_process(eng, steps)
+            for rid in reqs:
+                close(got[rid], want[rid], dtype)
+    # A decode batch of 20 requests takes the kernels for more than 16 rows.
+    from tokenizer_amd.engine import StepEntry
+    eng = engine_for(folder, "bfloat16", max_tokens=64 * 20, max_requests=20)
+    prompts = [random_ids(1000, 30 + i, 40 + i) for i in range(20)]
+    for rid, ids in enumerate(prompts):
+        eng.add_request(rid)
+        eng.step([StepEntry(rid, ids[:-1], [])])
+    logits = eng.step([StepEntry(rid, ids[-1:], [0]) for rid, ids in enumerate(prompts)]).float().cpu()
+    for rid, ids in enumerate(prompts):
+        close(logits[rid:rid + 1], plain.all_logits(cfg, tensors, ids)[-1:], "bfloat16")
