@@ -42,6 +42,59 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
   }
 }
 
+// The same for rows of up to 4096 elements (a multiple of 4): every thread keeps its four-element pieces in
+// registers, so the row is read once, 16 bytes at a time.
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4(const bf16_t* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  return make_float4(bf16_bits_to_float(raw.x & 0xffffu), bf16_bits_to_float(raw.x >> 16),
+                     bf16_bits_to_float(raw.y & 0xffffu), bf16_bits_to_float(raw.y >> 16));
+}
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+  uint2 raw;
+  raw.x = (uint32_t)float_to_bf16_bits(v.x) | ((uint32_t)float_to_bf16_bits(v.y) << 16);
+  raw.y = (uint32_t)float_to_bf16_bits(v.z) | ((uint32_t)float_to_bf16_bits(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = raw;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta, const float* __restrict__ weight,
+                       T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps, int store_residual) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* res = residual + (size_t)r * hidden;
+  const T* del = delta ? delta + (size_t)r * hidden : nullptr;
+  float4 x[4];
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int h = (c * 256 + threadIdx.x) * 4;
+    x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (h < hidden) {
+      x[c] = ld4(res + h);
+      if (del) {
+        const float4 d = ld4(del + h);
+        x[c].x += d.x; x[c].y += d.y; x[c].z += d.z; x[c].w += d.w;
+      }
+      if (store_residual && del) st4(res + h, x[c]);
+    }
+    sq += x[c].x * x[c].x + x[c].y * x[c].y + x[c].z * x[c].z + x[c].w * x[c].w;
+  }
+  const float total = block_sum(sq, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int h = (c * 256 + threadIdx.x) * 4;
+    if (h >= hidden) continue;
+    const float4 w = ld4(weight + h);
+    st4(dst + h, make_float4(x[c].x * inv * w.x, x[c].y * inv * w.y, x[c].z * inv * w.z, x[c].w * inv * w.w));
+  }
+}
+
 // out[t, j] = silu(in[t, j]) * in[t, inner + j], silu(z) = z * sigmoid(z), in float.
 template <typename T>
 __global__ void silu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, int inner, size_t total) {
@@ -69,6 +122,15 @@ extern "C" int ta_add_rmsnorm(void* residual, const void* delta, const void* wei
                               const void* rows, int n_rows, int hidden, float eps, int store_residual,
                               int dtype, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (hidden % 4 == 0 && hidden <= 4096) {
+    if (dtype == DT_F32)
+      add_rmsnorm_vec_kernel<float><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)delta, (const float*)weight,
+                                                                (float*)out, (const int*)rows, hidden, eps, store_residual);
+    else
+      add_rmsnorm_vec_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((float*)residual, (const bf16_t*)delta, (const float*)weight,
+                                                                 (bf16_t*)out, (const int*)rows, hidden, eps, store_residual);
+    return LAUNCH_STATUS();
+  }
   if (dtype == DT_F32)
     add_rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)delta, (const float*)weight,
                                                           (float*)out, (const int*)rows, hidden, eps, store_residual);

@@ -35,7 +35,10 @@ __device__ __forceinline__ bf16x8 fz8() {
   return z;
 }
 
-template <int NW, int EPI, bool NORM>
+// R: weight rows per workgroup (16, 8 or 4).  With fewer than 16 the lanes of an MFMA row group load the
+// same rows again (same addresses, no extra traffic) and only the first R rows of the result are kept: small
+// matrices are spread over more workgroups that way, which is what a latency-bound launch needs.
+template <int NW, int EPI, bool NORM, int R>
 __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs p) {
   constexpr int SETS = (EPI == EPI_RESIDUAL) ? 1 : 2;
   __shared__ float red[NW][SETS * 4][WAVE];
@@ -50,27 +53,27 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   bool paired = true;
   int n_pair_tiles = 0;
   if (EPI == EPI_ROPE_STORE) {
-    const int half = p.d / 2, per_half = half / 16;
+    const int half = p.d / 2, per_half = half / R;
     n_pair_tiles = (p.n_q + p.n_kv) * per_half;
     if (tile < n_pair_tiles) {
       const int hd = tile / per_half, j = tile % per_half;
-      row0 = hd * p.d + j * 16;
+      row0 = hd * p.d + j * R;
       row1 = row0 + half;
     } else {
       paired = false;
-      row0 = (p.n_q + p.n_kv) * p.d + (tile - n_pair_tiles) * 16;
+      row0 = (p.n_q + p.n_kv) * p.d + (tile - n_pair_tiles) * R;
       row1 = row0;
     }
   } else if (EPI == EPI_GATED) {
-    row0 = tile * 16;
+    row0 = tile * R;
     row1 = row0 + p.n / 2;
   } else {
-    row0 = tile * 16;
+    row0 = tile * R;
   }
   const int n_limit = (EPI == EPI_GATED) ? p.n / 2 : p.n;
   // Rows past the end are clamped: they only feed outputs that are never stored.
-  const bf16_t* w0 = p.w + (size_t)min(row0 + col, n_limit - 1) * K + 8 * g;
-  const bf16_t* w1 = p.w + (size_t)min(row1 + col, p.n - 1) * K + 8 * g;
+  const bf16_t* w0 = p.w + (size_t)min(row0 + (col % R), n_limit - 1) * K + 8 * g;
+  const bf16_t* w1 = p.w + (size_t)min(row1 + (col % R), p.n - 1) * K + 8 * g;
   const int a_m = min(col, M - 1);
   const int full_steps = K / 32;
   constexpr int UN = 4;
@@ -96,7 +99,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   float pre_a[4] = {0.f, 0.f, 0.f, 0.f}, pre_b[4] = {0.f, 0.f, 0.f, 0.f};   // bias, or the old residual
   float pre_cos[4] = {1.f, 1.f, 1.f, 1.f}, pre_sin[4] = {0.f, 0.f, 0.f, 0.f};
   int pre_slot = -1;
-  if (wave == 0 && col < M) {
+  if (wave == 0 && col < M && 4 * g < R) {
     if (EPI == EPI_RESIDUAL) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -213,7 +216,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   if (threadIdx.x >= WAVE) return;
   // Lane (col, g): output column m = col, rows 4g .. 4g+3 of the tile.
   const int m = col;
-  if (m >= M) return;
+  if (m >= M || 4 * g >= R) return;
   float v0[4], v1[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -268,35 +271,43 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   }
 }
 
-template <int NW, int EPI, bool NORM>
+template <int NW, int EPI, bool NORM, int R>
 static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
   size_t lds = NORM ? (size_t)16 * (args.k + 8) * sizeof(uint16_t) : 0;
   if (lds > 48 * 1024) {
     // More dynamic LDS than the default limit: ask for it (the device has 160 KB per compute unit).
     if (lds > 140 * 1024) return -1;
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM>),
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM, R>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
   }
-  fused_decode_kernel<NW, EPI, NORM><<<tiles, NW * WAVE, lds, stream>>>(args);
+  fused_decode_kernel<NW, EPI, NORM, R><<<tiles, NW * WAVE, lds, stream>>>(args);
   return LAUNCH_STATUS();
 }
 
-template <int EPI, bool NORM>
-static int launch_fused(const FusedArgs& args, int tiles, hipStream_t stream) {
+// tiles16: the number of 16-row tiles; fewer rows per workgroup when there are few of them.
+template <int EPI, bool NORM, int R>
+static int launch_rows(const FusedArgs& args, int tiles, int waves, hipStream_t stream) {
   const int k_steps = (args.k + 31) / 32;
-  if (tiles >= 1024 || k_steps <= 8) return launch_one<4, EPI, NORM>(args, tiles, stream);
-  if (tiles >= 256 || k_steps <= 32 || NORM) return launch_one<8, EPI, NORM>(args, tiles, stream);
-  if constexpr (!NORM) return launch_one<16, EPI, false>(args, tiles, stream);
+  if (waves == 0) waves = (tiles >= 1024 || k_steps <= 8) ? 4 : (tiles >= 256 || k_steps <= 64 || NORM) ? 8 : 16;
+  if (waves == 4) return launch_one<4, EPI, NORM, R>(args, tiles, stream);
+  if (waves == 8 || NORM) return launch_one<8, EPI, NORM, R>(args, tiles, stream);
+  if constexpr (!NORM) return launch_one<16, EPI, false, R>(args, tiles, stream);
   return -1;
+}
+
+static int rows_per_tile(int tiles16, int rows_override) {
+  if (rows_override == 16 || rows_override == 8 || rows_override == 4) return rows_override;
+  return tiles16 >= 256 ? 16 : tiles16 >= 128 ? 8 : 4;
 }
 
 // q/k/v projection of up to 16 rows read from the float residual (normalised on the fly): bias, rotation,
 // q into `q_out` [m, n_q * d], keys and values into their pages (slots null or negative: not stored).
+// rows / waves: 0 = the launcher's choice of weight rows per workgroup and waves sharing a tile's K.
 extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_weight, float eps, const void* w,
                                       const void* bias, void* q_out, const void* positions, const void* cos_sin,
                                       const void* slots, void* k_pages, void* v_pages, int m, int k, int n_q,
-                                      int n_kv, int d, int page_size, hipStream_t stream) {
+                                      int n_kv, int d, int page_size, int rows, int waves, hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || (k & 7) || (d & 31)) return -1;
   FusedArgs a = {};
@@ -305,33 +316,39 @@ extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_wei
   a.out = (bf16_t*)q_out; a.ldc = n_q * d;
   a.positions = (const int*)positions; a.cos_sin = (const float*)cos_sin; a.slots = (const int*)slots;
   a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
-  const int tiles = (n_q + n_kv) * (d / 32) + n_kv * d / 16;
-  return launch_fused<EPI_ROPE_STORE, true>(a, tiles, stream);
+  const int r = rows_per_tile(a.n / 16, rows);
+  const int tiles = (n_q + n_kv) * (d / 2 / r) + n_kv * d / r;
+  if (r == 16) return launch_rows<EPI_ROPE_STORE, true, 16>(a, tiles, waves, stream);
+  if (r == 8) return launch_rows<EPI_ROPE_STORE, true, 8>(a, tiles, waves, stream);
+  return launch_rows<EPI_ROPE_STORE, true, 4>(a, tiles, waves, stream);
 }
 
 // out [m, n/2] = silu(x Wg^T) * (x Wu^T), x = the normalised residual rows, W = [Wg; Wu] of shape [n, k].
 extern "C" int ta_fused_norm_gated(const void* residual, const void* norm_weight, float eps, const void* w,
-                                   void* out, int m, int n, int k, hipStream_t stream) {
+                                   void* out, int m, int n, int k, int rows, int waves, hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || (k & 7) || (n & 1)) return -1;
   FusedArgs a = {};
   a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
-  return launch_fused<EPI_GATED, true>(a, (n / 2 + 15) / 16, stream);
+  const int r = rows_per_tile((n / 2 + 15) / 16, rows);
+  const int tiles = (n / 2 + r - 1) / r;
+  if (r == 16) return launch_rows<EPI_GATED, true, 16>(a, tiles, waves, stream);
+  if (r == 8) return launch_rows<EPI_GATED, true, 8>(a, tiles, waves, stream);
+  return launch_rows<EPI_GATED, true, 4>(a, tiles, waves, stream);
 }
 
-// residual [m, n] += x W^T (+ bias), x bfloat16 [m, k] with row stride lda.  `waves` (4, 8, 16; 0 = the
-// launcher's choice) lets a caller pick how many waves share a tile's K.
+// residual [m, n] += x W^T (+ bias), x bfloat16 [m, k] with row stride lda.
 extern "C" int ta_fused_linear_residual(const void* x, int lda, const void* w, const void* bias, void* residual,
-                                        int m, int n, int k, int waves, hipStream_t stream) {
+                                        int m, int n, int k, int rows, int waves, hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || (k & 7) || (lda & 7)) return -1;
   FusedArgs a = {};
   a.a = (const bf16_t*)x; a.lda = lda; a.w = (const bf16_t*)w; a.bias = (const float*)bias;
   a.m = m; a.n = n; a.k = k; a.residual_out = (float*)residual;
-  const int tiles = (n + 15) / 16;
-  if (waves == 4) return launch_one<4, EPI_RESIDUAL, false>(a, tiles, stream);
-  if (waves == 8) return launch_one<8, EPI_RESIDUAL, false>(a, tiles, stream);
-  if (waves == 16) return launch_one<16, EPI_RESIDUAL, false>(a, tiles, stream);
-  return launch_fused<EPI_RESIDUAL, false>(a, tiles, stream);
+  const int r = rows_per_tile((n + 15) / 16, rows);
+  const int tiles = (n + r - 1) / r;
+  if (r == 16) return launch_rows<EPI_RESIDUAL, false, 16>(a, tiles, waves, stream);
+  if (r == 8) return launch_rows<EPI_RESIDUAL, false, 8>(a, tiles, waves, stream);
+  return launch_rows<EPI_RESIDUAL, false, 4>(a, tiles, waves, stream);
 }

@@ -306,7 +306,8 @@ class Ops:
     # ------------------------------------------------------- fused decode products
     FUSED_ROWS = 16
     use_fused_decode = True
-    linear_add_waves = 0      # 0: the launcher picks how many waves share a tile's K
+    fused_rows = 0            # 0: the launcher picks the weight rows per workgroup (16, 8, 4) ...
+    fused_waves = 0           # ... and how many waves share a tile's K (4, 8, 16)
 
     def can_fuse_decode(self, rows: int, dtype: torch.dtype) -> bool:
         """Batches of few bfloat16 rows can run the products that take the norm, the rotation with the
@@ -338,7 +339,8 @@ class Ops:
         self._check(self.lib.ta_fused_norm_qkv_rope(
             _ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(weight), _ptr(bias), _ptr(q), _ptr(positions),
             _ptr(cos_sin), _ptr(slots), _ptr(k_pages if slots is not None else None),
-            _ptr(v_pages if slots is not None else None), m, k, n_q, n_kv, head_dim, page_size, self._stream()),
+            _ptr(v_pages if slots is not None else None), m, k, n_q, n_kv, head_dim, page_size,
+            self.fused_rows, self.fused_waves, self._stream()),
             "fused_norm_qkv_rope")
         return q
 
@@ -352,7 +354,8 @@ class Ops:
         _need(m <= self.FUSED_ROWS and k % 8 == 0, "sizes the fused product does not take")
         out = torch.empty((m, weight.shape[0] // 2), dtype=torch.bfloat16, device=residual.device)
         self._check(self.lib.ta_fused_norm_gated(_ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(weight),
-                                                 _ptr(out), m, weight.shape[0], k, self._stream()), "fused_norm_gated")
+                                                 _ptr(out), m, weight.shape[0], k, self.fused_rows, self.fused_waves,
+                                                 self._stream()), "fused_norm_gated")
         return out
 
     def linear_add(self, x, weight, bias, residual) -> None:
@@ -368,7 +371,7 @@ class Ops:
         if bias is not None:
             _need(bias.dtype == torch.float32 and bias.numel() == n, "bias must be float32 [N]")
         self._check(self.lib.ta_fused_linear_residual(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(residual), m, n, k,
-                                                      self.linear_add_waves, self._stream()), "linear_add")
+                                                      self.fused_rows, self.fused_waves, self._stream()), "linear_add")
 
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
