@@ -6,7 +6,8 @@ Flags, defaults and the lines printed are the reference's: the generated text on
 output; prompt ids, parameters, generated ids, the stop reason and the timings on standard
 error.  The model comes from a folder (config.json, model.safetensors, tokenizer.json and,
 if present, generation_config.json) instead of a download.  `--token-ids` takes the prompt as
-comma-separated ids for folders without a tokenizer.
+comma-separated ids for folders without a tokenizer; `--random-weights SEED` needs only the folder's
+config.json; `--dtype` is bf16 (default) or fp32; `--num-blocks` is the size of the page pool.
 """
 from __future__ import annotations
 
@@ -14,7 +15,7 @@ import os
 import sys
 import time
 
-USAGE = ("usage: qwen-infer --model DIR [--dtype bfloat16|float32] [--num-blocks N] [--max-tokens N] "
+USAGE = ("usage: qwen-infer --model DIR [--dtype bf16|fp32] [--num-blocks N] [--random-weights SEED] [--max-tokens N] "
          "[--temperature T] [--top-p P] [--seed N] [--stop STRING]... [--token-ids] <prompt>")
 
 
@@ -24,7 +25,8 @@ class ArgError(ValueError):
 
 def parse_args(argv: list[str]) -> dict:
     args = {"prompt": None, "max_tokens": 20, "temperature": 0.0, "top_p": 1.0, "seed": 0, "stop": [],
-            "model": None, "dtype": "bfloat16", "num_blocks": 256, "token_ids": False, "help": False}
+            "model": None, "dtype": "bfloat16", "num_blocks": 256, "token_ids": False, "help": False,
+            "random_weights": None}
     it = iter(argv)
 
     def value(flag: str) -> str:
@@ -65,6 +67,11 @@ def parse_args(argv: list[str]) -> dict:
                 args["num_blocks"] = int(value(arg))
             except ValueError:
                 raise ArgError("--num-blocks wants an integer") from None
+        elif arg == "--random-weights":
+            try:
+                args["random_weights"] = int(value(arg))
+            except ValueError:
+                raise ArgError("--random-weights wants an integer seed") from None
         elif arg == "--stop":
             args["stop"].append(value(arg))
         elif arg == "--model":
@@ -95,7 +102,9 @@ def main(argv: list[str] | None = None) -> int:
         print(USAGE, file=sys.stderr)
         return 1
 
-    from .engine import Engine, GenerateParams, StopReason, generate, load_eos_token_ids, load_model
+    from .config import load_config
+    from .engine import (Engine, GenerateParams, StopReason, generate, load_eos_token_ids, load_model,
+                         random_model)
     from .tokenizer import Tokenizer
 
     folder = args["model"]
@@ -119,7 +128,10 @@ def main(argv: list[str] | None = None) -> int:
     print(f"max_tokens {params.max_tokens} temperature {params.temperature} top_p {params.top_p} "
           f"seed {params.seed} eos {params.eos}", file=sys.stderr)
 
-    model = load_model(folder, args["dtype"])
+    if args["random_weights"] is not None:      # the folder then needs its config.json only
+        model = random_model(load_config(folder), args["random_weights"], args["dtype"])
+    else:
+        model = load_model(folder, args["dtype"])
     engine = Engine(model, num_pages=args["num_blocks"], max_requests=1)
     token_bytes = (lambda token: tokenizer.decode_bytes([token])) if tokenizer else \
         (lambda token: f"{token} ".encode())

@@ -23,6 +23,14 @@ def _next(engine, cursor: SampleCursor, logits, token_bytes, on_chunk):
     return cursor.push_token(token, token_bytes, on_chunk)
 
 
+def _engine_for(model_or_engine, prompt, params):
+    """`generate(model, ...)` as in the reference: a bare model gets an engine sized for this one request."""
+    if hasattr(model_or_engine, "step"):
+        return model_or_engine
+    from .engine import Engine
+    return Engine(model_or_engine, max_tokens=len(prompt) + params.max_tokens + 1, max_requests=1)
+
+
 def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes=_no_bytes,
                   on_chunk=_go_on) -> Generated:
     """Prefill `prompt`, then sample up to `params.max_tokens` ids, one cached forward per id.
@@ -33,6 +41,7 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
     """
     if not prompt:
         raise ValueError("prompt encoded to no tokens")
+    engine = _engine_for(engine, prompt, params)
     cursor = SampleCursor(params)
     rid = ("generate", id(cursor))
     engine.add_request(rid)

@@ -22,6 +22,9 @@ ARCH = "gfx950"
 # Packed float32 instructions are switched off for all device code.
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               # Matrix-core accumulators stay in ordinary registers: the softmax and the epilogues work on
+               # them with vector instructions, which cannot read the accumulation registers directly.
+               "-mllvm", "-amdgpu-mfma-vgpr-form=1",
                "-Wno-unused-command-line-argument"]
 
 
