@@ -45,7 +45,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int item = blockIdx.z;
   const int t = rows ? rows[item] : item;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int heads_here = min(16, group - hb * 16);
   const int head = kvh * group + hb * 16 + col;          // valid when col < heads_here

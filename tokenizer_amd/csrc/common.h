@@ -23,6 +23,12 @@ __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_bits_to_float
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
 
+// The index of a thread's wave within its workgroup, as a scalar: conditions built from it are uniform
+// branches.  Matrix instructions run whatever the lane mask says, so a matrix instruction must never sit
+// in a block that the compiler enters by masking lanes; a condition that only looks divergent (one derived
+// from threadIdx) can end up as exactly that.
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);

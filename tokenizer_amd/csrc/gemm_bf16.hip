@@ -23,7 +23,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
   // step k+1 are in flight during the products of step k.
   __shared__ __attribute__((aligned(16))) uint16_t a_s[2][BM * GB_LDS];
   __shared__ __attribute__((aligned(16))) uint16_t w_s[2][BN * GB_LDS];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   floatx16 acc[TMI][TNI];

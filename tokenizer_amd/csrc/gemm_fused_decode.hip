@@ -38,12 +38,16 @@ __device__ __forceinline__ bf16x8 fz8() {
 // R: weight rows per workgroup (16, 8 or 4).  With fewer than 16 the lanes of an MFMA row group load the
 // same rows again (same addresses, no extra traffic) and only the first R rows of the result are kept: small
 // matrices are spread over more workgroups that way, which is what a latency-bound launch needs.
-template <int NW, int EPI, bool NORM, int R>
+//
+// UN: steps of 32 along K that a wave requests at once.  ONE: the host has checked that a wave's whole share
+// of K is one such batch, so there is no loop and no second set of registers for the batch after: a small
+// matrix is over after one trip to memory instead of several.
+template <int NW, int EPI, bool NORM, int R, int UN = 4, bool ONE = false>
 __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs p) {
   constexpr int SETS = (EPI == EPI_RESIDUAL) ? 1 : 2;
   __shared__ float red[NW][SETS * 4][WAVE];
   extern __shared__ __attribute__((aligned(16))) uint16_t a_s[];   // NORM: 16 normalised rows of K + 8 bfloat16
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int M = p.m, K = p.k;
   const int tile = blockIdx.x;
@@ -75,8 +79,10 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   const bf16_t* w0 = p.w + (size_t)min(row0 + (col % R), n_limit - 1) * K + 8 * g;
   const bf16_t* w1 = p.w + (size_t)min(row1 + (col % R), p.n - 1) * K + 8 * g;
   const int a_m = min(col, M - 1);
+  // A load costs the memory pipeline by its active lanes: lanes whose weight row (col >= R) or input row
+  // (col >= M) only feeds results that are never stored load nothing and hold zeros.
+  const bool w_lane = col < R, a_lane = col < M;
   const int full_steps = K / 32;
-  constexpr int UN = 4;
   const int lds_stride = K + 8;
 
   // Weight fragments come from HBM and take longest; the first batch is requested before the prologue.
@@ -88,11 +94,25 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int step = min(step_of(base_pair, u), max(full_steps - 1, 0));   // clamped loads are not used
-      wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + step * 32);
-      if (SETS == 2) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + step * 32);
+      wf[u][0] = fz8();
+      if (SETS == 2) wf[u][SETS - 1] = fz8();
+      if (w_lane) {
+        wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + step * 32);
+        if (SETS == 2) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + step * 32);
+      }
     }
   };
   load_w(wave);
+  const bf16_t* ar = NORM ? nullptr : p.a + (size_t)a_m * p.lda + 8 * g;
+  bf16x8 af_one[ONE ? UN : 1];
+  if (ONE && !NORM) {                                      // the rows' fragments as well
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+    {
+      af_one[u] = fz8();
+      if (a_lane) af_one[u] = *reinterpret_cast<const bf16x8*>(ar + min(step_of(wave, u), max(full_steps - 1, 0)) * 32);
+    }
+  }
 
   // What the epilogue needs besides the sums is requested now as well (wave 0 writes the results;
   // lane (col, g) owns column m = col and rows 4g .. 4g+3 of the tile).
@@ -172,32 +192,42 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
     }
     __syncthreads();
   }
-  const bf16_t* ar = NORM ? nullptr : p.a + (size_t)a_m * p.lda + 8 * g;
   const uint16_t* as_row = a_s + (size_t)a_m * lds_stride + 8 * g;
   auto load_a = [&](int k) -> bf16x8 {
     if (NORM) return *reinterpret_cast<const bf16x8*>(as_row + k);
-    return *reinterpret_cast<const bf16x8*>(ar + k);
+    return a_lane ? *reinterpret_cast<const bf16x8*>(ar + k) : fz8();
   };
 
   floatx4 acc[SETS];
 #pragma unroll
   for (int s = 0; s < SETS; ++s) acc[s] = (floatx4){0.f, 0.f, 0.f, 0.f};
   // Batches of UN steps; the next batch's weights are requested before the current one is multiplied.
-  for (int pair = wave; pair * 2 < full_steps; pair += (UN / 2) * NW) {
-    bf16x8 wc[UN][SETS], af[UN];
+  if constexpr (ONE) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      wc[u][0] = wf[u][0];
-      if (SETS == 2) wc[u][SETS - 1] = wf[u][SETS - 1];
-      af[u] = load_a(min(step_of(pair, u), full_steps - 1) * 32);
-    }
-    if ((pair + (UN / 2) * NW) * 2 < full_steps) load_w(pair + (UN / 2) * NW);
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      if (step_of(pair, u) >= full_steps) continue;
+      if (step_of(wave, u) >= full_steps) continue;
+      const bf16x8 af = NORM ? load_a(step_of(wave, u) * 32) : af_one[u];
 #pragma unroll
       for (int s = 0; s < SETS; ++s)
-        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][s], af[u], acc[s], 0, 0, 0);
+        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][s], af, acc[s], 0, 0, 0);
+    }
+  } else {
+    for (int pair = wave; pair * 2 < full_steps; pair += (UN / 2) * NW) {
+      bf16x8 wc[UN][SETS], af[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        wc[u][0] = wf[u][0];
+        if (SETS == 2) wc[u][SETS - 1] = wf[u][SETS - 1];
+        af[u] = load_a(min(step_of(pair, u), full_steps - 1) * 32);
+      }
+      if ((pair + (UN / 2) * NW) * 2 < full_steps) load_w(pair + (UN / 2) * NW);
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        if (step_of(pair, u) >= full_steps) continue;
+#pragma unroll
+        for (int s = 0; s < SETS; ++s)
+          acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][s], af[u], acc[s], 0, 0, 0);
+      }
     }
   }
   if ((K & 31) && wave == 0) {                             // tail of K (a multiple of 8): zero-filled
@@ -271,18 +301,32 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   }
 }
 
-template <int NW, int EPI, bool NORM, int R>
-static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
+template <int NW, int EPI, bool NORM, int R, int UN, bool ONE>
+static int launch_kernel(const FusedArgs& args, int tiles, hipStream_t stream) {
   size_t lds = NORM ? (size_t)16 * (args.k + 8) * sizeof(uint16_t) : 0;
   if (lds > 48 * 1024) {
     // More dynamic LDS than the default limit: ask for it (the device has 160 KB per compute unit).
     if (lds > 140 * 1024) return -1;
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM, R>),
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM, R, UN, ONE>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
   }
-  fused_decode_kernel<NW, EPI, NORM, R><<<tiles, NW * WAVE, lds, stream>>>(args);
+  fused_decode_kernel<NW, EPI, NORM, R, UN, ONE><<<tiles, NW * WAVE, lds, stream>>>(args);
   return LAUNCH_STATUS();
+}
+
+template <int NW, int EPI, bool NORM, int R>
+static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
+  // Steps of a wave: pairs of steps are dealt round-robin to the waves.
+  const int pairs = (args.k / 32 + 1) / 2;
+  const int steps_per_wave = 2 * ((pairs + NW - 1) / NW);
+  if (steps_per_wave <= 4) return launch_kernel<NW, EPI, NORM, R, 4, true>(args, tiles, stream);
+  if constexpr (!NORM) {
+    // Rows from memory: one trip for a wave's whole share if it fits the registers (128 a lane at 16 waves).
+    if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, R, 8, true>(args, tiles, stream);
+    if (steps_per_wave <= 10) return launch_kernel<NW, EPI, NORM, R, 10, true>(args, tiles, stream);
+  }
+  return launch_kernel<NW, EPI, NORM, R, 4, false>(args, tiles, stream);
 }
 
 // tiles16: the number of 16-row tiles; fewer rows per workgroup when there are few of them.

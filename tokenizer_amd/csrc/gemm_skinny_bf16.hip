@@ -35,7 +35,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
                    const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K) {
   constexpr int SETS = GATED ? 2 : 1;
   __shared__ float red[NW][SETS * MB * 4][WAVE];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int n_out = GATED ? N / 2 : N;
   const int n0 = blockIdx.x * 16;
