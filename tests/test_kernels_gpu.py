@@ -450,3 +450,29 @@ def test_sampling_kernel_follows_the_reference_rules(ops, ref):
     assert ops.sample(flat, ones, ones, torch.arange(8).cuda() / 8 + 0.01).cpu().tolist() == list(range(8))
     # All -inf: nothing to weigh, the first index, as the greedy scan gives.
     assert ops.sample(torch.full((1, 50), float("-inf")).cuda(), ones[:1], ones[:1], us[:1]).item() == 0
+
+
+@pytest.mark.parametrize("rows", [1, 3, 4, 7, 16, 19, 32])
+@pytest.mark.parametrize("waves", [0, 4, 8, 16])
+def test_fused_products_for_every_cut(ops, ref, rows, waves):
+    """Weight rows per workgroup (one or two blocks of up to sixteen, the last one partly filled) and waves per
+    workgroup are the launcher's choice; every choice gives the same numbers.  Sizes chosen so that waves
+    are left without a step, K has a tail, and the last workgroup reaches past the matrix."""
+    m, inner, hidden = 7, 328, 104
+    residual = rand((m, hidden), torch.float32, 60, 2.0)
+    norm_w = rand((hidden,), torch.float32, 61) * 0.1 + 1
+    w = rand((2 * inner, hidden), torch.bfloat16, 62, 0.1)
+    down = rand((hidden, inner), torch.bfloat16, 63, 0.05)
+    bias = rand((hidden,), torch.float32, 64)
+    ops.fused_rows, ops.fused_waves = rows, waves
+    try:
+        got = ops.fused_norm_gated(residual, norm_w, 1e-5, w)
+        res_a = residual.clone()
+        ops.linear_add(got, down, bias, res_a)
+    finally:
+        ops.fused_rows, ops.fused_waves = 0, 0
+    want = ref.fused_norm_gated(residual, norm_w, 1e-5, w)
+    torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    res_b = residual.clone()
+    ref.linear_add(got, down, bias, res_b)
+    torch.testing.assert_close(res_a, res_b, **linear_tol(torch.float32, got, down))

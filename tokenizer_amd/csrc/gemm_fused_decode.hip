@@ -26,6 +26,7 @@ struct FusedArgs {
   // EPI_ROPE_STORE
   const int* positions; const float* cos_sin; const int* slots;
   bf16_t* k_pages; bf16_t* v_pages; int n_q, n_kv, d, page_size;
+  int rows;                                                // weight rows per workgroup
 };
 
 __device__ __forceinline__ bf16x8 fz8() {
@@ -35,30 +36,32 @@ __device__ __forceinline__ bf16x8 fz8() {
   return z;
 }
 
-// R: weight rows per workgroup (16, 8 or 4).  With fewer than 16 the lanes of an MFMA row group load the
-// same rows again (same addresses, no extra traffic) and only the first R rows of the result are kept: small
-// matrices are spread over more workgroups that way, which is what a latency-bound launch needs.
+// A workgroup owns `p.rows` weight rows (output columns), in PASSES blocks of up to sixteen: the M side of the
+// MFMA.  Lanes whose weight row or input row only feeds results that are never stored load nothing: a
+// load costs the memory pipeline by its active lanes.  So a small matrix is spread thinly over many
+// workgroups (4 rows each), and a large one is cut so that every compute unit streams the same share.
 //
 // UN: steps of 32 along K that a wave requests at once.  ONE: the host has checked that a wave's whole share
-// of K is one such batch, so there is no loop and no second set of registers for the batch after: a small
-// matrix is over after one trip to memory instead of several.
-template <int NW, int EPI, bool NORM, int R, int UN = 4, bool ONE = false>
+// of K is one such batch, so there is no loop, the batches of all passes are requested at the start, and a
+// small matrix is over after one trip to memory instead of several.
+template <int NW, int EPI, bool NORM, int UN, bool ONE, int PASSES>
 __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs p) {
   constexpr int SETS = (EPI == EPI_RESIDUAL) ? 1 : 2;
+  constexpr int HELD = ONE ? PASSES : 1;                     // batches of weights held at once
+  static_assert(EPI != EPI_ROPE_STORE || PASSES == 1, "the rotation pairs rows within one block");
   __shared__ float red[NW][SETS * 4][WAVE];
   extern __shared__ __attribute__((aligned(16))) uint16_t a_s[];   // NORM: 16 normalised rows of K + 8 bfloat16
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
-  const int M = p.m, K = p.k;
+  const int M = p.m, K = p.k, R = p.rows;
   const int tile = blockIdx.x;
 
-  // Which weight rows this workgroup owns: `row0` (+ `row1` for the second set).
+  // Which weight rows this workgroup owns: `row0` onwards (+ `row1` onwards for the second set).
   int row0, row1 = 0;
   bool paired = true;
-  int n_pair_tiles = 0;
   if (EPI == EPI_ROPE_STORE) {
     const int half = p.d / 2, per_half = half / R;
-    n_pair_tiles = (p.n_q + p.n_kv) * per_half;
+    const int n_pair_tiles = (p.n_q + p.n_kv) * per_half;
     if (tile < n_pair_tiles) {
       const int hd = tile / per_half, j = tile % per_half;
       row0 = hd * p.d + j * R;
@@ -75,13 +78,18 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
     row0 = tile * R;
   }
   const int n_limit = (EPI == EPI_GATED) ? p.n / 2 : p.n;
-  // Rows past the end are clamped: they only feed outputs that are never stored.
-  const bf16_t* w0 = p.w + (size_t)min(row0 + (col % R), n_limit - 1) * K + 8 * g;
-  const bf16_t* w1 = p.w + (size_t)min(row1 + (col % R), p.n - 1) * K + 8 * g;
+  const bf16_t* w0[PASSES];
+  const bf16_t* w1[PASSES];
+  bool w_lane[PASSES];
+#pragma unroll
+  for (int ps = 0; ps < PASSES; ++ps) {
+    const int r = 16 * ps + col;
+    w_lane[ps] = r < R && row0 + r < n_limit;
+    w0[ps] = p.w + (size_t)min(row0 + r, n_limit - 1) * K + 8 * g;
+    w1[ps] = p.w + (size_t)min(row1 + r, p.n - 1) * K + 8 * g;
+  }
+  const bool a_lane = col < M;
   const int a_m = min(col, M - 1);
-  // A load costs the memory pipeline by its active lanes: lanes whose weight row (col >= R) or input row
-  // (col >= M) only feeds results that are never stored load nothing and hold zeros.
-  const bool w_lane = col < R, a_lane = col < M;
   const int full_steps = K / 32;
   const int lds_stride = K + 8;
 
@@ -89,48 +97,57 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   // Step j of a wave's batch: steps come in pairs (128 contiguous bytes of a weight row, one cache line),
   // pair q of the batch starting at pair `base` is pair base + q * NW.
   auto step_of = [&](int base_pair, int u) { return (base_pair + (u >> 1) * NW) * 2 + (u & 1); };
-  bf16x8 wf[UN][SETS];
-  auto load_w = [&](int base_pair) {
+  bf16x8 wf[HELD][UN][SETS];
+  auto load_w = [&](int held, int ps, int base_pair) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int step = min(step_of(base_pair, u), max(full_steps - 1, 0));   // clamped loads are not used
-      wf[u][0] = fz8();
-      if (SETS == 2) wf[u][SETS - 1] = fz8();
-      if (w_lane) {
-        wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + step * 32);
-        if (SETS == 2) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + step * 32);
+      wf[held][u][0] = fz8();
+      if (SETS == 2) wf[held][u][SETS - 1] = fz8();
+      if (w_lane[ps]) {
+        wf[held][u][0] = *reinterpret_cast<const bf16x8*>(w0[ps] + step * 32);
+        if (SETS == 2) wf[held][u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1[ps] + step * 32);
       }
     }
   };
-  load_w(wave);
+  load_w(0, 0, wave);
+  if (ONE) {
+#pragma unroll
+    for (int ps = 1; ps < PASSES; ++ps) load_w(HELD - PASSES + ps, ps, wave);
+  }
   const bf16_t* ar = NORM ? nullptr : p.a + (size_t)a_m * p.lda + 8 * g;
   bf16x8 af_one[ONE ? UN : 1];
   if (ONE && !NORM) {                                      // the rows' fragments as well
 #pragma unroll
-    for (int u = 0; u < UN; ++u)
-    {
+    for (int u = 0; u < UN; ++u) {
       af_one[u] = fz8();
       if (a_lane) af_one[u] = *reinterpret_cast<const bf16x8*>(ar + min(step_of(wave, u), max(full_steps - 1, 0)) * 32);
     }
   }
 
   // What the epilogue needs besides the sums is requested now as well (wave 0 writes the results;
-  // lane (col, g) owns column m = col and rows 4g .. 4g+3 of the tile).
-  float pre_a[4] = {0.f, 0.f, 0.f, 0.f}, pre_b[4] = {0.f, 0.f, 0.f, 0.f};   // bias, or the old residual
+  // lane (col, g) owns column m = col and rows 4g .. 4g+3 of each block).
+  float pre_a[PASSES][4], pre_b[4] = {0.f, 0.f, 0.f, 0.f};     // bias, or the old residual
   float pre_cos[4] = {1.f, 1.f, 1.f, 1.f}, pre_sin[4] = {0.f, 0.f, 0.f, 0.f};
   int pre_slot = -1;
-  if (wave == 0 && col < M && 4 * g < R) {
+#pragma unroll
+  for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) pre_a[ps][r] = 0.f;
+  if (wave == 0 && col < M) {
     if (EPI == EPI_RESIDUAL) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = row0 + 4 * g + r;
-        if (n < p.n) pre_a[r] = p.residual_out[(size_t)col * p.n + n] + (p.bias ? p.bias[n] : 0.f);
-      }
-    } else if (EPI == EPI_ROPE_STORE) {
+      for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int local = 16 * ps + 4 * g + r, n = row0 + local;
+          if (local < R && n < p.n) pre_a[ps][r] = p.residual_out[(size_t)col * p.n + n] + (p.bias ? p.bias[n] : 0.f);
+        }
+    } else if (EPI == EPI_ROPE_STORE && 4 * g < R) {
       pre_slot = p.slots ? p.slots[col] : -1;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        if (p.bias) { pre_a[r] = p.bias[row0 + 4 * g + r]; pre_b[r] = p.bias[row1 + 4 * g + r]; }
+        if (p.bias) { pre_a[0][r] = p.bias[row0 + 4 * g + r]; pre_b[r] = p.bias[row1 + 4 * g + r]; }
         if (paired && p.cos_sin) {
           const float* cs = p.cos_sin + (size_t)p.positions[col] * p.d;
           const int i = row0 % p.d + 4 * g + r;
@@ -198,156 +215,194 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
     return a_lane ? *reinterpret_cast<const bf16x8*>(ar + k) : fz8();
   };
 
-  floatx4 acc[SETS];
 #pragma unroll
-  for (int s = 0; s < SETS; ++s) acc[s] = (floatx4){0.f, 0.f, 0.f, 0.f};
-  // Batches of UN steps; the next batch's weights are requested before the current one is multiplied.
-  if constexpr (ONE) {
+  for (int ps = 0; ps < PASSES; ++ps) {
+    floatx4 acc[SETS];
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      if (step_of(wave, u) >= full_steps) continue;
-      const bf16x8 af = NORM ? load_a(step_of(wave, u) * 32) : af_one[u];
-#pragma unroll
-      for (int s = 0; s < SETS; ++s)
-        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][s], af, acc[s], 0, 0, 0);
-    }
-  } else {
-    for (int pair = wave; pair * 2 < full_steps; pair += (UN / 2) * NW) {
-      bf16x8 wc[UN][SETS], af[UN];
+    for (int s = 0; s < SETS; ++s) acc[s] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    if constexpr (ONE) {
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        wc[u][0] = wf[u][0];
-        if (SETS == 2) wc[u][SETS - 1] = wf[u][SETS - 1];
-        af[u] = load_a(min(step_of(pair, u), full_steps - 1) * 32);
-      }
-      if ((pair + (UN / 2) * NW) * 2 < full_steps) load_w(pair + (UN / 2) * NW);
-#pragma unroll
-      for (int u = 0; u < UN; ++u) {
-        if (step_of(pair, u) >= full_steps) continue;
+        if (step_of(wave, u) >= full_steps) continue;
+        const bf16x8 af = NORM ? load_a(step_of(wave, u) * 32) : af_one[u];
 #pragma unroll
         for (int s = 0; s < SETS; ++s)
-          acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][s], af[u], acc[s], 0, 0, 0);
+          acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[HELD - PASSES + ps][u][s], af, acc[s], 0, 0, 0);
       }
+    } else {
+      // Batches of UN steps; the next batch's weights are requested before the current one is multiplied.
+      for (int pair = wave; pair * 2 < full_steps; pair += (UN / 2) * NW) {
+        bf16x8 wc[UN][SETS], af[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          wc[u][0] = wf[0][u][0];
+          if (SETS == 2) wc[u][SETS - 1] = wf[0][u][SETS - 1];
+          af[u] = load_a(min(step_of(pair, u), full_steps - 1) * 32);
+        }
+        if ((pair + (UN / 2) * NW) * 2 < full_steps) load_w(0, ps, pair + (UN / 2) * NW);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          if (step_of(pair, u) >= full_steps) continue;
+#pragma unroll
+          for (int s = 0; s < SETS; ++s)
+            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][s], af[u], acc[s], 0, 0, 0);
+        }
+      }
+      if (ps + 1 < PASSES) load_w(0, ps + 1, wave);          // the next block's first batch, before this one's sums
     }
-  }
-  if ((K & 31) && wave == 0) {                             // tail of K (a multiple of 8): zero-filled
-    const int k = full_steps * 32;
-    const bool ok = k + 8 * g < K;
-    const bf16x8 af = ok ? load_a(k) : fz8();
-    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w0 + k) : fz8(), af, acc[0], 0, 0, 0);
-    if (SETS == 2)
-      acc[SETS - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w1 + k) : fz8(), af, acc[SETS - 1], 0, 0, 0);
-  }
-#pragma unroll
-  for (int s = 0; s < SETS; ++s)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][s * 4 + r][lane] = acc[s][r];
-  __syncthreads();
-  if (threadIdx.x >= WAVE) return;
-  // Lane (col, g): output column m = col, rows 4g .. 4g+3 of the tile.
-  const int m = col;
-  if (m >= M || 4 * g >= R) return;
-  float v0[4], v1[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      s0 += red[w][r][lane];
-      if (SETS == 2) s1 += red[w][4 + r][lane];
+    if ((K & 31) && wave == 0) {                             // tail of K (a multiple of 8): zero-filled
+      const int k = full_steps * 32;
+      const bool ok = k + 8 * g < K;
+      const bf16x8 af = ok ? load_a(k) : fz8();
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w0[ps] + k) : fz8(), af, acc[0], 0, 0, 0);
+      if (SETS == 2)
+        acc[SETS - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w1[ps] + k) : fz8(), af, acc[SETS - 1], 0, 0, 0);
     }
-    v0[r] = s0;
-    v1[r] = s1;
-  }
-  if (EPI == EPI_RESIDUAL) {
-    const int n = row0 + 4 * g;
-    float* dst = p.residual_out + (size_t)m * p.n + n;
+    if (ps > 0) __syncthreads();                             // wave 0 has read the block before
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (n + r < p.n) dst[r] = pre_a[r] + v0[r];            // old residual (+ bias) was fetched at the start
-  } else if (EPI == EPI_GATED) {
-    const int n = row0 + 4 * g;
-    bf16_t* dst = p.out + (size_t)m * p.ldc + n;
+    for (int s = 0; s < SETS; ++s)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (n + r < n_limit) st(dst + r, v0[r] / (1.0f + __expf(-v0[r])) * v1[r]);
-  } else {
-    const int d = p.d, half = d / 2;
-    const int slot = pre_slot;
-    const int page = slot >= 0 ? slot / p.page_size : 0, off = slot >= 0 ? slot % p.page_size : 0;
-    if (paired) {
-      const int hd = row0 / d, i = row0 % d + 4 * g;            // element i (< half) of head hd, and i + half
-      float r1[4], r2[4];
+      for (int r = 0; r < 4; ++r) red[wave][s * 4 + r][lane] = acc[s][r];
+    __syncthreads();
+    // Lane (col, g) of wave 0: output column m = col, rows 4g .. 4g+3 of the block.
+    const int m = col;
+    if (wave == 0 && m < M && 16 * ps + 4 * g < R) {
+      float v0[4], v1[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float x1 = v0[r] + pre_a[r], x2 = v1[r] + pre_b[r];
-        r1[r] = x1 * pre_cos[r] - x2 * pre_sin[r];              // cos 1, sin 0 without a rotation
-        r2[r] = x2 * pre_cos[r] + x1 * pre_sin[r];
-      }
-      bf16_t* dst = nullptr;
-      if (hd < p.n_q) dst = p.out + (size_t)m * p.ldc + (size_t)hd * d + i;
-      else if (slot >= 0) dst = p.k_pages + (((size_t)page * p.n_kv + (hd - p.n_q)) * p.page_size + off) * d + i;
-      if (dst) {
+        float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) { st(dst + r, r1[r]); st(dst + half + r, r2[r]); }
+        for (int w = 0; w < NW; ++w) {
+          s0 += red[w][r][lane];
+          if (SETS == 2) s1 += red[w][4 + r][lane];
+        }
+        v0[r] = s0;
+        v1[r] = s1;
       }
-    } else if (slot >= 0) {
-      const int e = row0 - (p.n_q + p.n_kv) * d + 4 * g;        // element of the joined value heads
-      const int kvh = e / d, dd = e % d;
-      bf16_t* dst = p.v_pages + (((size_t)page * p.n_kv + kvh) * d + dd) * p.page_size + off;
+      const int local = 16 * ps + 4 * g;                      // first of this lane's rows within the workgroup's
+      if (EPI == EPI_RESIDUAL) {
+        const int n = row0 + local;
+        float* dst = p.residual_out + (size_t)m * p.n + n;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) st(dst + (size_t)r * p.page_size, v0[r] + pre_a[r]);
+        for (int r = 0; r < 4; ++r)
+          if (local + r < R && n + r < p.n) dst[r] = pre_a[ps][r] + v0[r];   // old residual (+ bias) from the start
+      } else if (EPI == EPI_GATED) {
+        const int n = row0 + local;
+        bf16_t* dst = p.out + (size_t)m * p.ldc + n;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (local + r < R && n + r < n_limit) st(dst + r, v0[r] / (1.0f + __expf(-v0[r])) * v1[r]);
+      } else {
+        const int d = p.d, half = d / 2;
+        const int slot = pre_slot;
+        const int page = slot >= 0 ? slot / p.page_size : 0, off = slot >= 0 ? slot % p.page_size : 0;
+        if (paired) {
+          const int hd = row0 / d, i = row0 % d + 4 * g;            // element i (< half) of head hd, and i + half
+          float r1[4], r2[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float x1 = v0[r] + pre_a[0][r], x2 = v1[r] + pre_b[r];
+            r1[r] = x1 * pre_cos[r] - x2 * pre_sin[r];              // cos 1, sin 0 without a rotation
+            r2[r] = x2 * pre_cos[r] + x1 * pre_sin[r];
+          }
+          bf16_t* dst = nullptr;
+          if (hd < p.n_q) dst = p.out + (size_t)m * p.ldc + (size_t)hd * d + i;
+          else if (slot >= 0) dst = p.k_pages + (((size_t)page * p.n_kv + (hd - p.n_q)) * p.page_size + off) * d + i;
+          if (dst) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { st(dst + r, r1[r]); st(dst + half + r, r2[r]); }
+          }
+        } else if (slot >= 0) {
+          const int e = row0 - (p.n_q + p.n_kv) * d + 4 * g;        // element of the joined value heads
+          const int kvh = e / d, dd = e % d;
+          bf16_t* dst = p.v_pages + (((size_t)page * p.n_kv + kvh) * d + dd) * p.page_size + off;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) st(dst + (size_t)r * p.page_size, v0[r] + pre_a[0][r]);
+        }
+      }
     }
   }
 }
 
-template <int NW, int EPI, bool NORM, int R, int UN, bool ONE>
+template <int NW, int EPI, bool NORM, int UN, bool ONE, int PASSES>
 static int launch_kernel(const FusedArgs& args, int tiles, hipStream_t stream) {
   size_t lds = NORM ? (size_t)16 * (args.k + 8) * sizeof(uint16_t) : 0;
   if (lds > 48 * 1024) {
     // More dynamic LDS than the default limit: ask for it (the device has 160 KB per compute unit).
     if (lds > 140 * 1024) return -1;
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM, R, UN, ONE>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t err = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&fused_decode_kernel<NW, EPI, NORM, UN, ONE, PASSES>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
   }
-  fused_decode_kernel<NW, EPI, NORM, R, UN, ONE><<<tiles, NW * WAVE, lds, stream>>>(args);
+  fused_decode_kernel<NW, EPI, NORM, UN, ONE, PASSES><<<tiles, NW * WAVE, lds, stream>>>(args);
   return LAUNCH_STATUS();
 }
 
-template <int NW, int EPI, bool NORM, int R>
+template <int NW, int EPI, bool NORM, int PASSES>
 static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
   // Steps of a wave: pairs of steps are dealt round-robin to the waves.
   const int pairs = (args.k / 32 + 1) / 2;
   const int steps_per_wave = 2 * ((pairs + NW - 1) / NW);
-  if (steps_per_wave <= 4) return launch_kernel<NW, EPI, NORM, R, 4, true>(args, tiles, stream);
-  if constexpr (!NORM) {
+  if (steps_per_wave <= 4) return launch_kernel<NW, EPI, NORM, 4, true, PASSES>(args, tiles, stream);
+  if constexpr (!NORM && PASSES == 1) {
     // Rows from memory: one trip for a wave's whole share if it fits the registers (128 a lane at 16 waves).
-    if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, R, 8, true>(args, tiles, stream);
-    if (steps_per_wave <= 10) return launch_kernel<NW, EPI, NORM, R, 10, true>(args, tiles, stream);
+    if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, 8, true, 1>(args, tiles, stream);
+    if (steps_per_wave <= 10) return launch_kernel<NW, EPI, NORM, 10, true, 1>(args, tiles, stream);
   }
-  return launch_kernel<NW, EPI, NORM, R, 4, false>(args, tiles, stream);
+  return launch_kernel<NW, EPI, NORM, 4, false, PASSES>(args, tiles, stream);
 }
 
-// tiles16: the number of 16-row tiles; fewer rows per workgroup when there are few of them.
-template <int EPI, bool NORM, int R>
+// waves 0: the launcher's choice of how many waves share a workgroup's K.
+template <int EPI, bool NORM>
 static int launch_rows(const FusedArgs& args, int tiles, int waves, hipStream_t stream) {
   const int k_steps = (args.k + 31) / 32;
-  if (waves == 0) waves = (tiles >= 1024 || k_steps <= 8) ? 4 : (tiles >= 256 || k_steps <= 64 || NORM) ? 8 : 16;
-  if (waves == 4) return launch_one<4, EPI, NORM, R>(args, tiles, stream);
-  if (waves == 8 || NORM) return launch_one<8, EPI, NORM, R>(args, tiles, stream);
-  if constexpr (!NORM) return launch_one<16, EPI, false, R>(args, tiles, stream);
+  const bool two = args.rows > 16;
+  if (waves == 0) waves = (tiles >= 1024 || k_steps <= 8) ? 4 : (tiles >= 256 || k_steps <= 64 || NORM || two) ? 8 : 16;
+  if constexpr (EPI != EPI_ROPE_STORE) {
+    if (two) {
+      if (waves == 4) return launch_one<4, EPI, NORM, 2>(args, tiles, stream);
+      return launch_one<8, EPI, NORM, 2>(args, tiles, stream);
+    }
+  }
+  if (waves == 4) return launch_one<4, EPI, NORM, 1>(args, tiles, stream);
+  if (waves == 8 || NORM) return launch_one<8, EPI, NORM, 1>(args, tiles, stream);
+  if constexpr (!NORM) return launch_one<16, EPI, false, 1>(args, tiles, stream);
   return -1;
 }
 
+static int compute_units() {
+  static int count = 0;                                     // the same on every device of a machine
+  if (count == 0) {
+    int device = 0, value = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0)
+      count = value;
+    else
+      count = 256;
+  }
+  return count;
+}
+
+// Weight rows per workgroup for the rotation epilogue, where a block pairs rows half a head apart: 16, 8 or 4.
 static int rows_per_tile(int tiles16, int rows_override) {
   if (rows_override == 16 || rows_override == 8 || rows_override == 4) return rows_override;
   return tiles16 >= 256 ? 16 : tiles16 >= 128 ? 8 : 4;
 }
 
+// Weight rows per workgroup elsewhere: the matrix is cut into a multiple of the compute units' number of
+// equal shares of at most 32 rows, so that every unit streams the same number of bytes; never fewer than 4.
+static int rows_per_workgroup(int n_rows, int rows_override) {
+  if (rows_override >= 1 && rows_override <= 32) return rows_override;
+  const int units = compute_units();
+  const int rounds = (n_rows + units * 32 - 1) / (units * 32);
+  const int rows = (n_rows + units * rounds - 1) / (units * rounds);
+  return rows < 4 ? 4 : rows;
+}
+
 // q/k/v projection of up to 16 rows read from the float residual (normalised on the fly): bias, rotation,
 // q into `q_out` [m, n_q * d], keys and values into their pages (slots null or negative: not stored).
-// rows / waves: 0 = the launcher's choice of weight rows per workgroup and waves sharing a tile's K.
+// rows / waves: 0 = the launcher's choice of weight rows per workgroup and waves sharing a workgroup's K.
 extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_weight, float eps, const void* w,
                                       const void* bias, void* q_out, const void* positions, const void* cos_sin,
                                       const void* slots, void* k_pages, void* v_pages, int m, int k, int n_q,
@@ -360,11 +415,9 @@ extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_wei
   a.out = (bf16_t*)q_out; a.ldc = n_q * d;
   a.positions = (const int*)positions; a.cos_sin = (const float*)cos_sin; a.slots = (const int*)slots;
   a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
-  const int r = rows_per_tile(a.n / 16, rows);
-  const int tiles = (n_q + n_kv) * (d / 2 / r) + n_kv * d / r;
-  if (r == 16) return launch_rows<EPI_ROPE_STORE, true, 16>(a, tiles, waves, stream);
-  if (r == 8) return launch_rows<EPI_ROPE_STORE, true, 8>(a, tiles, waves, stream);
-  return launch_rows<EPI_ROPE_STORE, true, 4>(a, tiles, waves, stream);
+  a.rows = rows_per_tile(a.n / 16, rows);
+  const int tiles = (n_q + n_kv) * (d / 2 / a.rows) + n_kv * d / a.rows;
+  return launch_rows<EPI_ROPE_STORE, true>(a, tiles, waves, stream);
 }
 
 // out [m, n/2] = silu(x Wg^T) * (x Wu^T), x = the normalised residual rows, W = [Wg; Wu] of shape [n, k].
@@ -375,11 +428,8 @@ extern "C" int ta_fused_norm_gated(const void* residual, const void* norm_weight
   FusedArgs a = {};
   a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
-  const int r = rows_per_tile((n / 2 + 15) / 16, rows);
-  const int tiles = (n / 2 + r - 1) / r;
-  if (r == 16) return launch_rows<EPI_GATED, true, 16>(a, tiles, waves, stream);
-  if (r == 8) return launch_rows<EPI_GATED, true, 8>(a, tiles, waves, stream);
-  return launch_rows<EPI_GATED, true, 4>(a, tiles, waves, stream);
+  a.rows = rows_per_workgroup(n / 2, rows);
+  return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
 }
 
 // residual [m, n] += x W^T (+ bias), x bfloat16 [m, k] with row stride lda.
@@ -390,9 +440,6 @@ extern "C" int ta_fused_linear_residual(const void* x, int lda, const void* w, c
   FusedArgs a = {};
   a.a = (const bf16_t*)x; a.lda = lda; a.w = (const bf16_t*)w; a.bias = (const float*)bias;
   a.m = m; a.n = n; a.k = k; a.residual_out = (float*)residual;
-  const int r = rows_per_tile((n + 15) / 16, rows);
-  const int tiles = (n + r - 1) / r;
-  if (r == 16) return launch_rows<EPI_RESIDUAL, false, 16>(a, tiles, waves, stream);
-  if (r == 8) return launch_rows<EPI_RESIDUAL, false, 8>(a, tiles, waves, stream);
-  return launch_rows<EPI_RESIDUAL, false, 4>(a, tiles, waves, stream);
+  a.rows = rows_per_workgroup(n, rows);
+  return launch_rows<EPI_RESIDUAL, false>(a, (n + a.rows - 1) / a.rows, waves, stream);
 }

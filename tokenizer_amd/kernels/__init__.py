@@ -306,7 +306,7 @@ class Ops:
     # ------------------------------------------------------- fused decode products
     FUSED_ROWS = 16
     use_fused_decode = True
-    fused_rows = 0            # 0: the launcher picks the weight rows per workgroup (16, 8, 4) ...
+    fused_rows = 0            # 0: the launcher picks the weight rows per workgroup (1..32; 16, 8, 4 with rotation) ...
     fused_waves = 0           # ... and how many waves share a tile's K (4, 8, 16)
 
     def can_fuse_decode(self, rows: int, dtype: torch.dtype) -> bool:
