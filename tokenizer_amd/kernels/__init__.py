@@ -263,14 +263,17 @@ class Ops:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-            if (self.use_library_gemm and bias is None and out_dtype == torch.bfloat16 and m > self.SKINNY_ROWS
-                    and ((k >= 2048 and m >= 128) or m * n * k >= 2 ** 32)):
+            if (self.use_library_gemm and bias is None and out_dtype == torch.bfloat16
+                    and ((m > self.SKINNY_ROWS and ((k >= 2048 and m >= 128) or m * n * k >= 2 ** 32))
+                         or (m > self.FUSED_ROWS and k >= 2048 and n <= 4096))):
                 # Large plain products go to the vendor's library (hipBLASLt through torch), as the
                 # reference's engine uses a library for its matrix products; it is faster there than
-                # the tiled kernel of this package.
+                # the tiled kernel of this package.  So do products of 17 to 64 rows with a long K and few
+                # output columns: the weight-streaming kernel has too few tiles for them and the library
+                # splits K.
                 torch.matmul(x, weight.t(), out=out)
                 return out
-            if m <= self.SKINNY_ROWS:
+            if m <= self.FUSED_ROWS or (m <= self.SKINNY_ROWS and n < self.WIDE_OUTPUT):
                 status = self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, m, n, k,
                                                       _code(out_dtype), 0, self._stream())
             else:
@@ -279,7 +282,9 @@ class Ops:
         self._check(status, "linear")
         return out
 
-    SKINNY_ROWS = 64    # up to this many rows the weight-streaming kernel runs
+    SKINNY_ROWS = 64    # up to this many rows the weight-streaming kernel runs ...
+    WIDE_OUTPUT = 32768  # ... unless there are more than 16 rows and this many output columns (the vocabulary
+    #                      projection): there the rows' re-reading per tile of 16 columns costs more than tiling
     use_library_gemm = True
 
     def linear_silu_gate(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
