@@ -43,9 +43,15 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int wrow = min(n0 + col, n_out - 1);
   const bf16_t* w0 = W + (size_t)wrow * K + 8 * g;
   const bf16_t* w1 = W + (size_t)(wrow + n_out) * K + 8 * g;     // the `up` rows when GATED
+  // Lanes of activation rows past M load nothing and hold zeros: a load costs the memory pipeline by its
+  // active lanes, and with few rows most of a block's lanes are such.
   const bf16_t* a_row[MB];
+  bool a_ok[MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) a_row[mb] = A + (size_t)min(mb * 16 + col, M - 1) * lda + 8 * g;
+  for (int mb = 0; mb < MB; ++mb) {
+    a_ok[mb] = mb * 16 + col < M;
+    a_row[mb] = A + (size_t)min(mb * 16 + col, M - 1) * lda + 8 * g;
+  }
 
   floatx4 acc[SETS][MB];
 #pragma unroll
@@ -65,7 +71,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + k);
       if (GATED) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + k);
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) af[u][mb] = *reinterpret_cast<const bf16x8*>(a_row[mb] + k);
+      for (int mb = 0; mb < MB; ++mb) af[u][mb] = load8(a_row[mb] + k, a_ok[mb]);
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u)
@@ -82,7 +88,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     if (GATED) wf[SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + k);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const bf16x8 af = *reinterpret_cast<const bf16x8*>(a_row[mb] + k);
+      const bf16x8 af = load8(a_row[mb] + k, a_ok[mb]);
 #pragma unroll
       for (int s = 0; s < SETS; ++s)
         acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af, acc[s][mb], 0, 0, 0);
@@ -96,7 +102,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     if (GATED) wf1 = load8(w1 + k, k_ok);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const bf16x8 af = load8(a_row[mb] + k, k_ok);
+      const bf16x8 af = load8(a_row[mb] + k, k_ok && a_ok[mb]);
       acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, af, acc[0][mb], 0, 0, 0);
       if (GATED) acc[SETS - 1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, af, acc[SETS - 1][mb], 0, 0, 0);
     }
