@@ -163,7 +163,8 @@ def make_batch(lengths, q_lens):
         cu_q.append(cu_q[-1] + q_len)
     as_int = lambda values: torch.tensor(values, dtype=torch.int32).cuda()
     return types.SimpleNamespace(n_tokens=cu_q[-1], cu_q=as_int(cu_q), first_position=as_int(first),
-                                 q_tiles=as_int(tiles).reshape(-1, 2), decode_rows=as_int(rows))
+                                 q_tiles=as_int(tiles).reshape(-1, 2), decode_rows=as_int(rows),
+                                 max_position=max(lengths) - 1)
 
 
 # (dtype, fast): the generic kernel in both dtypes, the matrix-core kernels in bfloat16.
@@ -208,10 +209,13 @@ def test_paged_attention(ops, ref, attention_mode, geometry, window):
         torch.testing.assert_close(out_c.float(), out_b.float(), **attention_tol(dtype, True))
 
 
-@pytest.mark.parametrize("geometry", [(14, 2, 64, 16), (12, 2, 128, 16), (3, 1, 32, 32), (5, 5, 16, 16)])
+@pytest.mark.parametrize("geometry,waves", [((14, 2, 64, 16), 0), ((14, 2, 64, 16), 1), ((14, 2, 64, 16), 4),
+                                            ((12, 2, 128, 16), 0), ((3, 1, 32, 32), 2), ((5, 5, 16, 16), 4)])
 @pytest.mark.parametrize("window", [None, 100])
-def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, window):
-    # Portions that start in the middle of a page, end in the middle of a tile, and a long whole prompt.
+def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, window, waves, monkeypatch):
+    # Portions that start in the middle of a page, end in the middle of a tile, and a long whole prompt;
+    # with one wave per tile and with several that share its keys (some of them without a key of their own).
+    monkeypatch.setattr(ops, "prefill_waves", waves)
     n_q, n_kv, d, page_size = geometry
     lengths, q_lens = [700, 333, 40, 16, 1000], [700, 50, 33, 16, 2]
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(

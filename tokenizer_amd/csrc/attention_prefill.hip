@@ -1,6 +1,8 @@
 // Causal (optionally windowed) attention of prompt portions over paged bfloat16 keys and values on the
-// matrix cores.  One wave owns a tile of 16 consecutive tokens of one request, one kv head and a block of
-// HG of the query heads that share it.  As in the decode kernel both products are computed transposed
+// matrix cores.  A workgroup owns a tile of 16 consecutive tokens of one request, one kv head and a block of
+// HG of the query heads that share it; its NWV waves take the blocks of 64 keys in turn and merge their
+// partial softmax states through LDS at the end, so that a tile late in a long prompt is not one long
+// serial walk and a SIMD holds several waves whose matrix and vector work overlap.  As in the decode kernel both products are computed transposed
 // (S^T = K Q^T, O^T = V^T P^T) with 16x16x32 MFMAs: the token index sits in `lane % 16` for scores and
 // outputs, keys and values are read 16 bytes per lane straight from the pages, each key tile once for all
 // HG heads.  Softmax runs online in float; probabilities are rounded to bfloat16 for the second product.
@@ -119,8 +121,8 @@ __device__ __forceinline__ void prefill_block(
 // tiles: [n_tiles, 2] = (entry, offset of the tile's first token inside the entry's tokens).
 // cu_q[e]: first row of entry e; first_position[e]: position of that row.
 // K pages [n_pages, n_kv, page_size, D]; V^T pages [n_pages, n_kv, D, page_size]; page_size % 16 == 0.
-template <int D, int HG>
-__global__ void __launch_bounds__(WAVE)
+template <int D, int HG, int NWV>
+__global__ void __launch_bounds__(NWV * WAVE)
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                          const int* __restrict__ tiles, const int* __restrict__ cu_q,
@@ -128,7 +130,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
                          int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
-  const int lane = threadIdx.x;
+  __shared__ float merge[NWV > 1 ? NWV - 1 : 1][HG][DB * 4 + 2][WAVE];
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int group = n_q / n_kv;
   const int head_blocks = (group + HG - 1) / HG;
@@ -168,13 +171,51 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     for (int db = 0; db < DB; ++db) acc[h][db] = (floatx4){0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int kb = (lo / 64) * 64; kb <= hi; kb += 64) {
+  for (int kb = (lo / 64) * 64 + 64 * wave; kb <= hi; kb += 64 * NWV) {
     if (kb >= lo_all && kb + 63 <= p0)
       prefill_block<D, HG, true>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
                                  my_lo, lo, hi, scale_log2, qf, acc, m, l);
     else
       prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
                                   my_lo, lo, hi, scale_log2, qf, acc, m, l);
+  }
+  if (NWV > 1) {
+    // Waves 1.. hand their state to wave 0: maximum, sum and the output accumulators of each head.
+    if (wave > 0) {
+#pragma unroll
+      for (int h = 0; h < HG; ++h) {
+        merge[wave - 1][h][DB * 4][lane] = m[h];
+        merge[wave - 1][h][DB * 4 + 1][lane] = l[h];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) merge[wave - 1][h][db * 4 + r][lane] = acc[h][db][r];
+      }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+      float m_all = m[h];
+#pragma unroll
+      for (int w = 0; w < NWV - 1; ++w) m_all = fmaxf(m_all, merge[w][h][DB * 4][lane]);
+      const float mc = (m_all == -INFINITY) ? 0.f : m_all * scale_log2;
+      const float f0 = __builtin_amdgcn_exp2f(m[h] * scale_log2 - mc);       // a wave without keys: exp2(-inf) = 0
+      l[h] *= f0;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[h][db][r] *= f0;
+#pragma unroll
+      for (int w = 0; w < NWV - 1; ++w) {
+        const float f = __builtin_amdgcn_exp2f(merge[w][h][DB * 4][lane] * scale_log2 - mc);
+        l[h] += f * merge[w][h][DB * 4 + 1][lane];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[h][db][r] += f * merge[w][h][db * 4 + r][lane];
+      }
+    }
   }
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
@@ -195,33 +236,52 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   }
 }
 
-template <int D, int HG>
-static int launch_prefill(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
-                          const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
-                          const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
-                          float scale, hipStream_t stream) {
+template <int D, int HG, int NWV>
+static int launch_prefill_waves(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
+                                const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
+                                const void* block_table, int table_stride, int n_q, int n_kv, int page_size,
+                                int window, float scale, hipStream_t stream) {
   const int group = n_q / n_kv;
   dim3 grid(n_tiles, n_kv * ((group + HG - 1) / HG));
-  prefill_attention_kernel<D, HG><<<grid, WAVE, 0, stream>>>(
+  prefill_attention_kernel<D, HG, NWV><<<grid, NWV * WAVE, 0, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
       (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
       window, scale * 1.4426950408889634f);
   return LAUNCH_STATUS();
 }
 
+// waves: waves per tile (1, 2 or 4); 0 = by the longest reach of a token: one wave per 256 keys or so.
+template <int D, int HG>
+static int launch_prefill(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
+                          const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
+                          const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
+                          float scale, int max_keys, int waves, hipStream_t stream) {
+  if (waves == 0) {
+    const int reach = (window >= 0 && window + 16 < max_keys) ? window + 16 : max_keys;
+    waves = reach > 768 ? 4 : reach > 256 ? 2 : 1;
+  }
+#define GO(NWV) launch_prefill_waves<D, HG, NWV>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
+    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream)
+  if (waves >= 4) return GO(4);
+  if (waves >= 2) return GO(2);
+  return GO(1);
+#undef GO
+}
+
 // Returns -2 for a head size without an instance (the caller then uses another kernel).
+// max_keys: the highest position of the batch + 1 (a hint for the number of waves per tile).
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
                                          int n_q, int n_kv, int d, int page_size, int window, float scale,
-                                         int heads_per_wave, hipStream_t stream) {
+                                         int heads_per_wave, int max_keys, int waves, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
   if (d == 64 && heads_per_wave == 1)
     return launch_prefill<64, 1>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position,
-                                 block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
+                                 block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, stream);
 #define CASE(DD, HG) case DD: return launch_prefill<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
-    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
+    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, stream);
   switch (d) {
     CASE(16, 4) CASE(32, 4) CASE(48, 2) CASE(64, 2) CASE(80, 2) CASE(96, 2) CASE(112, 2) CASE(128, 2)
     CASE(160, 1) CASE(192, 1) CASE(224, 1) CASE(256, 1)

@@ -194,7 +194,8 @@ class Ops:
                 _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(batch.q_tiles),
                 batch.q_tiles.shape[0], _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
                 block_table.shape[1], n_q, n_kv, head_dim, page_size, -1 if window is None else int(window),
-                ctypes.c_float(scale), self.prefill_heads_per_wave, self._stream()), "prefill_attention")
+                ctypes.c_float(scale), self.prefill_heads_per_wave, int(batch.max_position) + 1,
+                self.prefill_waves, self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
                 self._decode_attention(*args, rows=batch.decode_rows)
             return out
@@ -207,6 +208,7 @@ class Ops:
 
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
     use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
+    prefill_waves = 0          # waves that share a tile's keys in the prompt kernel: 0 lets the launcher choose
     prefill_heads_per_wave = 0    # 0: the kernel's own choice for the head size
     target_workgroups = 1024      # what the split of the key range aims at
 
