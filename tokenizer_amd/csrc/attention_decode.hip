@@ -50,7 +50,8 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int heads_here = min(16, group - hb * 16);
   const int head = kvh * group + hb * 16 + col;          // valid when col < heads_here
   const int pos = positions[t];
-  const int* table = block_table + (size_t)entry_of_token[t] * table_stride;
+  // entry_of_token null: every request has one token in the batch, request e is row e (one dependent load fewer).
+  const int* table = block_table + (size_t)(entry_of_token ? entry_of_token[t] : t) * table_stride;
   const int lo = (window >= 0 && pos > window) ? pos - window : 0;
   const int first = (lo / 32) * 32 + split * split_keys;  // first key of this split (a multiple of 32)
   const int last = min(pos, first + split_keys - 1);
@@ -123,8 +124,8 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(m, mx);
-    if (m_new == -INFINITY) continue;                      // nothing visible yet (uniform over the head's lanes)
-    const float corr = __expf(m - m_new);
+    if (__all(m_new == -INFINITY)) continue;               // nothing visible yet: the same for every head, a scalar branch
+    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
     bf16x8 pf;
     float psum = 0.f;
 #pragma unroll
@@ -178,8 +179,9 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   }
 }
 
-// out[t, head, :] = sum_s part_o[s] * exp(m_s - M) / sum_s l_s * exp(m_s - M).  One wave per (item, head):
-// the lanes first share out the splits (maximum and denominator), then the elements of the head.
+// out[t, head, :] = sum_s part_o[s] * exp(m_s - M) / sum_s l_s * exp(m_s - M).  One wave per (item, head).
+// Sixteen lanes share a split's 64 elements (a float4 each), the four groups of sixteen take every fourth
+// split, and all of a lane's loads are requested before the first is used: the kernel is one trip to memory.
 // A separate kernel on purpose: a last-arrival merge inside the first kernel needs device-wide fences,
 // which flush the L2 of every XCD and cost more than this launch.
 __global__ void __launch_bounds__(WAVE)
@@ -188,25 +190,60 @@ decode_attention_merge(const float* __restrict__ part_o, const float* __restrict
   const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
   const int t = rows ? rows[item] : item;
   const size_t base = ((size_t)item * n_q + head) * splits;
-  const int lane = threadIdx.x;
-  float big = -INFINITY;
-  for (int s = lane; s < splits; s += WAVE) big = fmaxf(big, part_ml[(base + s) * 2]);
-  big = wave_max(big);
-  float denom = 0.f;
-  for (int s = lane; s < splits; s += WAVE) {
-    const float ms = part_ml[(base + s) * 2];
-    if (ms != -INFINITY) denom += part_ml[(base + s) * 2 + 1] * __expf(ms - big);
-  }
-  denom = wave_sum(denom);
-  for (int i = lane; i < d; i += WAVE) {
-    float o = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < splits; ++s) {
-      const float ms = part_ml[(base + s) * 2];                 // the same address for every lane: one load
-      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - big);
-      o += part_o[(base + s) * d + i] * w;
+  const int lane = threadIdx.x, part = lane & 15, grp = lane >> 4;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
+  constexpr int HELD = 8;                                    // splits a lane holds at once: 32 per round
+  for (int e0 = 0; e0 < d; e0 += 64) {
+    const int e = e0 + 4 * part;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    float big = -INFINITY, denom = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += 4 * HELD) {
+      float4 v[HELD];
+      float2 stat[HELD];
+#pragma unroll
+      for (int j = 0; j < HELD; ++j) {
+        const int s = s0 + 4 * j + grp;
+        v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        stat[j] = make_float2(-INFINITY, 0.f);
+        if (s < splits) {
+          stat[j] = ml[s];
+          if (e < d) v[j] = *reinterpret_cast<const float4*>(part_o + (base + s) * d + e);
+        }
+      }
+      float round_big = big;
+#pragma unroll
+      for (int j = 0; j < HELD; ++j) round_big = fmaxf(round_big, stat[j].x);
+      const float keep = (big == -INFINITY) ? 0.f : __expf(big - round_big);   // this lane's sums so far, rescaled
+      o.x *= keep; o.y *= keep; o.z *= keep; o.w *= keep;
+      denom *= keep;
+      big = round_big;
+#pragma unroll
+      for (int j = 0; j < HELD; ++j) {
+        const float w = (stat[j].x == -INFINITY) ? 0.f : __expf(stat[j].x - big);
+        o.x += v[j].x * w; o.y += v[j].y * w; o.z += v[j].z * w; o.w += v[j].w * w;
+        denom += stat[j].y * w;
+      }
     }
-    st(out + (size_t)t * n_q * d + (size_t)head * d + i, o / denom);
+    // The four lane groups hold sums over different splits under different maxima: bring them together.
+    float all_big = fmaxf(big, __shfl_xor(big, 16, WAVE));
+    all_big = fmaxf(all_big, __shfl_xor(all_big, 32, WAVE));
+    const float w = (big == -INFINITY) ? 0.f : __expf(big - all_big);
+    o.x *= w; o.y *= w; o.z *= w; o.w *= w;
+    denom *= w;
+#pragma unroll
+    for (int shift = 16; shift <= 32; shift *= 2) {
+      o.x += __shfl_xor(o.x, shift, WAVE); o.y += __shfl_xor(o.y, shift, WAVE);
+      o.z += __shfl_xor(o.z, shift, WAVE); o.w += __shfl_xor(o.w, shift, WAVE);
+      denom += __shfl_xor(denom, shift, WAVE);
+    }
+    if (grp == 0 && e < d) {
+      const float inv = 1.0f / denom;
+      bf16_t* dst = out + (size_t)t * n_q * d + (size_t)head * d + e;
+      union { bf16x4 v; uint2 bits; } packed;
+      packed.v[0] = (__bf16)(o.x * inv); packed.v[1] = (__bf16)(o.y * inv);
+      packed.v[2] = (__bf16)(o.z * inv); packed.v[3] = (__bf16)(o.w * inv);
+      *reinterpret_cast<uint2*>(dst) = packed.bits;
+    }
   }
 }
 

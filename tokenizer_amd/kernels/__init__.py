@@ -186,8 +186,11 @@ class Ops:
                 and qkv.shape[1] % 8 == 0 and self.use_fast_attention):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
-            if batch is None or batch.q_tiles.numel() == 0:
+            if batch is None:
                 return self._decode_attention(*args)
+            if batch.q_tiles.numel() == 0:
+                # One token per request: request e is row e, the kernel needs no entry-of-token lookup.
+                return self._decode_attention(*args, identity_entries=batch.n_tokens == block_table.shape[0])
             _need(batch.n_tokens == n_tokens and batch.cu_q.numel() == block_table.shape[0] + 1,
                   "the batch description does not belong to these tokens")
             self._check(self.lib.ta_prefill_attention_bf16(
@@ -213,7 +216,8 @@ class Ops:
     target_workgroups = 1024      # what the split of the key range aims at
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
-                          n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None):
+                          n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None,
+                          identity_entries=False):
         """Matrix-core attention of single tokens with the key range split over workgroups."""
         n_items = qkv.shape[0] if rows is None else rows.numel()
         max_keys = (block_table.shape[1] * page_size) if max_position is None else max_position + 1
@@ -230,7 +234,8 @@ class Ops:
             part_ml = torch.empty((n_items, n_q, splits, 2), dtype=torch.float32, device=qkv.device)
         self._check(self.lib.ta_decode_attention_bf16(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(rows), _ptr(positions),
-            _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], _ptr(part_o), _ptr(part_ml), n_items,
+            _ptr(None if identity_entries and rows is None else entry_of_token), _ptr(block_table),
+            block_table.shape[1], _ptr(part_o), _ptr(part_ml), n_items,
             n_q, n_kv, head_dim, page_size, -1 if window is None else int(window), ctypes.c_float(scale),
             split_keys, splits, self._stream()), "decode_attention")
         return out
