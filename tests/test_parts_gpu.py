@@ -335,3 +335,178 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype, twice):
                 ids.append(plain.greedy_token(toy_plain_logits(tensors, ids, 2, twice)[-1]))
             assert results[rid].tokens == ids[len(prompt):]
     sched.assert_idle()
+
+
+# ------------------------------------------------------------------------------------------------
+# A second toy architecture: a feed-forward with routing and another position encoding, again defined
+# here.  Layer 0: attention with distance decay + two routed experts; layer 1: windowed attention with
+# rotation + a dense feed-forward.  So one model has different mixers' options, position encodings and
+# feed-forwards in different layers, and two cache groups.
+def register_routed_toys():
+    from tokenizer_amd.config import get_architecture, register_architecture, registered_architectures
+    from tokenizer_amd.config.base import ModelConfig
+    if "ToyRoutedForCausalLM" in registered_architectures():
+        return get_architecture("ToyRoutedForCausalLM").config_class
+    from tokenizer_amd.parts import (FEED_FORWARDS, POSITIONS, FeedForward, FeedForwardSpec, LayerSpec, MixerSpec,
+                                     ModelSpec, NormSpec, PositionSpec, ScheduleEntry, TensorSpec)
+    from tokenizer_amd.parts.position import NoPosition
+
+    if "distance_decay" not in POSITIONS.kinds():
+        @POSITIONS.register("distance_decay")
+        class DistanceDecay(NoPosition):
+            """q_i is scaled by g^-i and k_j by g^j, so that a score is q_i.k_j * g^(j - i): only distances
+            count.  The scaling is this test's own torch code; the store into the pages is the package's."""
+            graph_safe = False
+
+            def __init__(self, spec, runtime):
+                super().__init__(spec, runtime)
+                self.gamma = float(spec.options["gamma"])
+
+            def encode_and_store(self, qkv, bias, n_q, n_kv, head_dim, ctx, cache):
+                assert bias is None
+                pos = ctx.positions.to(torch.float32)[:, None]
+                q_end, k_end = n_q * head_dim, (n_q + n_kv) * head_dim
+                qkv[:, :q_end] = (qkv[:, :q_end].float() * self.gamma ** (-pos)).to(qkv.dtype)
+                qkv[:, q_end:k_end] = (qkv[:, q_end:k_end].float() * self.gamma ** pos).to(qkv.dtype)
+                super().encode_and_store(qkv, None, n_q, n_kv, head_dim, ctx, cache)
+
+    if "top1_experts" not in FEED_FORWARDS.kinds():
+        @FEED_FORWARDS.register("top1_experts")
+        class Top1Experts(FeedForward):
+            """Router logits in float32, the first maximum picks one expert a token, its output is scaled by the
+            softmax weight of that expert.  Every expert is the package's dense gated part."""
+
+            def __init__(self, spec, tensors, runtime):
+                self.runtime, self.n = runtime, int(spec.options["experts"])
+                self.router = tensors["router.weight"].float()
+                dense = FEED_FORWARDS.get("gated_dense")
+                inner = FeedForwardSpec("gated_dense", spec.hidden_size, spec.intermediate_size, "silu")
+                self.experts = [dense(inner, {k[len(f"experts.{e}."):]: v for k, v in tensors.items()
+                                              if k.startswith(f"experts.{e}.")}, runtime) for e in range(self.n)]
+
+            @staticmethod
+            def tensor_specs(spec):
+                dense = FEED_FORWARDS.get("gated_dense")
+                inner = FeedForwardSpec("gated_dense", spec.hidden_size, spec.intermediate_size, "silu")
+                specs = {"router.weight": TensorSpec((int(spec.options["experts"]), spec.hidden_size), std=0.5,
+                                                     role="keep")}
+                for e in range(int(spec.options["experts"])):
+                    specs.update({f"experts.{e}.{k}": v for k, v in dense.tensor_specs(inner).items()})
+                return specs
+
+            def forward(self, x, ctx):
+                logits = x.float() @ self.router.t()
+                choice = torch.argmax(logits, dim=-1)
+                weight = torch.softmax(logits, dim=-1).gather(1, choice[:, None])
+                out = torch.zeros_like(x)
+                for e, expert in enumerate(self.experts):
+                    rows = torch.nonzero(choice == e).flatten()
+                    if rows.numel():
+                        out[rows] = expert.forward(x[rows].contiguous(), ctx)
+                return (out.float() * weight).to(x.dtype)
+
+    @dataclasses.dataclass(frozen=True)
+    class RoutedConfig(ModelConfig):
+        vocab_size: int
+        hidden_size: int
+        heads: int
+        kv_heads: int
+        inner: int
+        experts: int
+        gamma: float
+        window: int
+
+    def routed_spec(cfg):
+        d = cfg.hidden_size // cfg.heads
+        norm = NormSpec("rmsnorm", cfg.hidden_size, 1e-5)
+        decay = PositionSpec("distance_decay", d, options={"gamma": cfg.gamma})
+        rope = PositionSpec("rope_half_split", d, 10000.0, 512)
+        mixers = [MixerSpec("gqa_attention", cfg.hidden_size, cfg.heads, cfg.kv_heads, d, qkv_bias=False, position=decay),
+                  MixerSpec("gqa_attention", cfg.hidden_size, cfg.heads, cfg.kv_heads, d, qkv_bias=False, position=rope,
+                            window=cfg.window)]
+        ffs = [FeedForwardSpec("top1_experts", cfg.hidden_size, cfg.inner, "silu", options={"experts": cfg.experts}),
+               FeedForwardSpec("gated_dense", cfg.hidden_size, 2 * cfg.inner, "silu")]
+        layers = tuple(LayerSpec("pre_norm", m, f, norm, norm, f"l.{i}.mix", f"l.{i}.ff", f"l.{i}.n1", f"l.{i}.n2")
+                       for i, (m, f) in enumerate(zip(mixers, ffs)))
+        return ModelSpec("ToyRoutedForCausalLM", cfg.vocab_size, cfg.hidden_size, 512, "emb.weight", layers,
+                         (ScheduleEntry(0), ScheduleEntry(1)), norm, "final", tied_head=True, head_name="head.weight")
+
+    register_architecture("ToyRoutedForCausalLM", RoutedConfig, routed_spec)
+    return RoutedConfig
+
+
+def routed_plain_logits(tensors, ids, cfg):
+    """The routed toy model on whole sequences with the plain parts."""
+    t = {k: v.float() for k, v in tensors.items()}
+    hidden, heads, kv = cfg["hidden_size"], cfg["heads"], cfg["kv_heads"]
+    d, n = hidden // heads, len(ids)
+    pos = list(range(n))
+    x = t["emb.weight"][ids]
+
+    def attention(x, i, window, encode):
+        h = plain.rms_norm(x, t[f"l.{i}.n1.weight"], 1e-5)
+        def heads_of(name, count):
+            return (h @ t[f"l.{i}.mix.{name}.weight"].t()).reshape(n, count, d).transpose(0, 1)
+        q, k, v = encode(heads_of("q_proj", heads), True), encode(heads_of("k_proj", kv), False), heads_of("v_proj", kv)
+        k, v = plain.repeat_kv(k, heads // kv), plain.repeat_kv(v, heads // kv)
+        mixed = plain.attend(q, k, v, plain.attention_mask(pos, pos, window)).transpose(0, 1).reshape(n, hidden)
+        return x + mixed @ t[f"l.{i}.mix.o_proj.weight"].t()
+
+    def dense(h, prefix):
+        return plain.mlp(h, {f"m.{k[len(prefix):]}": v for k, v in t.items() if k.startswith(prefix)}, "m")
+
+    steps = torch.tensor(pos, dtype=torch.float32)[None, :, None]
+    x = attention(x, 0, None, lambda v, is_q: v * cfg["gamma"] ** (-steps if is_q else steps))
+    h = plain.rms_norm(x, t["l.0.n2.weight"], 1e-5)
+    logits = h @ t["l.0.ff.router.weight"].t()
+    choice = [plain.greedy_token(row) for row in logits]
+    top2 = torch.topk(logits, 2, dim=-1).values
+    routed_plain_logits.smallest_gap = float((top2[:, 0] - top2[:, 1]).min())
+    weight = torch.softmax(logits, dim=-1)
+    out = torch.stack([dense(h[j:j + 1], f"l.0.ff.experts.{choice[j]}.")[0] * weight[j, choice[j]] for j in range(n)])
+    x = x + out
+    cos, sin = plain.rope_tables(10000.0, d, 512)
+    x = attention(x, 1, cfg["window"], lambda v, is_q: plain.apply_rope(v, cos[pos], sin[pos]))
+    x = x + dense(plain.rms_norm(x, t["l.1.n2.weight"], 1e-5), "l.1.ff.")
+    return plain.rms_norm(x, t["final.weight"], 1e-5) @ t["emb.weight"].t()
+
+
+def test_distance_decay_counts_only_distances():
+    """What pins the toy position encoding's plain form: shifting every position changes no score."""
+    q, k = rand((1, 5, 8), 90).cpu(), rand((1, 5, 8), 91).cpu()
+    def scores(first):
+        steps = torch.arange(first, first + 5, dtype=torch.float32)[None, :, None]
+        return (q * 0.97 ** -steps) @ (k * 0.97 ** steps).transpose(1, 2)
+    torch.testing.assert_close(scores(0), scores(40), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_architecture(tmp_path, dtype):
+    import trace_tools as tt
+    import tokenizer_amd as ta
+    from safetensors.torch import load_file
+    from tokenizer_amd.engine import Engine, load_model
+
+    config_cls = register_routed_toys()
+    values = {"vocab_size": 80, "hidden_size": 96, "heads": 6, "kv_heads": 2, "inner": 56, "experts": 3,
+              "gamma": 0.97, "window": 19}
+    cfg = config_cls.from_dict(values)
+    folder = ta.write_random_model(cfg, 5, str(tmp_path / "routed"))
+    tensors = load_file(folder + "/model.safetensors")
+    assert tensors["l.0.ff.router.weight"].dtype == torch.float32 and "l.0.ff.experts.2.down_proj.weight" in tensors
+    model = load_model(folder, dtype)
+    assert [n.kind for n in model.cache_needs] == ["full", "window"]
+    # Seeds picked (on the CPU, with the plain model) so that the narrowest router decision is clear.
+    requests = {f"r{i}": random_ids(80, n, seed) for i, (n, seed) in enumerate([(50, 92), (3, 70), (77, 99), (34, 123)])}
+    steps = tt.mixed(requests, 9, max_live=3)
+    engine = Engine(model, max_tokens=tt.peak_tokens(steps), max_requests=3)
+    assert len(engine.cache.groups) == 2
+    engine.pools.poison()
+    got = tt.run_in_process(engine, steps)
+    for rid, ids in requests.items():
+        want = routed_plain_logits(tensors, ids, values)
+        # The inputs are chosen so that no router decision is near a tie, which bfloat16 could turn the other way.
+        assert routed_plain_logits.smallest_gap > 0.2, routed_plain_logits.smallest_gap
+        err = float((got[rid] - want).abs().max())
+        assert err <= (3e-5 if dtype == "float32" else 4e-2) * max(1.0, float(want.abs().max())), (rid, err)
+    engine.cache.check_invariants()

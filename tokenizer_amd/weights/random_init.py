@@ -35,7 +35,9 @@ def random_tensor(name: str, spec: TensorSpec, seed: int) -> torch.Tensor:
         raise ValueError(f"unknown init {spec.init!r} for {name}")
     values = torch.empty(spec.shape, dtype=torch.float32)
     values.normal_(0.0, spec.std, generator=_generator(seed, name))
-    return values.to(torch.bfloat16)
+    # A tensor that is kept as stored is written in 32-bit: that is what such tensors (router weights,
+    # decay rates and the like) are stored in, and the loader then leaves it so in both modes.
+    return values if spec.role == "keep" else values.to(torch.bfloat16)
 
 
 def random_tensors(expected: dict[str, TensorSpec], seed: int) -> dict[str, torch.Tensor]:
