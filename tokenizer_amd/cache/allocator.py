@@ -1,18 +1,17 @@
 """Page allocator: free stack, reference counts, prefix index and a list of cached pages.
 
-Behaviour follows qwen-infer/src/paged.rs:125-519.  Page ids are 0..n-1 and the first
-allocation returns 0; the page freed last is handed out next.  A page published under the
-hash of its tokens stays out of the free stack when its count falls to zero, so a later
-request with the same prefix can take it; `alloc` evicts such pages, oldest first, only
-after the free stack is empty.
+The allocator itself is C++ (`csrc/host/page_allocator.cpp`); this class binds it.  Behaviour follows
+qwen-infer/src/paged.rs:125-519.  Page ids are 0..n-1 and the first allocation returns 0; the page freed
+last is handed out next.  A page published under the hash of its tokens stays out of the free stack when
+its count falls to zero, so a later request with the same prefix can take it; `alloc` evicts such pages,
+oldest first, only after the free stack is empty.
 """
 from __future__ import annotations
 
-import collections
-import dataclasses
+import ctypes
 import enum
 
-_MASK = (1 << 64) - 1
+from .. import host as _host
 
 
 class AllocError(Exception):
@@ -42,214 +41,151 @@ class Release(enum.Enum):
     FREED = "freed"      # back on the free stack
 
 
+_RELEASES = (Release.SHARED, Release.CACHED, Release.FREED)
+_CAPACITY, _FREE, _CACHED, _AVAILABLE, _LIVE, _OCCUPIED, _REFCOUNT, _ALL_ZERO, _PEAK_LIVE, _PEAK_OCCUPIED = range(10)
+
+
 def prefix_page_hash(parent: int, tokens) -> int:
     """Chained hash of one full page of token ids (qwen-infer/src/paged.rs:93-100)."""
-    value = 0xCBF29CE484222325 ^ parent
-    for token in tokens:
-        value ^= int(token) & 0xFFFFFFFF
-        value = (value * 0x100000001B3) & _MASK
-    return value
+    keep, pointer = _host.token_array(tokens)
+    return int(_host.lib().ta_prefix_page_hash(parent, pointer, len(keep)))
 
 
-@dataclasses.dataclass
-class _PrefixEntry:
-    page: int
-    parent_hash: int
-    parent_page: int | None
-    tokens: tuple[int, ...]
+_tokens = _host.token_array
 
 
 class PageAllocator:
-    def __init__(self, num_pages: int, page_size: int = 16):
-        if num_pages < 0 or page_size <= 0:
-            raise ValueError("num_pages must not be negative and page_size must be positive")
+    def __init__(self, num_pages: int, page_size: int = 16, _borrowed=None):
+        self._lib = _host.lib()
+        if _borrowed is not None:                 # an allocator that lives inside a cache manager
+            self._handle, self._owned = _borrowed, False
+        else:
+            if num_pages < 0 or page_size <= 0:
+                raise ValueError("num_pages must not be negative and page_size must be positive")
+            self._handle, self._owned = self._lib.ta_alloc_new(num_pages, page_size), True
         self.page_size = page_size
-        self._capacity = num_pages
-        self._free = list(range(num_pages - 1, -1, -1))
-        self._refcount = [0] * num_pages
-        self._hash_of: list[int | None] = [None] * num_pages
-        self._cached: "collections.OrderedDict[int, None]" = collections.OrderedDict()  # oldest first
-        self._index: dict[int, _PrefixEntry] = {}
-        self._live = 0
-        self.peak_live = 0
-        self.peak_occupied = 0
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self._handle:
+            self._lib.ta_alloc_delete(self._handle)
+            self._handle = None
+
+    def _get(self, what: int, arg: int = 0) -> int:
+        return self._lib.ta_alloc_get(self._handle, what, arg)
+
+    def _raise(self, status: int, page: int, length: int = 0) -> None:
+        if status == -1:
+            raise DoubleFree(page)
+        if status == -2:
+            raise UnknownPage(page)
+        if status == -3:
+            raise NotFull(page, length, self.page_size)
 
     # ------------------------------------------------------------------ counters
     def capacity(self) -> int:
-        return self._capacity
+        return self._get(_CAPACITY)
 
     def free_count(self) -> int:
-        return len(self._free)
+        return self._get(_FREE)
 
     def cached_count(self) -> int:
-        return len(self._cached)
+        return self._get(_CACHED)
 
     def available(self) -> int:
         """Pages an allocation can draw on: the free stack plus cached pages."""
-        return len(self._free) + len(self._cached)
+        return self._get(_AVAILABLE)
 
     def live_count(self) -> int:
-        return self._live
+        return self._get(_LIVE)
 
     def occupied(self) -> int:
-        return self._live + len(self._cached)
+        return self._get(_OCCUPIED)
 
     def refcount(self, page: int) -> int | None:
-        return self._refcount[page] if 0 <= page < self._capacity else None
+        count = self._get(_REFCOUNT, page)
+        return None if count < 0 else count
 
     def all_refcounts_zero(self) -> bool:
-        return not any(self._refcount)
+        return bool(self._get(_ALL_ZERO))
+
+    @property
+    def peak_live(self) -> int:
+        return self._get(_PEAK_LIVE)
+
+    @property
+    def peak_occupied(self) -> int:
+        return self._get(_PEAK_OCCUPIED)
 
     def peak_mark(self) -> tuple[int, int]:
         return self.peak_live, self.peak_occupied
 
     def rewind_peaks(self, mark: tuple[int, int]) -> None:
-        self.peak_live = max(mark[0], self._live)
-        self.peak_occupied = max(mark[1], self.occupied())
-
-    def _note_peaks(self) -> None:
-        self.peak_live = max(self.peak_live, self._live)
-        self.peak_occupied = max(self.peak_occupied, self.occupied())
+        self._lib.ta_alloc_rewind_peaks(self._handle, mark[0], mark[1])
 
     # ---------------------------------------------------------------- alloc/free
     def alloc(self) -> int | None:
-        if self._free:
-            page = self._free.pop()
-        elif self._cached:
-            page, _ = self._cached.popitem(last=False)
-            self._unindex(page)
-        else:
-            return None
-        self._refcount[page] = 1
-        self._live += 1
-        self._note_peaks()
-        return page
+        page = self._lib.ta_alloc_alloc(self._handle)
+        return None if page < 0 else page
 
     def alloc_n(self, n: int) -> list[int] | None:
         """`n` pages or none at all."""
-        if self.available() < n:
+        out = (ctypes.c_int32 * max(1, n))()
+        if not self._lib.ta_alloc_alloc_n(self._handle, n, out):
             return None
-        return [self.alloc() for _ in range(n)]
+        return list(out[:n])
 
     def free_page(self, page: int) -> Release:
-        if not 0 <= page < self._capacity:
-            raise UnknownPage(page)
-        if self._refcount[page] == 0:
-            raise DoubleFree(page)
-        self._refcount[page] -= 1
-        if self._refcount[page] > 0:
-            return Release.SHARED
-        self._live -= 1
-        if self._hash_of[page] is not None:
-            self._cached[page] = None
-            self._note_peaks()
-            return Release.CACHED
-        self._free.append(page)
-        self._note_peaks()
-        return Release.FREED
+        how = ctypes.c_int32(0)
+        self._raise(self._lib.ta_alloc_free(self._handle, page, ctypes.byref(how)), page)
+        return _RELEASES[how.value]
 
     def incref(self, page: int) -> None:
-        if not 0 <= page < self._capacity:
-            raise UnknownPage(page)
-        if self._refcount[page] == 0:
-            if page not in self._cached:
-                raise DoubleFree(page)
-            del self._cached[page]
-            self._refcount[page] = 1
-            self._live += 1
-            self._note_peaks()
-            return
-        self._refcount[page] += 1
+        self._raise(self._lib.ta_alloc_incref(self._handle, page), page)
 
     # -------------------------------------------------------------- prefix index
     def publish_full_page(self, parent_hash: int, tokens, page: int) -> None:
-        if len(tokens) != self.page_size:
-            raise NotFull(page, len(tokens), self.page_size)
-        if not 0 <= page < self._capacity or self._refcount[page] == 0:
-            raise UnknownPage(page)
-        self._publish_at(prefix_page_hash(parent_hash, tokens), parent_hash, None, tuple(tokens), page)
+        keep, pointer = _tokens(tokens)
+        self._raise(self._lib.ta_alloc_publish_full_page(self._handle, parent_hash, pointer, len(keep), page),
+                    page, len(keep))
 
     def find_full_page(self, parent_hash: int, parent_page: int | None, tokens) -> int | None:
-        if len(tokens) != self.page_size:
-            return None
-        return self._find_at(prefix_page_hash(parent_hash, tokens), parent_hash, parent_page, tuple(tokens))
+        keep, pointer = _tokens(tokens)
+        page = self._lib.ta_alloc_find_full_page(self._handle, parent_hash, -1 if parent_page is None else parent_page,
+                                                 pointer, len(keep))
+        return None if page < 0 else page
 
     def take_shared_prefix(self, tokens) -> list[int]:
         """Published full pages of `tokens`, in order, each with one more holder; stops at the first miss."""
-        parent_hash, parent_page, shared, offset = 0, None, [], 0
-        size = self.page_size
-        while offset + size <= len(tokens):
-            chunk = tuple(tokens[offset:offset + size])
-            page = self.find_full_page(parent_hash, parent_page, chunk)
-            if page is None:
-                break
-            try:
-                self.incref(page)
-            except AllocError:
-                break
-            shared.append(page)
-            parent_hash = prefix_page_hash(parent_hash, chunk)
-            parent_page = page
-            offset += size
-        return shared
+        keep, pointer = _tokens(tokens)
+        out = (ctypes.c_int32 * max(1, len(keep) // self.page_size))()
+        count = self._lib.ta_alloc_take_shared_prefix(self._handle, pointer, len(keep), out)
+        return list(out[:count])
 
     def publish_prompt_pages(self, tokens, pages) -> None:
         """Index every full page of `tokens`; pages[i] holds tokens [i*size, (i+1)*size)."""
-        size = self.page_size
-        parent_hash, parent_page = 0, None
-        for index in range(len(tokens) // size):
-            if index >= len(pages):
-                break
-            chunk = tuple(tokens[index * size:(index + 1) * size])
-            page = pages[index]
-            value = prefix_page_hash(parent_hash, chunk)
-            if not 0 <= page < self._capacity or self._refcount[page] == 0:
-                break
-            self._publish_at(value, parent_hash, parent_page, chunk, page)
-            if self._find_at(value, parent_hash, parent_page, chunk) != page:
-                break
-            parent_hash, parent_page = value, page
+        keep, pointer = _tokens(tokens)
+        held, page_pointer = _host.int_array(list(pages))
+        self._lib.ta_alloc_publish_prompt_pages(self._handle, pointer, len(keep), page_pointer, len(held))
+
+    def _publish_at(self, value: int, parent_hash: int, parent_page: int | None, tokens, page: int) -> bool:
+        """Index `page` under a given hash value (what publishing does after hashing)."""
+        keep, pointer = _tokens(tokens)
+        return bool(self._lib.ta_alloc_publish_at(self._handle, value, parent_hash,
+                                                  -1 if parent_page is None else parent_page, pointer, len(keep), page))
+
+    def _find_at(self, value: int, parent_hash: int, parent_page: int | None, tokens) -> int | None:
+        keep, pointer = _tokens(tokens)
+        page = self._lib.ta_alloc_find_at(self._handle, value, parent_hash, -1 if parent_page is None else parent_page,
+                                          pointer, len(keep))
+        return None if page < 0 else page
 
     def reclaim_cached(self) -> None:
-        while self._cached:
-            page, _ = self._cached.popitem(last=False)
-            self._unindex(page)
-            self._free.append(page)
-
-    def _publish_at(self, value, parent_hash, parent_page, tokens, page) -> bool:
-        existing = self._index.get(value)
-        if existing is not None:
-            return (existing.page == page and existing.parent_hash == parent_hash
-                    and existing.parent_page == parent_page and existing.tokens == tokens)
-        if self._hash_of[page] is not None:
-            return False
-        self._index[value] = _PrefixEntry(page, parent_hash, parent_page, tokens)
-        self._hash_of[page] = value
-        return True
-
-    def _find_at(self, value, parent_hash, parent_page, tokens) -> int | None:
-        entry = self._index.get(value)
-        if entry and entry.parent_hash == parent_hash and entry.parent_page == parent_page and entry.tokens == tokens:
-            return entry.page
-        return None
-
-    def _unindex(self, page: int) -> None:
-        value = self._hash_of[page]
-        self._hash_of[page] = None
-        if value is not None and value in self._index and self._index[value].page == page:
-            del self._index[value]
+        self._lib.ta_alloc_reclaim_cached(self._handle)
 
     # ------------------------------------------------------------------- checking
     def check_invariants(self) -> None:
         """Every page is in exactly one place: free, cached (count 0, indexed) or live (count > 0)."""
-        seen = collections.Counter(self._free)
-        assert all(count == 1 for count in seen.values()), "a page is on the free stack twice"
-        for page in range(self._capacity):
-            places = (page in seen) + (page in self._cached) + (self._refcount[page] > 0)
-            assert places == 1, f"page {page} is in {places} places"
-            if page in self._cached:
-                assert self._hash_of[page] is not None
-        assert self._live == sum(1 for count in self._refcount if count > 0)
+        assert self._lib.ta_alloc_check(self._handle) == 0, _host.message()
 
 
 def pages_for_len(length: int, page_size: int) -> int:

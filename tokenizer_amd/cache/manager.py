@@ -6,12 +6,18 @@ all layers of a group use the same page ids in their own pool tensors.  A "windo
 pages back once every later query is past them.  Beside the pages, each live request holds
 one *slot* for per-request state of fixed size (used by mixers that declare a `state_shape`).
 
-This class only does bookkeeping on the host; the tensors live in `CachePools`.
+This class only does bookkeeping on the host; the tensors live in `CachePools`.  The bookkeeping itself
+(tables, reservation, window release, prefix sharing, slots, and the packing of a step's batch description)
+is C++ (`csrc/host/cache_core.cpp`); this class binds it and keeps the Python-side names of requests.
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
 
+import numpy as np
+
+from .. import host as _host
 from ..parts.spec import CacheNeed
 from .allocator import PageAllocator, pages_for_len
 
@@ -56,97 +62,126 @@ def plan_groups(needs: list[CacheNeed]) -> tuple[list[tuple[CacheNeed, list[int]
     return groups, group_of
 
 
+class _Requests:
+    """The live requests, looked up by the caller's request id: `requests[rid]` is a snapshot
+    (`RequestCache`) of what the request holds now."""
+
+    def __init__(self, manager: "CacheManager"):
+        self._manager = manager
+
+    def __contains__(self, rid) -> bool:
+        return rid in self._manager._ids
+
+    def __len__(self) -> int:
+        return len(self._manager._ids)
+
+    def __iter__(self):
+        return iter(list(self._manager._ids))
+
+    def __getitem__(self, rid) -> RequestCache:
+        manager = self._manager
+        handle = manager._handle_of(rid)
+        tables = [manager.table(rid, g) for g in range(len(manager.groups))]
+        return RequestCache(manager._lib.ta_cache_seq_len(manager._core, handle), tables,
+                            manager._lib.ta_cache_slot(manager._core, handle))
+
+    def values(self):
+        return [self[rid] for rid in self]
+
+
 class CacheManager:
     def __init__(self, needs: list[CacheNeed], num_pages: int, page_size: int = 16, max_requests: int = 8,
                  prefix_cache: bool = False):
         planned, self.group_of_layer = plan_groups(needs)
         self.page_size = page_size
         self.num_pages = num_pages
-        self.groups = [CacheGroup(need, layers, PageAllocator(num_pages, page_size)) for need, layers in planned]
         self.max_requests = max_requests
-        self._free_slots = list(range(max_requests - 1, -1, -1))
-        self.requests: dict[object, RequestCache] = {}
+        self._lib = _host.lib()
+        kinds = (ctypes.c_int32 * max(1, len(planned)))(*[1 if need.kind == "window" else 0 for need, _ in planned])
+        windows = (ctypes.c_int32 * max(1, len(planned)))(*[need.window if need.kind == "window" else -1
+                                                           for need, _ in planned])
+        self._core = self._lib.ta_cache_new(len(planned), kinds, windows, num_pages, page_size, max_requests,
+                                            1 if prefix_cache else 0)
+        if not self._core:
+            raise ValueError("num_pages and max_requests must not be negative and page_size must be positive")
+        self.groups = [CacheGroup(need, layers, PageAllocator(num_pages, page_size,
+                                                              _borrowed=self._lib.ta_cache_allocator(self._core, g)))
+                       for g, (need, layers) in enumerate(planned)]
         # Sharing a prefix needs every group to keep all positions (a window group drops pages).
-        self.prefix_cache = prefix_cache and all(g.need.kind == "full" for g in self.groups)
+        self.prefix_cache = bool(self._lib.ta_cache_prefix_enabled(self._core))
         self.state_layers = [i for i, need in enumerate(needs) if need.state_shape is not None]
+        self._ids: dict[object, int] = {}        # the caller's request id -> the core's handle
+        self._next_handle = 0
+        self.requests = _Requests(self)
+
+    def __del__(self):
+        if getattr(self, "_core", None):
+            self._lib.ta_cache_delete(self._core)
+            self._core = None
+
+    def _handle_of(self, rid) -> int:
+        return self._ids[rid]                     # KeyError for a request that is not live
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid) -> RequestCache:
-        if rid in self.requests:
+        if rid in self._ids:
             raise KeyError(f"request {rid!r} is already live")
-        if not self._free_slots:
+        handle = self._next_handle
+        slot = self._lib.ta_cache_add_request(self._core, handle)
+        if slot < 0:
             raise OutOfPages(f"all {self.max_requests} request slots are taken")
-        entry = RequestCache(0, [[] for _ in self.groups], self._free_slots.pop())
-        self.requests[rid] = entry
-        return entry
+        self._next_handle += 1
+        self._ids[rid] = handle
+        return RequestCache(0, [[] for _ in self.groups], slot)
 
     def has_request(self, rid) -> bool:
-        return rid in self.requests
+        return rid in self._ids
 
     def seq_len(self, rid) -> int:
-        return self.requests[rid].seq_len
+        return self._lib.ta_cache_seq_len(self._core, self._handle_of(rid))
 
     def slot(self, rid) -> int:
-        return self.requests[rid].slot
+        return self._lib.ta_cache_slot(self._core, self._handle_of(rid))
 
     def table(self, rid, group: int) -> list[int]:
-        return self.requests[rid].tables[group]
+        handle = self._handle_of(rid)
+        length = self._lib.ta_cache_table_len(self._core, handle, group)
+        out = (ctypes.c_int32 * max(1, length))()
+        self._lib.ta_cache_table(self._core, handle, group, out)
+        return list(out[:length])
 
     def free_slot_count(self) -> int:
-        return len(self._free_slots)
+        return self._lib.ta_cache_free_slots(self._core)
 
     # --------------------------------------------------------------------- pages
     def first_needed_position(self, group: int, seq_len: int) -> int:
         """Lowest key position any query at or past `seq_len` still reads in this group."""
-        need = self.groups[group].need
-        if need.kind == "window":
-            return max(0, seq_len - need.window)
-        return 0
+        return self._lib.ta_cache_first_needed_position(self._core, group, seq_len)
 
     def pages_missing(self, rid, new_len: int) -> list[int]:
         """Pages each group lacks for the request to hold `new_len` tokens."""
-        entry = self.requests[rid]
-        return [max(0, pages_for_len(new_len, self.page_size) - len(table)) for table in entry.tables]
+        out = (ctypes.c_int32 * max(1, len(self.groups)))()
+        self._lib.ta_cache_pages_missing(self._core, self._handle_of(rid), new_len, out)
+        return list(out[:len(self.groups)])
 
     def can_reserve(self, rid, new_len: int) -> bool:
-        return all(group.allocator.available() >= missing
-                   for group, missing in zip(self.groups, self.pages_missing(rid, new_len)))
+        return self._lib.ta_cache_can_reserve(self._core, self._handle_of(rid), new_len) == 1
 
     def reserve(self, rid, new_len: int) -> bool:
         """Give the request pages for `new_len` tokens in every group, or change nothing."""
-        missing = self.pages_missing(rid, new_len)
-        if not all(group.allocator.available() >= count for group, count in zip(self.groups, missing)):
-            return False
-        entry = self.requests[rid]
-        for group, table, count in zip(self.groups, entry.tables, missing):
-            table.extend(group.allocator.alloc_n(count))
-        return True
+        return self._lib.ta_cache_reserve(self._core, self._handle_of(rid), new_len) == 1
 
     def advance(self, rid, new_len: int) -> None:
         """The request now holds `new_len` tokens; window groups give back pages no query reads again."""
-        entry = self.requests[rid]
-        if new_len < entry.seq_len:
+        status = self._lib.ta_cache_advance(self._core, self._handle_of(rid), new_len)
+        if status == -4:
             raise ValueError("a request's length never shrinks")
-        if any(pages_for_len(new_len, self.page_size) > len(table) for table in entry.tables):
+        if status == -5:
             raise ValueError(f"request {rid!r} holds too few pages for {new_len} tokens")
-        entry.seq_len = new_len
-        for index, (group, table) in enumerate(zip(self.groups, entry.tables)):
-            if group.need.kind != "window":
-                continue
-            first = self.first_needed_position(index, new_len)
-            for page_index in range(first // self.page_size):
-                if table[page_index] >= 0:
-                    group.allocator.free_page(table[page_index])
-                    table[page_index] = -1
 
     def release(self, rid) -> None:
         """End a request: every page and its slot go back."""
-        entry = self.requests.pop(rid)
-        for group, table in zip(self.groups, entry.tables):
-            for page in table:
-                if page >= 0:
-                    group.allocator.free_page(page)
-        self._free_slots.append(entry.slot)
+        self._lib.ta_cache_release(self._core, self._ids.pop(rid))
 
     # -------------------------------------------------------------- prefix cache
     def attach_shared_prefix(self, rid, tokens) -> int:
@@ -155,57 +190,60 @@ class CacheManager:
         The last token is left out of the lookup so that the page it lands in stays private
         (qwen-server/src/engine.rs:490-495,519-527).  Only for a request that holds nothing yet.
         """
-        entry = self.requests[rid]
-        if not self.prefix_cache or entry.seq_len or any(entry.tables):
-            return 0
-        lookup = tokens[:-1] if len(tokens) else tokens
-        marks = [group.allocator.peak_mark() for group in self.groups]
-        taken = [group.allocator.take_shared_prefix(lookup) for group in self.groups]
-        count = min(len(pages) for pages in taken) if taken else 0
-        for group, pages, mark in zip(self.groups, taken, marks):
-            for page in pages[count:]:
-                group.allocator.free_page(page)
-            if len(pages) > count:
-                group.allocator.rewind_peaks(mark)
-        for table, pages in zip(entry.tables, taken):
-            table.extend(pages[:count])
-        entry.seq_len = count * self.page_size
-        return entry.seq_len
+        keep, pointer = _host.token_array(tokens)
+        return self._lib.ta_cache_attach_shared_prefix(self._core, self._handle_of(rid), pointer, len(keep))
 
     def detach(self, rid) -> None:
         """Give back everything a request holds but keep it known (used when an admission is rolled back)."""
-        entry = self.requests[rid]
-        for group, table in zip(self.groups, entry.tables):
-            for page in table:
-                if page >= 0:
-                    group.allocator.free_page(page)
-            table.clear()
-        entry.seq_len = 0
+        self._lib.ta_cache_detach(self._core, self._handle_of(rid))
 
     def publish(self, rid, tokens) -> None:
         """Make the full, written pages of `tokens` findable by later requests."""
         if not self.prefix_cache:
             return
-        entry = self.requests[rid]
-        written = tokens[:entry.seq_len]
-        for group, table in zip(self.groups, entry.tables):
-            group.allocator.publish_prompt_pages(written, table)
+        keep, pointer = _host.token_array(tokens)
+        self._lib.ta_cache_publish(self._core, self._handle_of(rid), pointer, len(keep))
+
+    # ------------------------------------------------------------------- packing
+    def pack_batch(self, rids, token_lists, want_lists, out: np.ndarray, table_width: int | None = None):
+        """Write one step's batch description into the int32 array `out` (see `engine/batch.py` for the
+        order of its parts).  Returns (total length, the parts' lengths, the table width per group, and per
+        entry its first row, token count, first position and state slot)."""
+        n = len(rids)
+        ids = np.array([self._handle_of(rid) for rid in rids], dtype=np.int64)
+        n_tokens = np.array([len(t) for t in token_lists], dtype=np.int32)
+        n_want = np.array([len(w) for w in want_lists], dtype=np.int32)
+        tokens = np.fromiter((t for ts in token_lists for t in ts), dtype=np.int32, count=int(n_tokens.sum()))
+        want = np.fromiter((w for ws in want_lists for w in ws), dtype=np.int32, count=int(n_want.sum()))
+        n_groups = len(self.groups)
+        sizes = np.zeros(9 + 2 * n_groups, dtype=np.int64)
+        widths = np.zeros(max(1, n_groups), dtype=np.int32)
+        info = np.zeros(max(1, 4 * n), dtype=np.int32)
+        as_i32 = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+        as_i64 = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int64))
+        total = self._lib.ta_cache_pack_batch(self._core, n, as_i64(ids), as_i32(n_tokens), as_i32(tokens),
+                                              as_i32(n_want), as_i32(want),
+                                              -1 if table_width is None else table_width, as_i32(out), out.size,
+                                              as_i64(sizes), as_i32(widths), as_i32(info))
+        if total == -6:
+            raise RuntimeError("a request writes a position into a page it gave back")
+        if total == -7:
+            raise ValueError("a block table is wider than the fixed width")
+        if total == -8:
+            raise ValueError("the packed batch does not fit the buffers it should land in")
+        if total < 0:
+            raise RuntimeError(f"the batch could not be packed (status {total})")
+        return int(total), sizes.tolist(), widths[:n_groups].tolist(), info[:4 * n].reshape(n, 4).tolist()
+
+    def packed_size(self, token_counts, want_counts, table_widths) -> int:
+        """Length of the packed description of a batch with these token and want counts and table widths."""
+        n, tokens = len(token_counts), sum(token_counts)
+        tiles = sum(-(-c // 16) for c in token_counts if c != 1)
+        single = sum(1 for c in token_counts if c == 1)
+        return (3 * tokens + (n + 1) + 2 * n + sum(want_counts) + 2 * tiles + single
+                + sum(tokens + n * w for w in table_widths))
 
     # ------------------------------------------------------------------ checking
     def check_invariants(self) -> None:
         """No page lost, held twice or freed twice; slots likewise."""
-        for index, group in enumerate(self.groups):
-            group.allocator.check_invariants()
-            held: dict[int, int] = {}
-            for entry in self.requests.values():
-                for page in entry.tables[index]:
-                    if page >= 0:
-                        held[page] = held.get(page, 0) + 1
-            for page in range(group.allocator.capacity()):
-                assert group.allocator.refcount(page) == held.get(page, 0), \
-                    f"group {index} page {page}: count {group.allocator.refcount(page)}, held {held.get(page, 0)}"
-            assert (group.allocator.free_count() + group.allocator.cached_count()
-                    + group.allocator.live_count() == group.allocator.capacity())
-        slots = [entry.slot for entry in self.requests.values()]
-        assert len(set(slots)) == len(slots), "a slot is held twice"
-        assert sorted(slots + self._free_slots) == list(range(self.max_requests)), "a slot was lost"
+        assert self._lib.ta_cache_check(self._core) == 0, _host.message()

@@ -1,0 +1,157 @@
+// C entry points of the host library (bound from Python through ctypes).  Objects are opaque pointers;
+// functions return a status or a value as their headers say; `ta_host_message` holds the text of the last
+// failed check of the calling thread.
+#include <cstring>
+#include <string>
+
+#include "cache_core.h"
+#include "page_allocator.h"
+#include "sampler.h"
+
+using namespace ta;
+
+static thread_local std::string g_message;
+
+extern "C" {
+
+const char* ta_host_message() { return g_message.c_str(); }
+
+// ---------------------------------------------------------------------------------------- allocator
+void* ta_alloc_new(int num_pages, int page_size) {
+  if (num_pages < 0 || page_size <= 0) return nullptr;
+  return new PageAllocator(num_pages, page_size);
+}
+void ta_alloc_delete(void* a) { delete (PageAllocator*)a; }
+// what: 0 capacity, 1 free, 2 cached, 3 available, 4 live, 5 occupied, 6 refcount(arg), 7 all counts zero,
+// 8 peak live, 9 peak occupied, 10 page size.
+int ta_alloc_get(void* a, int what, int arg) {
+  const PageAllocator& p = *(PageAllocator*)a;
+  switch (what) {
+    case 0: return p.capacity();
+    case 1: return p.free_count();
+    case 2: return p.cached_count();
+    case 3: return p.available();
+    case 4: return p.live_count();
+    case 5: return p.occupied();
+    case 6: return p.refcount(arg);
+    case 7: return p.all_refcounts_zero() ? 1 : 0;
+    case 8: return p.peak_live();
+    case 9: return p.peak_occupied();
+    case 10: return p.page_size();
+    default: return -1;
+  }
+}
+void ta_alloc_rewind_peaks(void* a, int live, int occupied) { ((PageAllocator*)a)->rewind_peaks(live, occupied); }
+int ta_alloc_alloc(void* a) { return ((PageAllocator*)a)->alloc(); }
+// `count` pages into out, or none: returns 1 or 0.
+int ta_alloc_alloc_n(void* a, int count, int* out) {
+  std::vector<int> pages;
+  if (!((PageAllocator*)a)->alloc_n(count, &pages)) return 0;
+  std::copy(pages.begin(), pages.end(), out);
+  return 1;
+}
+int ta_alloc_free(void* a, int page, int* how) { return ((PageAllocator*)a)->free_page(page, how); }
+int ta_alloc_incref(void* a, int page) { return ((PageAllocator*)a)->incref(page); }
+uint64_t ta_prefix_page_hash(uint64_t parent, const int32_t* tokens, int count) {
+  return prefix_page_hash(parent, tokens, count);
+}
+int ta_alloc_publish_full_page(void* a, uint64_t parent_hash, const int32_t* tokens, int count, int page) {
+  return ((PageAllocator*)a)->publish_full_page(parent_hash, tokens, count, page);
+}
+int ta_alloc_find_full_page(void* a, uint64_t parent_hash, int parent_page, const int32_t* tokens, int count) {
+  return ((PageAllocator*)a)->find_full_page(parent_hash, parent_page, tokens, count);
+}
+int ta_alloc_publish_at(void* a, uint64_t value, uint64_t parent_hash, int parent_page, const int32_t* tokens,
+                        int count, int page) {
+  PageAllocator& p = *(PageAllocator*)a;
+  if (count != p.page_size() || p.refcount(page) < 0) return 0;
+  return p.publish_at(value, parent_hash, parent_page, tokens, page) ? 1 : 0;
+}
+int ta_alloc_find_at(void* a, uint64_t value, uint64_t parent_hash, int parent_page, const int32_t* tokens, int count) {
+  const PageAllocator& p = *(PageAllocator*)a;
+  return count == p.page_size() ? p.find_at(value, parent_hash, parent_page, tokens) : -1;
+}
+// Pages into out (room for count / page_size); returns how many.
+int ta_alloc_take_shared_prefix(void* a, const int32_t* tokens, int count, int* out) {
+  std::vector<int> pages;
+  ((PageAllocator*)a)->take_shared_prefix(tokens, count, &pages);
+  std::copy(pages.begin(), pages.end(), out);
+  return (int)pages.size();
+}
+void ta_alloc_publish_prompt_pages(void* a, const int32_t* tokens, int count, const int* pages, int n_pages) {
+  ((PageAllocator*)a)->publish_prompt_pages(tokens, count, pages, n_pages);
+}
+void ta_alloc_reclaim_cached(void* a) { ((PageAllocator*)a)->reclaim_cached(); }
+// 0 when all is well, else 1 with the finding in ta_host_message().
+int ta_alloc_check(void* a) {
+  g_message = ((PageAllocator*)a)->check_invariants();
+  return g_message.empty() ? 0 : 1;
+}
+
+// ------------------------------------------------------------------------------------------- cache
+void* ta_cache_new(int n_groups, const int* kinds, const int* windows, int num_pages, int page_size,
+                   int max_requests, int prefix_cache) {
+  if (n_groups < 0 || num_pages < 0 || page_size <= 0 || max_requests < 0) return nullptr;
+  return new CacheCore(n_groups, kinds, windows, num_pages, page_size, max_requests, prefix_cache != 0);
+}
+void ta_cache_delete(void* c) { delete (CacheCore*)c; }
+void* ta_cache_allocator(void* c, int group) { return ((CacheCore*)c)->allocator(group); }   // borrowed
+int ta_cache_prefix_enabled(void* c) { return ((CacheCore*)c)->prefix_cache() ? 1 : 0; }
+int ta_cache_n_requests(void* c) { return ((CacheCore*)c)->n_requests(); }
+int ta_cache_free_slots(void* c) { return ((CacheCore*)c)->free_slot_count(); }
+int ta_cache_add_request(void* c, int64_t id) { return ((CacheCore*)c)->add_request(id); }
+int ta_cache_has_request(void* c, int64_t id) { return ((const CacheCore*)c)->find(id) ? 1 : 0; }
+int ta_cache_seq_len(void* c, int64_t id) {
+  const Request* r = ((const CacheCore*)c)->find(id);
+  return r ? r->seq_len : CACHE_UNKNOWN_REQUEST;
+}
+int ta_cache_slot(void* c, int64_t id) {
+  const Request* r = ((const CacheCore*)c)->find(id);
+  return r ? r->slot : CACHE_UNKNOWN_REQUEST;
+}
+int ta_cache_table_len(void* c, int64_t id, int group) {
+  const Request* r = ((const CacheCore*)c)->find(id);
+  return r ? (int)r->tables[group].size() : CACHE_UNKNOWN_REQUEST;
+}
+int ta_cache_table(void* c, int64_t id, int group, int* out) {
+  const Request* r = ((const CacheCore*)c)->find(id);
+  if (!r) return CACHE_UNKNOWN_REQUEST;
+  std::copy(r->tables[group].begin(), r->tables[group].end(), out);
+  return (int)r->tables[group].size();
+}
+int ta_cache_first_needed_position(void* c, int group, int seq_len) {
+  return ((CacheCore*)c)->first_needed_position(group, seq_len);
+}
+int ta_cache_pages_missing(void* c, int64_t id, int new_len, int* per_group) {
+  return ((CacheCore*)c)->pages_missing(id, new_len, per_group);
+}
+int ta_cache_can_reserve(void* c, int64_t id, int new_len) { return ((CacheCore*)c)->can_reserve(id, new_len); }
+int ta_cache_reserve(void* c, int64_t id, int new_len) { return ((CacheCore*)c)->reserve(id, new_len); }
+int ta_cache_advance(void* c, int64_t id, int new_len) { return ((CacheCore*)c)->advance(id, new_len); }
+int ta_cache_release(void* c, int64_t id) { return ((CacheCore*)c)->release(id); }
+int ta_cache_detach(void* c, int64_t id) { return ((CacheCore*)c)->detach(id); }
+int ta_cache_attach_shared_prefix(void* c, int64_t id, const int32_t* tokens, int count) {
+  return ((CacheCore*)c)->attach_shared_prefix(id, tokens, count);
+}
+int ta_cache_publish(void* c, int64_t id, const int32_t* tokens, int count) {
+  return ((CacheCore*)c)->publish(id, tokens, count);
+}
+int ta_cache_check(void* c) {
+  g_message = ((CacheCore*)c)->check_invariants();
+  return g_message.empty() ? 0 : 1;
+}
+int64_t ta_cache_pack_batch(void* c, int n_entries, const int64_t* ids, const int* n_tokens, const int32_t* tokens,
+                            const int* n_want, const int* want, int table_width, int32_t* out, int64_t capacity,
+                            int64_t* sizes, int* widths, int* entry_info) {
+  return ((CacheCore*)c)->pack_batch(n_entries, ids, n_tokens, tokens, n_want, want, table_width, out, capacity,
+                                     sizes, widths, entry_info);
+}
+
+// ----------------------------------------------------------------------------------------- sampling
+float ta_uniform_f32(uint64_t seed, uint64_t counter) { return uniform_f32(seed, counter); }
+int ta_greedy_token(const float* logits, int64_t count) { return greedy_token(logits, count); }
+int ta_sample_with_uniform(const float* logits, int64_t count, float temperature, float top_p, float uniform) {
+  return sample_with_uniform(logits, count, temperature, top_p, uniform);
+}
+
+}  // extern "C"

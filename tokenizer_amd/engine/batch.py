@@ -3,7 +3,6 @@ from __future__ import annotations
 
 import dataclasses
 
-import numpy as np
 import torch
 
 
@@ -57,65 +56,28 @@ def build_context(entries: list[StepEntry], manager, device, table_width: int | 
     """
     page_size = manager.page_size
     n_groups = len(manager.groups)
-    token_ids, positions, entry_of_token, want_rows = [], [], [], []
-    cu_q, first_position, state_slots, infos = [0], [], [], []
-    slots = [[] for _ in range(n_groups)]
-    tables = [[] for _ in range(n_groups)]
-    for index, entry in enumerate(entries):
-        start = manager.seq_len(entry.rid)
-        count = len(entry.tokens)
-        row0 = len(token_ids)
-        token_ids.extend(entry.tokens)
-        positions.extend(range(start, start + count))
-        entry_of_token.extend([index] * count)
-        want_rows.extend(row0 + w for w in entry.want)
-        cu_q.append(row0 + count)
-        first_position.append(start)
-        state_slots.append(manager.slot(entry.rid))
-        infos.append(EntryInfo(entry.rid, row0, count, start, manager.slot(entry.rid)))
-        for g in range(n_groups):
-            table = manager.table(entry.rid, g)
-            tables[g].append(table)
-            for p in range(start, start + count):
-                page = table[p // page_size]
-                if page < 0:
-                    raise RuntimeError(f"request {entry.rid!r} writes position {p} into a page it gave back")
-                slots[g].append(page * page_size + p % page_size)
-    q_tiles, decode_rows = [], []
-    for index, info in enumerate(infos):
-        if info.q_len == 1:
-            decode_rows.append(info.q_start)
-        else:
-            for offset in range(0, info.q_len, 16):
-                q_tiles.extend((index, offset))
-    n_tokens, n_entries = len(token_ids), len(entries)
-    widths = [max(1, max((len(t) for t in tables[g]), default=1)) for g in range(n_groups)]
-    if table_width is not None:
-        if any(width > table_width for width in widths):
-            raise ValueError("a block table is wider than the fixed width")
-        widths = [table_width] * n_groups
-    parts = [token_ids, positions, entry_of_token, cu_q, first_position, state_slots, want_rows, q_tiles,
-             decode_rows]
-    for g in range(n_groups):
-        parts.append(slots[g])
-        flat = np.full((n_entries, widths[g]), -1, dtype=np.int32)
-        for row, table in enumerate(tables[g]):
-            flat[row, :len(table)] = table
-        parts.append(flat.reshape(-1))
-    sizes = [len(p) for p in parts]
-    packed = np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in parts]) if sum(sizes) else \
-        np.zeros(0, dtype=np.int32)
+    rids = [entry.rid for entry in entries]
+    token_lists = [entry.tokens for entry in entries]
+    want_lists = [entry.want for entry in entries]
     if into is not None:
         host, dev = into
-        if host.numel() != packed.size:
-            raise ValueError("the packed batch does not fit the buffers it should land in")
-        host.numpy()[:] = packed
-        dev.copy_(host, non_blocking=True)
     else:
-        host = torch.from_numpy(packed)
+        # The packing itself is the cache manager's (C++); what is needed here is the buffer's size.
+        widths = [table_width if table_width is not None else
+                  max([1] + [len(manager.table(rid, g)) for rid in rids]) for g in range(n_groups)]
+        size = manager.packed_size([len(t) for t in token_lists], [len(w) for w in want_lists], widths)
+        host = torch.empty(size, dtype=torch.int32)
         if torch.device(device).type == "cuda":
             host = host.pin_memory()
+    total, sizes, widths, info = manager.pack_batch(rids, token_lists, want_lists, host.numpy(), table_width)
+    if total != host.numel():
+        raise ValueError("the packed batch does not fit the buffers it should land in")
+    if into is not None:
+        dev.copy_(host, non_blocking=True)
+    else:
         dev = host.to(device, non_blocking=True)
+    infos = [EntryInfo(rid, row, count, start, slot) for rid, (row, count, start, slot) in zip(rids, info)]
+    n_tokens, n_entries = sizes[0], len(entries)
     views, offset = [], 0
     for size in sizes:
         views.append(dev[offset:offset + size])

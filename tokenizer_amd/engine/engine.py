@@ -92,51 +92,19 @@ class DecodeGraph:
         with torch.cuda.graph(self.graph, pool=engine.graph_pool):
             self.logits = engine.model.decoder.forward(self.ctx, engine.layer_caches)
             self.ids = ops.argmax(self.logits)
-
-    def _views(self, n_entries: int, n_groups: int) -> None:
-        """Numpy views into the pinned buffer, in the packing order of `build_context` (one token per entry)."""
-        flat = self.host.numpy()
-        sizes = [n_entries, n_entries, n_entries, n_entries + 1, n_entries, n_entries, n_entries, 0, n_entries]
-        for _ in range(n_groups):
-            sizes += [n_entries, n_entries * self.width]
-        views, offset = [], 0
-        for size in sizes:
-            views.append(flat[offset:offset + size])
-            offset += size
-        self.v_tokens, self.v_positions, self.v_first, self.v_state = views[0], views[1], views[4], views[5]
-        self.v_slots = [views[9 + 2 * g] for g in range(n_groups)]
-        self.v_tables = [views[10 + 2 * g].reshape(n_entries, self.width) for g in range(n_groups)]
-        self.row_owner = [[None] * n_entries for _ in range(n_groups)]   # whose pages a table row holds
-        self.row_len = [[0] * n_entries for _ in range(n_groups)]
-        self.uploaded = torch.cuda.Event()
+        self.uploaded = None
 
     def run(self, engine: "Engine", entries: list[StepEntry]) -> torch.Tensor:
-        """Refill the batch's tables in place (only what changed since the last replay) and replay."""
+        """Pack the batch's description into the fixed buffers again and replay."""
+        if self.uploaded is not None:
+            self.uploaded.synchronize()                 # the last upload has left the pinned buffer
+        else:
+            self.uploaded = torch.cuda.Event()
         manager = engine.cache
-        if not hasattr(self, "v_tokens"):
-            self._views(len(entries), len(manager.groups))
-            self.uploaded.record()
-        self.uploaded.synchronize()                     # the last upload has left the pinned buffer
-        page_size = manager.page_size
-        windowed = [group.need.kind == "window" for group in manager.groups]
-        for i, entry in enumerate(entries):
-            held = manager.requests[entry.rid]
-            pos = held.seq_len
-            self.v_tokens[i] = entry.tokens[0]
-            self.v_positions[i] = pos
-            self.v_first[i] = pos
-            self.v_state[i] = held.slot
-            for g, table in enumerate(held.tables):
-                self.v_slots[g][i] = table[pos // page_size] * page_size + pos % page_size
-                count, row = len(table), self.v_tables[g][i]
-                if self.row_owner[g][i] is held and not windowed[g] and self.row_len[g][i] <= count:
-                    if self.row_len[g][i] < count:
-                        row[self.row_len[g][i]:count] = table[self.row_len[g][i]:]
-                else:
-                    row[:count] = table
-                    row[count:] = -1
-                    self.row_owner[g][i] = held
-                self.row_len[g][i] = count
+        total, _, _, _ = manager.pack_batch([e.rid for e in entries], [e.tokens for e in entries],
+                                            [e.want for e in entries], self.host.numpy(), self.width)
+        if total != self.host.numel():
+            raise ValueError("the packed batch does not fit the graph's buffers")
         self.dev.copy_(self.host, non_blocking=True)
         self.uploaded.record()
         self.graph.replay()

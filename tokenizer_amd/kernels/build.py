@@ -1,8 +1,9 @@
-"""Compile the HIP sources under `csrc/` for gfx950 into one shared library.
+"""Compile the sources under `csrc/` into two shared libraries.
 
-`hipcc` turns each `.hip` file into an object (in parallel), then links them.
-The library lands beside this package when that folder can be written, else in
-a per-user folder under the temporary directory.
+The HIP kernels (`csrc/*.hip`): `hipcc` turns each file into an object for gfx950 (in parallel), then links
+them.  The host core (`csrc/host/*.cpp`: page allocator, cache manager, batch packing, host sampler): one
+call of the C++ compiler, no GPU code and no dependency on HIP.  A library lands beside this package when
+that folder can be written, else in a per-user folder under the temporary directory.
 """
 from __future__ import annotations
 
@@ -18,6 +19,9 @@ import time
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SOURCE_DIR = os.path.join(PACKAGE_DIR, "csrc")
 LIB_NAME = "libtokenizer_amd_kernels.so"
+HOST_LIB_NAME = "libtokenizer_amd_host.so"
+HOST_SOURCE_DIR = os.path.join(SOURCE_DIR, "host")
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra"]
 ARCH = "gfx950"
 # Packed float32 instructions are switched off for all device code.
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
@@ -40,20 +44,20 @@ def hipcc_path() -> str:
                        "the HIP kernels cannot be built")
 
 
-def library_candidates() -> list[str]:
+def library_candidates(name: str = LIB_NAME) -> list[str]:
     fallback = os.path.join(tempfile.gettempdir(), f"tokenizer_amd_{os.getuid()}")
-    return [os.path.join(PACKAGE_DIR, LIB_NAME), os.path.join(fallback, LIB_NAME)]
+    return [os.path.join(PACKAGE_DIR, name), os.path.join(fallback, name)]
 
 
-def find_library() -> str | None:
-    for path in library_candidates():
+def find_library(name: str = LIB_NAME) -> str | None:
+    for path in library_candidates(name):
         if os.path.exists(path):
             return path
     return None
 
 
-def _writable_target() -> str:
-    for path in library_candidates():
+def _writable_target(name: str = LIB_NAME) -> str:
+    for path in library_candidates(name):
         folder = os.path.dirname(path)
         try:
             os.makedirs(folder, exist_ok=True)
@@ -113,5 +117,45 @@ def build_library(verbose: bool = True) -> str:
     return target
 
 
+def host_compiler() -> str:
+    for candidate in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                      "/opt/rocm/lib/llvm/bin/clang++"):
+        if candidate and (os.path.exists(candidate) or shutil.which(candidate)):
+            return candidate
+    raise RuntimeError("no C++ compiler was found (looked at $CXX, g++, c++, clang++); the host library cannot be built")
+
+
+def host_sources() -> list[str]:
+    return sorted(glob.glob(os.path.join(HOST_SOURCE_DIR, "*.cpp")))
+
+
+def find_host_library() -> str | None:
+    """A built host library that is not older than its sources."""
+    path = find_library(HOST_LIB_NAME)
+    if path is None:
+        return None
+    newest = max((os.path.getmtime(f) for f in glob.glob(os.path.join(HOST_SOURCE_DIR, "*"))), default=0.0)
+    return path if os.path.getmtime(path) >= newest else None
+
+
+def build_host_library(verbose: bool = True) -> str:
+    """Compile the host core; returns the library's path."""
+    sources = host_sources()
+    if not sources:
+        raise RuntimeError(f"no C++ sources under {HOST_SOURCE_DIR}")
+    compiler, target = host_compiler(), _writable_target(HOST_LIB_NAME)
+    started = time.time()
+    partial = target + f".{os.getpid()}.tmp"
+    proc = subprocess.run([compiler, *HOST_FLAGS, "-I", HOST_SOURCE_DIR, *sources, "-o", partial],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"compiling the host library failed:\n{proc.stderr[-4000:]}")
+    os.replace(partial, target)
+    if verbose:
+        _say(f"built {target} in {time.time() - started:.1f} s")
+    return target
+
+
 if __name__ == "__main__":
+    build_host_library()
     build_library()
