@@ -62,6 +62,13 @@ def plan_groups(needs: list[CacheNeed]) -> tuple[list[tuple[CacheNeed, list[int]
     return groups, group_of
 
 
+_FIRST_NAMED = 1 << 62      # handles of requests whose id is not a small non-negative integer
+
+
+def _is_handle(rid) -> bool:
+    return isinstance(rid, int) and not isinstance(rid, bool) and 0 <= rid < _FIRST_NAMED
+
+
 class _Requests:
     """The live requests, looked up by the caller's request id: `requests[rid]` is a snapshot
     (`RequestCache`) of what the request holds now."""
@@ -70,13 +77,17 @@ class _Requests:
         self._manager = manager
 
     def __contains__(self, rid) -> bool:
-        return rid in self._manager._ids
+        return self._manager.has_request(rid)
 
     def __len__(self) -> int:
-        return len(self._manager._ids)
+        return self._manager._lib.ta_cache_n_requests(self._manager._core)
 
     def __iter__(self):
-        return iter(list(self._manager._ids))
+        manager = self._manager
+        out = (ctypes.c_int64 * max(1, len(self)))()
+        count = manager._lib.ta_cache_request_ids(manager._core, out)
+        names = {handle: rid for rid, handle in manager._ids.items()}
+        return iter([names.get(handle, handle) for handle in out[:count]])
 
     def __getitem__(self, rid) -> RequestCache:
         manager = self._manager
@@ -110,8 +121,10 @@ class CacheManager:
         # Sharing a prefix needs every group to keep all positions (a window group drops pages).
         self.prefix_cache = bool(self._lib.ta_cache_prefix_enabled(self._core))
         self.state_layers = [i for i, need in enumerate(needs) if need.state_shape is not None]
-        self._ids: dict[object, int] = {}        # the caller's request id -> the core's handle
-        self._next_handle = 0
+        # A request id that is a small non-negative integer is its own handle in the core (so the scheduler core,
+        # which numbers its sequences, and this class speak of the same requests); any other id gets one here.
+        self._ids: dict[object, int] = {}
+        self._next_handle = _FIRST_NAMED
         self.requests = _Requests(self)
 
     def __del__(self):
@@ -120,21 +133,29 @@ class CacheManager:
             self._core = None
 
     def _handle_of(self, rid) -> int:
-        return self._ids[rid]                     # KeyError for a request that is not live
+        """The core's handle of a live request; KeyError for one that is not live."""
+        if _is_handle(rid):
+            if not self._lib.ta_cache_has_request(self._core, rid):
+                raise KeyError(rid)
+            return rid
+        return self._ids[rid]
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid) -> RequestCache:
-        if rid in self._ids:
+        if self.has_request(rid):
             raise KeyError(f"request {rid!r} is already live")
-        handle = self._next_handle
+        handle = rid if _is_handle(rid) else self._next_handle
         slot = self._lib.ta_cache_add_request(self._core, handle)
         if slot < 0:
             raise OutOfPages(f"all {self.max_requests} request slots are taken")
-        self._next_handle += 1
-        self._ids[rid] = handle
+        if not _is_handle(rid):
+            self._next_handle += 1
+            self._ids[rid] = handle
         return RequestCache(0, [[] for _ in self.groups], slot)
 
     def has_request(self, rid) -> bool:
+        if _is_handle(rid):
+            return bool(self._lib.ta_cache_has_request(self._core, rid))
         return rid in self._ids
 
     def seq_len(self, rid) -> int:
@@ -181,7 +202,9 @@ class CacheManager:
 
     def release(self, rid) -> None:
         """End a request: every page and its slot go back."""
-        self._lib.ta_cache_release(self._core, self._ids.pop(rid))
+        handle = self._handle_of(rid)
+        self._ids.pop(rid, None)
+        self._lib.ta_cache_release(self._core, handle)
 
     # -------------------------------------------------------------- prefix cache
     def attach_shared_prefix(self, rid, tokens) -> int:
@@ -210,7 +233,7 @@ class CacheManager:
         order of its parts).  Returns (total length, the parts' lengths, the table width per group, and per
         entry its first row, token count, first position and state slot)."""
         n = len(rids)
-        ids = np.array([self._handle_of(rid) for rid in rids], dtype=np.int64)
+        ids = np.array([rid if _is_handle(rid) else self._ids[rid] for rid in rids], dtype=np.int64)
         n_tokens = np.array([len(t) for t in token_lists], dtype=np.int32)
         n_want = np.array([len(w) for w in want_lists], dtype=np.int32)
         tokens = np.fromiter((t for ts in token_lists for t in ts), dtype=np.int32, count=int(n_tokens.sum()))
@@ -225,6 +248,8 @@ class CacheManager:
                                               as_i32(n_want), as_i32(want),
                                               -1 if table_width is None else table_width, as_i32(out), out.size,
                                               as_i64(sizes), as_i32(widths), as_i32(info))
+        if total == -3:
+            raise KeyError("a request of the batch is not live")
         if total == -6:
             raise RuntimeError("a request writes a position into a page it gave back")
         if total == -7:

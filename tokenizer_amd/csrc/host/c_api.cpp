@@ -7,6 +7,7 @@
 #include "cache_core.h"
 #include "page_allocator.h"
 #include "sampler.h"
+#include "scheduler_core.h"
 
 using namespace ta;
 
@@ -99,6 +100,8 @@ void* ta_cache_allocator(void* c, int group) { return ((CacheCore*)c)->allocator
 int ta_cache_prefix_enabled(void* c) { return ((CacheCore*)c)->prefix_cache() ? 1 : 0; }
 int ta_cache_n_requests(void* c) { return ((CacheCore*)c)->n_requests(); }
 int ta_cache_free_slots(void* c) { return ((CacheCore*)c)->free_slot_count(); }
+// The ids of the live requests into out (room for ta_cache_n_requests); returns how many.
+int ta_cache_request_ids(void* c, int64_t* out) { return ((CacheCore*)c)->request_ids(out); }
 int ta_cache_add_request(void* c, int64_t id) { return ((CacheCore*)c)->add_request(id); }
 int ta_cache_has_request(void* c, int64_t id) { return ((const CacheCore*)c)->find(id) ? 1 : 0; }
 int ta_cache_seq_len(void* c, int64_t id) {
@@ -146,6 +149,70 @@ int64_t ta_cache_pack_batch(void* c, int n_entries, const int64_t* ids, const in
   return ((CacheCore*)c)->pack_batch(n_entries, ids, n_tokens, tokens, n_want, want, table_width, out, capacity,
                                      sizes, widths, entry_info);
 }
+
+// ---------------------------------------------------------------------------------------- scheduler
+void* ta_sched_new(void* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk) {
+  if (!cache || max_batch_size <= 0 || token_budget <= 0) return nullptr;
+  return new SchedulerCore((CacheCore*)cache, num_pages, max_batch_size, token_budget, prefill_chunk);
+}
+void ta_sched_delete(void* s) { delete (SchedulerCore*)s; }
+int ta_sched_enqueue(void* s, int64_t id, const int32_t* prompt, int count) {
+  return ((SchedulerCore*)s)->enqueue(id, prompt, count);
+}
+int ta_sched_append_token(void* s, int64_t id, int32_t token) { return ((SchedulerCore*)s)->append_token(id, token); }
+// what: 0 running, 1 waiting, 2 most running at once, 3 preemptions, 4 last preempted id, 5 front of the queue
+// (-1: empty), 6 pages to admit `id`, 7 tokens of `id` in the cache, 8 tokens `id` holds, 9 whether `id` runs.
+int64_t ta_sched_get(void* s, int what, int64_t id) {
+  const SchedulerCore& core = *(SchedulerCore*)s;
+  const Sequence* seq = what >= 7 ? core.find(id) : nullptr;
+  switch (what) {
+    case 0: return core.n_running();
+    case 1: return core.n_waiting();
+    case 2: return core.max_running();
+    case 3: return core.preemptions();
+    case 4: return core.last_preempted_id();
+    case 5: return core.front_waiting();
+    case 6: return core.pages_to_admit(id);
+    case 7: return seq ? seq->computed : -1;
+    case 8: return seq ? (int64_t)seq->tokens.size() : -1;
+    case 9: return seq ? (seq->running ? 1 : 0) : -1;
+    default: return -1;
+  }
+}
+// planned: rows of (id, first token, count, completes); preempted: ids; failed: rows of (id, pages needed).
+// Each array has room for `room` rows.  Returns 0, or -1 if a list did not fit (nothing is lost: the lists are
+// never longer than the number of sequences the scheduler knows, which the caller passes as `room`).
+int ta_sched_plan_step(void* s, int room, int64_t* planned, int* n_planned, int64_t* preempted, int* n_preempted,
+                       int64_t* failed, int* n_failed) {
+  std::vector<PlannedEntry> plan;
+  std::vector<int64_t> out;
+  std::vector<FailedEntry> fail;
+  ((SchedulerCore*)s)->plan_step(&plan, &out, &fail);
+  *n_planned = (int)plan.size(); *n_preempted = (int)out.size(); *n_failed = (int)fail.size();
+  if ((int)plan.size() > room || (int)out.size() > room || (int)fail.size() > room) return -1;
+  for (size_t i = 0; i < plan.size(); ++i) {
+    planned[4 * i] = plan[i].id; planned[4 * i + 1] = plan[i].first; planned[4 * i + 2] = plan[i].count;
+    planned[4 * i + 3] = plan[i].completes ? 1 : 0;
+  }
+  std::copy(out.begin(), out.end(), preempted);
+  for (size_t i = 0; i < fail.size(); ++i) { failed[2 * i] = fail[i].id; failed[2 * i + 1] = fail[i].pages_needed; }
+  return 0;
+}
+// The running (which = 0, in order of admission) or waiting (1, front first) ids into out; returns how many.
+int ta_sched_list(void* s, int which, int64_t* out) {
+  const SchedulerCore& core = *(SchedulerCore*)s;
+  if (which == 0) { std::copy(core.running().begin(), core.running().end(), out); return (int)core.running().size(); }
+  std::copy(core.waiting().begin(), core.waiting().end(), out);
+  return (int)core.waiting().size();
+}
+int ta_sched_tokens(void* s, int64_t id, int first, int count, int32_t* out) {
+  const Sequence* seq = ((const SchedulerCore*)s)->find(id);
+  if (!seq || first < 0 || count < 0 || first + count > (int)seq->tokens.size()) return -1;
+  std::copy(seq->tokens.begin() + first, seq->tokens.begin() + first + count, out);
+  return count;
+}
+int ta_sched_commit(void* s, int64_t id, int count) { return ((SchedulerCore*)s)->commit(id, count); }
+int ta_sched_finish(void* s, int64_t id) { return ((SchedulerCore*)s)->finish(id); }
 
 // ----------------------------------------------------------------------------------------- sampling
 float ta_uniform_f32(uint64_t seed, uint64_t counter) { return uniform_f32(seed, counter); }

@@ -24,6 +24,13 @@ const Request* CacheCore::find(int64_t id) const {
   return found == requests_.end() ? nullptr : &found->second;
 }
 
+int CacheCore::request_ids(int64_t* out) const {
+  int count = 0;
+  for (const auto& item : requests_) out[count++] = item.first;
+  std::sort(out, out + count);
+  return count;
+}
+
 Request* CacheCore::find(int64_t id) {
   auto found = requests_.find(id);
   return found == requests_.end() ? nullptr : &found->second;

@@ -43,6 +43,7 @@ class CacheCore {
   int n_requests() const { return (int)requests_.size(); }
   int free_slot_count() const { return (int)free_slots_.size(); }
   const Request* find(int64_t id) const;
+  int request_ids(int64_t* out) const;
 
   int add_request(int64_t id);                            // the slot, or a CacheStatus
   int first_needed_position(int group, int seq_len) const;

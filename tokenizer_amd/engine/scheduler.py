@@ -11,15 +11,19 @@ Beyond the reference, one iteration is a single mixed batch under a token budget
 for every decoding sequence first, then portions of prompts in order of arrival.  A preempted
 sequence is recomputed from its prompt and the tokens it sampled so far, and nothing is
 sampled again for positions that already have a token.
+
+The decisions (queue, admission, plan, preemption, every exchange with the cache manager) are
+made by the C++ scheduler core (`csrc/host/scheduler_core.cpp`), which also owns the token lists;
+this class runs the plan through the engine, samples, keeps stop conditions, texts and results.
 """
 from __future__ import annotations
 
-import collections
+import ctypes
 import dataclasses
 import time
 from typing import Callable
 
-from ..cache.allocator import pages_for_len
+from .. import host as _host
 from .batch import StepEntry
 from .generate import (Control, GenerateParams, Generated, SampleCursor, Sampled, StopReason, _go_on,
                        _no_bytes)
@@ -61,30 +65,22 @@ class Failure:
 
 
 class Sequence:
-    def __init__(self, seq_id: int, prompt: list[int], params: GenerateParams, token_bytes, on_chunk):
+    """What the host keeps of a sequence: its sampler, callbacks and timings.  Its tokens live in the core."""
+
+    def __init__(self, seq_id: int, prompt_len: int, params: GenerateParams, token_bytes, on_chunk):
         self.id = seq_id
-        self.prompt = list(prompt)
-        self.tokens = list(prompt)       # prompt and every sampled id that is to be forwarded
+        self.prompt_len = prompt_len
         self.params = params
         self.cursor = SampleCursor(params)
         self.token_bytes = token_bytes
         self.on_chunk = on_chunk
-        self.computed = 0                # tokens whose keys and values are in the cache
         self.prefill = 0.0
         self.decode = 0.0
         self.result: Generated | Failure | None = None
 
-    @property
-    def sampled(self) -> int:
-        return len(self.tokens) - len(self.prompt)
 
-    @property
-    def remaining(self) -> int:
-        return len(self.tokens) - self.computed
-
-    @property
-    def decoding(self) -> bool:
-        return self.sampled > 0 and self.remaining == 1
+_RUNNING, _WAITING, _MAX_RUNNING, _PREEMPTIONS, _LAST_PREEMPTED, _FRONT, _PAGES_TO_ADMIT, _COMPUTED, _N_TOKENS, \
+    _IS_RUNNING = range(10)
 
 
 class Scheduler:
@@ -99,11 +95,38 @@ class Scheduler:
         self.engine = engine
         self.cache = engine.cache
         self.config = config or SchedulerConfig()
-        self.waiting: collections.deque[Sequence] = collections.deque()
-        self.running: list[Sequence] = []
+        self._lib = _host.lib()
+        self._core = self._lib.ta_sched_new(self.cache._core, self.cache.num_pages, self.config.max_batch_size,
+                                            self.config.max_num_batched_tokens, self.config.prefill_chunk or 0)
+        if not self._core:
+            raise ValueError("max_batch_size and max_num_batched_tokens must be positive")
+        self.sequences: dict[int, Sequence] = {}          # every sequence the core knows: waiting or running
         self.finished: dict[int, Generated | Failure] = {}
         self.stats = EngineStats()
         self._next_id = 1
+
+    def __del__(self):
+        if getattr(self, "_core", None):
+            self._lib.ta_sched_delete(self._core)
+            self._core = None
+
+    def _get(self, what: int, seq_id: int = 0) -> int:
+        return int(self._lib.ta_sched_get(self._core, what, seq_id))
+
+    def _listed(self, which: int) -> list[Sequence]:
+        out = (ctypes.c_int64 * max(1, len(self.sequences)))()
+        count = self._lib.ta_sched_list(self._core, which, out)
+        return [self.sequences[i] for i in out[:count]]
+
+    @property
+    def running(self) -> list[Sequence]:
+        """The running sequences in order of admission."""
+        return self._listed(0)
+
+    @property
+    def waiting(self) -> list[Sequence]:
+        """The queue, its front first."""
+        return self._listed(1)
 
     # ------------------------------------------------------------------- requests
     def add_request(self, prompt: list[int], params: GenerateParams | None = None,
@@ -112,8 +135,8 @@ class Scheduler:
         """Queue a request; returns its id.  Problems with the request itself are recorded as a failed
         result under that id (as the reference answers them on the request's own channel)."""
         params = params or GenerateParams()
-        if len(self.waiting) >= self.config.max_waiting:
-            raise QueueFull(f"{len(self.waiting)} requests are already waiting")
+        if self._get(_WAITING) >= self.config.max_waiting:
+            raise QueueFull(f"{self._get(_WAITING)} requests are already waiting")
         seq_id = self._next_id
         self._next_id += 1
         if not prompt:
@@ -125,11 +148,13 @@ class Scheduler:
                                    f"exceeds max_position_embeddings {limit}")
             return seq_id
         try:
-            seq = Sequence(seq_id, prompt, params, token_bytes, on_chunk)
+            seq = Sequence(seq_id, len(prompt), params, token_bytes, on_chunk)
         except ValueError as err:
             self._fail_new(seq_id, str(err))
             return seq_id
-        self.waiting.append(seq)
+        keep, pointer = _host.int_array(list(prompt))
+        self._lib.ta_sched_enqueue(self._core, seq_id, pointer, len(keep))
+        self.sequences[seq_id] = seq
         return seq_id
 
     def _fail_new(self, seq_id: int, message: str) -> None:
@@ -137,104 +162,52 @@ class Scheduler:
         self.stats.requests_failed += 1
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.sequences)
 
-    # ------------------------------------------------------------------ admission
-    def _pages_to_admit(self, seq: Sequence) -> int:
-        # A new request needs its prompt; one that already sampled also gets room for the next token, so
-        # that it is not evicted again at once (engine.rs:696-704).
-        length = len(seq.tokens) + (1 if seq.sampled else 0)
-        return pages_for_len(length, self.cache.page_size)
+    def _pool_message(self, pages_needed: int) -> str:
+        return (f"kv pool has {self.cache.num_pages} blocks of {self.cache.page_size}; "
+                f"this sequence needs {pages_needed}")
 
-    def _admit(self) -> None:
-        while self.waiting and len(self.running) < self.config.max_batch_size:
-            seq = self.waiting[0]
-            needed = self._pages_to_admit(seq)
-            if needed > self.cache.num_pages:
-                self.waiting.popleft()
-                self._fail(seq, f"kv pool has {self.cache.num_pages} blocks of {self.cache.page_size}; "
-                                f"this sequence needs {needed}")
-                continue
-            if self.cache.free_slot_count() == 0:
-                break
-            self.cache.add_request(seq.id)
-            shared = self.cache.attach_shared_prefix(seq.id, seq.tokens)
-            if not self.cache.reserve(seq.id, needed * self.cache.page_size):
-                self.cache.release(seq.id)      # gives back the shared pages and the slot
-                break
-            self.waiting.popleft()
-            seq.computed = shared
-            self.running.append(seq)
-        self.stats.max_running = max(self.stats.max_running, len(self.running))
-
-    # ------------------------------------------------------------------- planning
-    def _preempt(self, seq: Sequence, preempted: list[Sequence]) -> None:
-        self.running.remove(seq)
-        self.cache.release(seq.id)
-        seq.computed = 0
-        self.stats.preemptions += 1
-        self.stats.last_preempted_id = seq.id
-        preempted.append(seq)
-
-    def _fail(self, seq: Sequence, message: str) -> None:
-        if seq in self.running:
-            self.running.remove(seq)
-            self.cache.release(seq.id)
+    def _record_failure(self, seq_id: int, message: str) -> None:
+        """The core has already dropped the sequence and given back what it held."""
+        seq = self.sequences.pop(seq_id)
         seq.result = Failure(message)
-        self.finished[seq.id] = seq.result
+        self.finished[seq_id] = seq.result
         self.stats.requests_failed += 1
-
-    def _plan(self, preempted: list[Sequence]) -> list[tuple[Sequence, int]]:
-        """(sequence, tokens to run) for this iteration, pages reserved.  Oldest first; decoding
-        sequences before prompt portions."""
-        budget = self.config.max_num_batched_tokens
-        chunk = self.config.prefill_chunk or budget
-        order = sorted(self.running, key=lambda s: (not s.decoding, s.id))
-        planned: list[tuple[Sequence, int]] = []
-        for seq in order:
-            if seq not in self.running or budget <= 0:
-                continue
-            count = 1 if seq.decoding else min(seq.remaining, budget, chunk)
-            new_len = seq.computed + count
-            while not self.cache.reserve(seq.id, new_len):
-                needed = pages_for_len(new_len, self.cache.page_size)
-                if needed > self.cache.num_pages:
-                    self._fail(seq, f"kv pool has {self.cache.num_pages} blocks of {self.cache.page_size}; "
-                                    f"this sequence needs {needed}")
-                    break
-                victim = max(self.running, key=lambda s: s.id)       # the newest (engine.rs:632-639)
-                planned = [(s, n) for s, n in planned if s is not victim]
-                self._preempt(victim, preempted)
-                if victim is seq:
-                    break
-            if seq in self.running:
-                planned.append((seq, count))
-                budget -= count
-        return planned
 
     # ----------------------------------------------------------------------- step
     def step(self) -> bool:
-        """One iteration.  Returns False when there was nothing to run."""
-        self._admit()
-        if not self.running:
-            return False
-        preempted: list[Sequence] = []
-        planned = self._plan(preempted)
-        if planned:
-            self._run(planned)
+        """One iteration: the core admits, plans (pages reserved, the newest sequence preempted when they run
+        out) and requeues; the plan is then run as one batch.  Returns False when there was nothing to run."""
+        room = max(1, len(self.sequences))
+        planned = (ctypes.c_int64 * (4 * room))()
+        preempted = (ctypes.c_int64 * room)()
+        failed = (ctypes.c_int64 * (2 * room))()
+        counts = [ctypes.c_int32(0) for _ in range(3)]
+        status = self._lib.ta_sched_plan_step(self._core, room, planned, ctypes.byref(counts[0]), preempted,
+                                              ctypes.byref(counts[1]), failed, ctypes.byref(counts[2]))
+        if status != 0:
+            raise RuntimeError("the scheduler core's plan did not fit its buffers")
+        n_planned, n_preempted, n_failed = (c.value for c in counts)
+        for i in range(n_failed):
+            self._record_failure(int(failed[2 * i]), self._pool_message(int(failed[2 * i + 1])))
+        plan = [(self.sequences[int(planned[4 * i])], int(planned[4 * i + 1]), int(planned[4 * i + 2]),
+                 bool(planned[4 * i + 3])) for i in range(n_planned)]
+        if plan:
+            self._run(plan)
         self._note_peaks()
-        # Oldest preempted sequence first, ahead of requests that never ran (engine.rs:369-376).
-        for seq in sorted(preempted, key=lambda s: s.id, reverse=True):
-            self.waiting.appendleft(seq)
-        return bool(planned) or bool(preempted)
+        return bool(plan) or n_preempted > 0
 
-    def _run(self, planned: list[tuple[Sequence, int]]) -> None:
+    def _tokens(self, seq_id: int, first: int, count: int) -> list[int]:
+        out = (ctypes.c_int32 * max(1, count))()
+        self._lib.ta_sched_tokens(self._core, seq_id, first, count, out)
+        return list(out[:count])
+
+    def _run(self, plan: list[tuple[Sequence, int, int, bool]]) -> None:
         entries, wanting = [], []
-        for seq, count in planned:
-            tokens = seq.tokens[seq.computed:seq.computed + count]
-            completes = seq.computed + count == len(seq.tokens)
+        for seq, first, count, completes in plan:
             wants = completes and seq.params.max_tokens > 0
-            entries.append(StepEntry(seq.id, tokens, [count - 1] if wants else []))
+            entries.append(StepEntry(seq.id, self._tokens(seq.id, first, count), [count - 1] if wants else []))
             if wants:
                 wanting.append(seq)
         started = time.perf_counter()
@@ -258,55 +231,46 @@ class Scheduler:
             warm_logits = self.engine.rows_to_host(logits, warm_rows)
         elapsed = time.perf_counter() - started
         self.stats.steps += 1
-        self.stats.tokens_forwarded += sum(count for _, count in planned)
-        n_decoding = sum(1 for seq, _ in planned if seq.decoding) or 1
-        for seq, count in planned:
-            if seq.decoding:
+        self.stats.tokens_forwarded += sum(count for _, _, count, _ in plan)
+        decoding = [first >= seq.prompt_len and count == 1 for seq, first, count, _ in plan]
+        n_decoding = sum(decoding) or 1
+        for (seq, _, count, _), is_decoding in zip(plan, decoding):
+            if is_decoding:
                 seq.decode += elapsed / n_decoding     # shares add up to the step (engine.rs:909-916)
             else:
                 seq.prefill += elapsed
-            seq.computed += count
-            if seq.computed - count < len(seq.prompt):      # the portion held prompt tokens
-                self.cache.publish(seq.id, seq.prompt)
+            self._lib.ta_sched_commit(self._core, seq.id, count)     # full prompt pages become shareable
         for row, seq in enumerate(wanting):
             if row in picked:
                 outcome = seq.cursor.push_token(picked[row], seq.token_bytes, seq.on_chunk)
             else:
                 outcome = seq.cursor.push_logits(warm_logits[warm_rows.index(row)], seq.token_bytes, seq.on_chunk)
-            self._after_sample(seq, outcome)
-        for seq, _ in planned:
-            if seq.result is None and seq.computed == len(seq.tokens) and seq.params.max_tokens == 0:
+            if isinstance(outcome, Sampled):
+                self._finish(seq, outcome)
+            else:
+                self._lib.ta_sched_append_token(self._core, seq.id, int(outcome))
+        for seq, _, _, completes in plan:
+            if seq.result is None and completes and seq.params.max_tokens == 0:
                 self._finish(seq, seq.cursor.finish_without_sample(seq.on_chunk))
-
-    def _after_sample(self, seq: Sequence, outcome) -> None:
-        if isinstance(outcome, Sampled):
-            self._finish(seq, outcome)
-        else:
-            seq.tokens.append(int(outcome))
 
     def _finish(self, seq: Sequence, done: Sampled) -> None:
         seq.result = Generated(done.tokens, done.text, done.chunks, done.reason, done.completion_tokens,
                                seq.prefill, seq.decode)
         self.finished[seq.id] = seq.result
-        self.running.remove(seq)
-        self.cache.release(seq.id)
+        self._lib.ta_sched_finish(self._core, seq.id)       # pages and the slot go back
+        del self.sequences[seq.id]
         self.stats.requests_finished += 1
 
     def cancel(self, seq_id: int) -> None:
         """Stop a request before its next forward; what it sampled so far is its result."""
-        for seq in list(self.running) + list(self.waiting):
-            if seq.id == seq_id:
-                if seq in self.running:
-                    self._finish(seq, seq.cursor.snapshot(StopReason.Cancelled))
-                else:
-                    self.waiting.remove(seq)
-                    done = seq.cursor.snapshot(StopReason.Cancelled)
-                    self.finished[seq.id] = Generated(done.tokens, done.text, done.chunks, done.reason,
-                                                      done.completion_tokens, seq.prefill, seq.decode)
-                    self.stats.requests_finished += 1
-                return
+        seq = self.sequences.get(seq_id)
+        if seq is not None:
+            self._finish(seq, seq.cursor.snapshot(StopReason.Cancelled))
 
     def _note_peaks(self) -> None:
+        self.stats.max_running = self._get(_MAX_RUNNING)
+        self.stats.preemptions = self._get(_PREEMPTIONS)
+        self.stats.last_preempted_id = self._get(_LAST_PREEMPTED)
         for group in self.cache.groups:
             self.stats.peak_blocks = max(self.stats.peak_blocks, group.allocator.peak_live)
             self.stats.peak_occupied = max(self.stats.peak_occupied, group.allocator.peak_occupied)
@@ -318,11 +282,12 @@ class Scheduler:
         while self.has_work():
             progressed = self.step()
             steps += 1
-            if not progressed and not self.running and self.waiting:
+            if not progressed and self._get(_RUNNING) == 0 and self._get(_WAITING) > 0:
                 # The front of the queue cannot be admitted into an empty batch: it never will be.
-                seq = self.waiting.popleft()
-                self._fail(seq, f"kv pool has {self.cache.num_pages} blocks of {self.cache.page_size}; "
-                                f"this sequence needs {self._pages_to_admit(seq)}")
+                front = self._get(_FRONT)
+                needed = self._get(_PAGES_TO_ADMIT, front)
+                self._lib.ta_sched_finish(self._core, front)
+                self._record_failure(front, self._pool_message(needed))
             if max_steps is not None and steps >= max_steps:
                 break
         return self.finished
@@ -330,7 +295,7 @@ class Scheduler:
     def assert_idle(self) -> None:
         """With nothing live every count is zero and, cached pages reclaimed, every page is free
         (engine.rs:385-400)."""
-        assert not self.running and not self.waiting
+        assert self._get(_RUNNING) == 0 and self._get(_WAITING) == 0 and not self.sequences
         assert not self.cache.requests
         for group in self.cache.groups:
             assert group.allocator.all_refcounts_zero(), "kv refcounts still held"

@@ -57,6 +57,17 @@ _SIGNATURES = {
     "ta_cache_check": (_int, [_vp]),
     "ta_cache_pack_batch": (_i64, [_vp, _int, _i64p, _i32p, _i32p, _i32p, _i32p, _int, _i32p, _i64, _i64p, _i32p,
                                    _i32p]),
+    "ta_cache_request_ids": (_int, [_vp, _i64p]),
+    "ta_sched_new": (_vp, [_vp, _int, _int, _int, _int]),
+    "ta_sched_delete": (None, [_vp]),
+    "ta_sched_enqueue": (_int, [_vp, _i64, _i32p, _int]),
+    "ta_sched_append_token": (_int, [_vp, _i64, ctypes.c_int32]),
+    "ta_sched_get": (_i64, [_vp, _int, _i64]),
+    "ta_sched_plan_step": (_int, [_vp, _int, _i64p, _i32p, _i64p, _i32p, _i64p, _i32p]),
+    "ta_sched_list": (_int, [_vp, _int, _i64p]),
+    "ta_sched_tokens": (_int, [_vp, _i64, _int, _int, _i32p]),
+    "ta_sched_commit": (_int, [_vp, _i64, _int]),
+    "ta_sched_finish": (_int, [_vp, _i64]),
     "ta_uniform_f32": (_f32, [_u64, _u64]),
     "ta_greedy_token": (_int, [_f32p, _i64]),
     "ta_sample_with_uniform": (_int, [_f32p, _i64, _f32, _f32, _f32]),
