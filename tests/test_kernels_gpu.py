@@ -272,6 +272,38 @@ def test_paged_attention_finds_one_far_key(ops, attention_mode):
     torch.testing.assert_close(out.reshape(n_q, d).float()[0], v_pages[page, 0, :, off].float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("attention_mode", ATTENTION_MODES, indirect=True)
+@pytest.mark.parametrize("waves", [0, 1])
+def test_every_row_of_a_portion_sees_exactly_to_its_window_edge(ops, attention_mode, waves, monkeypatch):
+    """A portion of 100 prompt tokens under a window of 77: the query at position p is made to look at the key
+    at p - 77, the farthest it may see; those keys cross page and tile edges.  The output must be that key's
+    value row; with a window of 76 the key is out of sight and the output is something else."""
+    dtype = attention_mode
+    monkeypatch.setattr(ops, "prefill_waves", waves)
+    n_q, n_kv, d, page_size, window = 4, 2, 64, 16, 77
+    lengths, q_lens = [700], [100]
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        dtype, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=21)
+    group = n_q // n_kv
+    want = torch.empty((q_lens[0], n_q, d))
+    for row in range(q_lens[0]):
+        target = int(positions[row]) - window
+        page, off = int(table[0, target // page_size]), target % page_size
+        for h in range(n_q):
+            key = k_pages[page, h // group, off].float()
+            qkv[row, h * d:(h + 1) * d] = (key * (30.0 / float(key.dot(key)))).to(dtype)   # its score is 30
+            want[row, h] = v_pages[page, h // group, :, off].float().cpu()
+    batch = make_batch(lengths, q_lens) if ops.use_fast_attention else None
+    out = torch.full((q_lens[0], n_q * d), float("nan"), dtype=dtype).cuda()
+    ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, 1.0,
+                        max_position=lengths[0] - 1, batch=batch)
+    torch.testing.assert_close(out.float().cpu().reshape(q_lens[0], n_q, d), want, rtol=2e-2, atol=2e-2)
+    ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window - 1, 1.0,
+                        max_position=lengths[0] - 1, batch=batch)
+    off_by = (out.float().cpu().reshape(q_lens[0], n_q, d) - want).abs().amax(dim=(1, 2))
+    assert float(off_by.min()) > 0.1          # every row lost its key
+
+
 def linear_tol(out_dtype, x, w):
     # A float32 sum of K products errs by about sqrt(K) * 2^-24 * |x||w| per term, also where the
     # result cancels to nearly zero; allow eight times that.  bfloat16 output adds its own rounding.
