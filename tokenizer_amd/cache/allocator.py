@@ -55,10 +55,11 @@ _tokens = _host.token_array
 
 
 class PageAllocator:
-    def __init__(self, num_pages: int, page_size: int = 16, _borrowed=None):
+    def __init__(self, num_pages: int, page_size: int = 16, _borrowed=None, _owner=None):
         self._lib = _host.lib()
-        if _borrowed is not None:                 # an allocator that lives inside a cache manager
+        if _borrowed is not None:                 # an allocator that lives inside a cache manager's core
             self._handle, self._owned = _borrowed, False
+            self._owner = _owner                  # whose core it is: kept alive as long as this object
         else:
             if num_pages < 0 or page_size <= 0:
                 raise ValueError("num_pages must not be negative and page_size must be positive")

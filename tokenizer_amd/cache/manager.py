@@ -100,6 +100,19 @@ class _Requests:
         return [self[rid] for rid in self]
 
 
+class _CoreOwner:
+    """Deletes the C++ core when the last Python object that points into it has gone (the manager itself, the
+    allocators of its groups, a scheduler built on it)."""
+
+    def __init__(self, lib, core):
+        self._lib, self._core = lib, core
+
+    def __del__(self):
+        if self._core:
+            self._lib.ta_cache_delete(self._core)
+            self._core = None
+
+
 class CacheManager:
     def __init__(self, needs: list[CacheNeed], num_pages: int, page_size: int = 16, max_requests: int = 8,
                  prefix_cache: bool = False):
@@ -115,8 +128,10 @@ class CacheManager:
                                             1 if prefix_cache else 0)
         if not self._core:
             raise ValueError("num_pages and max_requests must not be negative and page_size must be positive")
+        self._core_owner = _CoreOwner(self._lib, self._core)
         self.groups = [CacheGroup(need, layers, PageAllocator(num_pages, page_size,
-                                                              _borrowed=self._lib.ta_cache_allocator(self._core, g)))
+                                                              _borrowed=self._lib.ta_cache_allocator(self._core, g),
+                                                              _owner=self._core_owner))
                        for g, (need, layers) in enumerate(planned)]
         # Sharing a prefix needs every group to keep all positions (a window group drops pages).
         self.prefix_cache = bool(self._lib.ta_cache_prefix_enabled(self._core))
@@ -126,11 +141,6 @@ class CacheManager:
         self._ids: dict[object, int] = {}
         self._next_handle = _FIRST_NAMED
         self.requests = _Requests(self)
-
-    def __del__(self):
-        if getattr(self, "_core", None):
-            self._lib.ta_cache_delete(self._core)
-            self._core = None
 
     def _handle_of(self, rid) -> int:
         """The core's handle of a live request; KeyError for one that is not live."""

@@ -100,6 +100,7 @@ class Scheduler:
                                             self.config.max_num_batched_tokens, self.config.prefill_chunk or 0)
         if not self._core:
             raise ValueError("max_batch_size and max_num_batched_tokens must be positive")
+        self._cache_core_owner = self.cache._core_owner      # the cache core outlives this scheduler's core
         self.sequences: dict[int, Sequence] = {}          # every sequence the core knows: waiting or running
         self.finished: dict[int, Generated | Failure] = {}
         self.stats = EngineStats()
