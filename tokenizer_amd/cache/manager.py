@@ -260,6 +260,8 @@ class CacheManager:
                                               as_i64(sizes), as_i32(widths), as_i32(info))
         if total == -3:
             raise KeyError("a request of the batch is not live")
+        if total == -5:
+            raise RuntimeError("a request holds too few pages for its new tokens (they are reserved before a step)")
         if total == -6:
             raise RuntimeError("a request writes a position into a page it gave back")
         if total == -7:
