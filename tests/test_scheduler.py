@@ -183,3 +183,48 @@ def test_cancel(model_folders):
     sched.cancel(waiting)
     sched.run()
     sched.assert_idle()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed):
+    """Random prompts, output lengths, pool sizes, batch caps, token budgets, portion sizes and arrival times
+    (shared prefixes included): whatever the scheduler decides, every request gets the tokens it would get alone,
+    and when all is over no page, count or slot is left."""
+    import random
+    rng = random.Random(seed)
+    folder = model_folders["A"]
+    page = 16
+    num_pages = rng.choice([4, 6, 9, 24])
+    config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 3, 5]), num_blocks=num_pages,
+                             prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 16, 40]),
+                             prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64)
+    engine = cpu_engine(folder, num_pages=num_pages, max_requests=config.max_batch_size,
+                        prefix_cache=config.prefix_cache)
+    sched = Scheduler(engine, config)
+    shared = random_ids(256, 35, 900 + seed)
+    plan = []
+    for i in range(rng.randint(4, 9)):
+        prompt = random_ids(256, rng.choice([1, 2, 7, 16, 17, 33, 48]), 100 * seed + i)
+        if rng.random() < 0.4:
+            prompt = shared[:rng.choice([16, 32, 35])] + prompt
+        plan.append((rng.randint(0, 6), prompt, rng.randint(0, 7)))
+    ids, step = {}, 0
+    pending = sorted(plan, key=lambda item: item[0])
+    while pending or sched.has_work():
+        while pending and pending[0][0] <= step:
+            _, prompt, n = pending.pop(0)
+            ids[sched.add_request(prompt, GenerateParams.greedy(n))] = (prompt, n)
+        if sched.has_work():
+            sched.run(max_steps=1)
+        step += 1
+        assert step < 2000
+        engine.cache.check_invariants()
+    assert all(sum(tokens) <= config.max_num_batched_tokens for tokens in engine.forwards)
+    for rid, (prompt, n) in ids.items():
+        result = sched.finished[rid]
+        if isinstance(result, Failure):
+            # Only a sequence that the whole pool cannot hold may fail, and it says so.
+            assert "kv pool has" in result.message and -(-(len(prompt) + n) // page) > num_pages
+            continue
+        assert result.tokens == solo(folder, prompt, GenerateParams.greedy(n)).tokens, (rid, len(prompt), n)
+    sched.assert_idle()
