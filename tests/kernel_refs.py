@@ -107,7 +107,7 @@ class PlainOps:
     # The fused decode products, as compositions of the ops above.
     fuse_rows = 16
 
-    def can_fuse_decode(self, rows, dtype):
+    def can_fuse_decode(self, rows, dtype, hidden=0):
         return 0 < rows <= self.fuse_rows
 
     def fused_norm_qkv_rope(self, residual, norm_weight, eps, weight, bias, positions, cos_sin, slots,

@@ -321,10 +321,14 @@ class Ops:
     fused_rows = 0            # 0: the launcher picks the weight rows per workgroup (1..32; 16, 8, 4 with rotation) ...
     fused_waves = 0           # ... and how many waves share a tile's K (4, 8, 16)
 
-    def can_fuse_decode(self, rows: int, dtype: torch.dtype) -> bool:
+    FUSED_LDS_BYTES = 140 * 1024     # what the norm prologue may take of a compute unit's 160 KB of LDS
+
+    def can_fuse_decode(self, rows: int, dtype: torch.dtype, hidden: int = 0) -> bool:
         """Batches of few bfloat16 rows can run the products that take the norm, the rotation with the
-        cache write, the gated activation and the residual add into the same kernel."""
-        return self.use_fused_decode and dtype == torch.bfloat16 and 0 < rows <= self.FUSED_ROWS
+        cache write, the gated activation and the residual add into the same kernel.  The norm prologue
+        keeps sixteen normalised rows of `hidden` elements in LDS, which bounds `hidden`."""
+        return (self.use_fused_decode and dtype == torch.bfloat16 and 0 < rows <= self.FUSED_ROWS
+                and 16 * (hidden + 8) * 2 <= self.FUSED_LDS_BYTES)
 
     def fused_norm_qkv_rope(self, residual, norm_weight, eps, weight, bias, positions, cos_sin, slots,
                             k_pages, v_pages, n_q: int, n_kv: int, head_dim: int) -> torch.Tensor:

@@ -5,6 +5,7 @@ import math
 
 import torch
 
+from .base import can_fuse_decode as _can_fuse
 from .base import MIXERS, POSITIONS, Mixer, Runtime
 from .norm import RMSNorm
 from .position import NoPosition, RotaryHalfSplit
@@ -66,7 +67,7 @@ class GQAttention(Mixer):
         ops = self.runtime.ops
         fused = (delta is None and type(norm) is RMSNorm and type(self.position) in (NoPosition, RotaryHalfSplit)
                  and self.d % 32 == 0 and cache.group is not None
-                 and getattr(ops, "can_fuse_decode", lambda rows, dtype: False)(residual.shape[0], self.runtime.dtype))
+                 and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
             return super().forward_normed(residual, delta, norm, ctx, cache)
         q = ops.fused_norm_qkv_rope(residual, norm.weight, norm.eps, self.w_qkv, self.b_qkv, ctx.positions,

@@ -121,3 +121,10 @@ class Block:
 
     def forward(self, residual: torch.Tensor, delta: torch.Tensor | None, ctx, cache) -> torch.Tensor:
         raise NotImplementedError
+
+
+def can_fuse_decode(ops, residual, dtype) -> bool:
+    """Whether the kernel library offers its fused decode products for these rows of the residual stream
+    (few bfloat16 rows of a width whose normalised copy fits in LDS); a library without them says no."""
+    check = getattr(ops, "can_fuse_decode", None)
+    return bool(check and check(residual.shape[0], dtype, residual.shape[1]))

@@ -3,6 +3,7 @@ from __future__ import annotations
 
 import torch
 
+from .base import can_fuse_decode as _can_fuse
 from .base import FEED_FORWARDS, FeedForward, Runtime
 from .norm import RMSNorm
 from .spec import FeedForwardSpec, TensorSpec
@@ -36,7 +37,7 @@ class GatedDense(FeedForward):
         down product added straight into the residual stream."""
         ops = self.runtime.ops
         fused = (delta is None and type(norm) is RMSNorm
-                 and getattr(ops, "can_fuse_decode", lambda rows, dtype: False)(residual.shape[0], self.runtime.dtype))
+                 and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
             return super().forward_normed(residual, delta, norm, ctx)
         act = ops.fused_norm_gated(residual, norm.weight, norm.eps, self.w_gate_up)
