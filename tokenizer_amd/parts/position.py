@@ -35,16 +35,21 @@ class RotaryHalfSplit(NoPosition):
     every position up to `max_positions`.  Keys are stored after the rotation.
     """
 
+    _tables: dict[tuple, torch.Tensor] = {}
+
     def __init__(self, spec: PositionSpec, runtime: Runtime):
         super().__init__(spec, runtime)
         if spec.head_dim % 2:
             raise ValueError(f"rope needs an even head size, found {spec.head_dim}")
         d = spec.head_dim
-        inv_freq = torch.tensor([1.0 / (float(spec.theta) ** (i / d)) for i in range(0, d, 2)],
-                                dtype=torch.float64).to(torch.float32)
-        positions = torch.arange(spec.max_positions, dtype=torch.float32)
-        angles = positions[:, None] * inv_freq[None, :]
-        self.cos_sin = torch.cat([angles.cos(), angles.sin()], dim=1).contiguous().to(runtime.device)
+        key = (d, float(spec.theta), spec.max_positions, str(runtime.device))
+        if key not in self._tables:               # the layers of a model share one table
+            inv_freq = torch.tensor([1.0 / (float(spec.theta) ** (i / d)) for i in range(0, d, 2)],
+                                    dtype=torch.float64).to(torch.float32)
+            positions = torch.arange(spec.max_positions, dtype=torch.float32)
+            angles = positions[:, None] * inv_freq[None, :]
+            self._tables[key] = torch.cat([angles.cos(), angles.sin()], dim=1).contiguous().to(runtime.device)
+        self.cos_sin = self._tables[key]
         self.max_positions = spec.max_positions
 
     def table(self):
