@@ -87,19 +87,18 @@ def run_decode(model, batch: int, steps: int, warmup: int):
         logits = engine.step([StepEntry(rid, prompt, [len(prompt) - 1])])
         last.append(engine.argmax(logits)[0])
 
-    def decode_step(tokens):
-        logits = engine.step([StepEntry(rid, [tokens[rid]], [0]) for rid in range(batch)])
-        return engine.argmax(logits)
-
-    for _ in range(warmup):
-        last = decode_step(last)
+    # Greedy decode steps back to back: each step's ids feed the next on the device and reach the host one
+    # step late (`Engine.decode_greedy`), so the host's work on a step hides behind the device's.
+    rids = list(range(batch))
+    if warmup:
+        last = engine.decode_greedy(rids, last, warmup)[-1]
     torch.cuda.synchronize()
     kv_start = engine.cache.seq_len(0)
     started = time.perf_counter()
-    for _ in range(steps):
-        last = decode_step(last)
+    picked = engine.decode_greedy(rids, last, steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
+    assert len(picked) == steps and all(len(ids) == batch for ids in picked)
     kv_mean = kv_start + (steps - 1) / 2 + 1          # keys each step reads, averaged over the timed steps
     for rid in range(batch):
         engine.end_request(rid)

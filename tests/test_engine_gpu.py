@@ -188,6 +188,42 @@ def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
     assert len(engines[0].graphs) >= 3
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, dtype, monkeypatch):
+    """`decode_greedy` feeds each step's ids to the next on the device and reads them a step late; it must pick
+    what stepping one by one picks, also across a change of graph (the context bucket is made small), and an
+    early end returns exactly one step more than was asked for."""
+    from tokenizer_amd.engine import Engine, StepEntry
+    name = "B"
+    vocab = TINY[name][0]["vocab_size"]
+    monkeypatch.setattr(Engine, "GRAPH_BUCKET", 48)
+    prompts = {rid: random_ids(vocab, n, 90 + rid) for rid, n in enumerate([40, 3, 21])}
+    runs = []
+    for pipelined in (True, False):
+        eng = engine_for(model_folders[name], dtype, max_tokens=512, max_requests=4)
+        first = []
+        for rid, ids in prompts.items():
+            eng.add_request(rid)
+            first.append(eng.argmax(eng.step([StepEntry(rid, ids, [len(ids) - 1])]))[0])
+        if pipelined:
+            picked = eng.decode_greedy(list(prompts), first, 30)
+            assert len(eng.graphs) >= 2                      # the contexts crossed a bucket's end
+        else:
+            picked, current = [], first
+            for _ in range(30):
+                current = eng.argmax(eng.step([StepEntry(rid, [t], [0]) for rid, t in zip(prompts, current)]))
+                picked.append(current)
+        runs.append(picked)
+        assert [eng.cache.seq_len(rid) for rid in prompts] == [len(ids) + 30 for ids in prompts.values()]
+        # An early end: the step already launched when the answer came still counts.
+        seen = []
+        more = eng.decode_greedy(list(prompts), picked[-1], 10, on_step=lambda k, ids: seen.append(k) or k < 3)
+        assert len(more) == 5 and seen == [0, 1, 2, 3]
+        runs.append(more[:4])
+        eng.cache.check_invariants()
+    assert runs[0] == runs[2] and runs[1] == runs[3]
+
+
 def sharpened(folder, out_folder, factor):
     """A copy of a model folder whose query and key projections are scaled up: attention becomes nearly
     one-hot, so a wrong key, page or window edge changes the logits by far more than any rounding."""

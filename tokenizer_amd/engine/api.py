@@ -57,12 +57,25 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
         elif on_chunk("") == Control.Stop:
             done = Sampled([], "", [], StopReason.Cancelled, 0)
         else:
-            while True:
-                outcome = _next(engine, cursor, logits, token_bytes, on_chunk)
-                if isinstance(outcome, Sampled):
-                    done = outcome
-                    break
+            outcome = _next(engine, cursor, logits, token_bytes, on_chunk)
+            if not isinstance(outcome, Sampled) and cursor.is_greedy and hasattr(engine, "decode_greedy"):
+                # Greedy: the remaining steps run back to back on the device; the cursor sees each id one step
+                # late and ends the run when it stops (at most one forward is then run for nothing).
+                ended = []
+
+                def on_step(_k, ids):
+                    result = cursor.push_token(ids[0], token_bytes, on_chunk)
+                    if isinstance(result, Sampled):
+                        ended.append(result)
+                        return False
+                    return True
+
+                engine.decode_greedy([rid], [int(outcome)], params.max_tokens - cursor.produced, on_step)
+                outcome = ended[0]
+            while not isinstance(outcome, Sampled):
                 logits = engine.step([StepEntry(rid, [int(outcome)], [0])])
+                outcome = _next(engine, cursor, logits, token_bytes, on_chunk)
+            done = outcome
         decode = time.perf_counter() - started
     finally:
         engine.end_request(rid)

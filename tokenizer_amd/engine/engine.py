@@ -94,8 +94,9 @@ class DecodeGraph:
             self.ids = ops.argmax(self.logits)
         self.uploaded = None
 
-    def run(self, engine: "Engine", entries: list[StepEntry]) -> torch.Tensor:
-        """Pack the batch's description into the fixed buffers again and replay."""
+    def run(self, engine: "Engine", entries: list[StepEntry], tokens_on_device: torch.Tensor | None = None) -> torch.Tensor:
+        """Pack the batch's description into the fixed buffers again and replay.  `tokens_on_device`: the token
+        ids come from this int32 tensor on the device (the ids an earlier replay picked), not from the entries."""
         if self.uploaded is not None:
             self.uploaded.synchronize()                 # the last upload has left the pinned buffer
         else:
@@ -107,6 +108,8 @@ class DecodeGraph:
             raise ValueError("the packed batch does not fit the graph's buffers")
         self.dev.copy_(self.host, non_blocking=True)
         self.uploaded.record()
+        if tokens_on_device is not None:
+            self.dev[:len(entries)].copy_(tokens_on_device, non_blocking=True)   # the token ids lead the buffer
         self.graph.replay()
         return self.logits
 
@@ -174,7 +177,63 @@ class Engine:
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):
         return logits[rows].float().cpu().numpy()
 
-    def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
+    def decode_greedy(self, rids: list, tokens: list[int], n_steps: int, on_step=None) -> list[list[int]]:
+        """`n_steps` greedy decode steps for the live requests `rids`, whose next tokens are `tokens`; returns the
+        ids picked at every step, `n_steps` lists in the order of `rids`.
+
+        The steps run back to back on the device: the ids a step picks feed the next step there, and the next
+        step is launched before they have reached the host, which reads them one step late.  So the host's work
+        on a step (tables, launch) hides behind the device's work on the step before.  `on_step(k, ids)` is
+        called as each step's ids arrive; if it returns False the run ends after the step already launched (whose
+        ids are still returned: the caller drops what it does not want; the cache holds those tokens too).
+        Without captured graphs the steps run one by one through `step`."""
+        if n_steps <= 0:
+            return []
+        if len(rids) != len(tokens) or not rids:
+            raise ValueError("one next token per request")
+        if not self.use_graphs:
+            picked, current = [], list(tokens)
+            for k in range(n_steps):
+                current = self.argmax(self.step([StepEntry(rid, [int(t)], [0]) for rid, t in zip(rids, current)]))
+                picked.append(list(current))
+                if on_step is not None and on_step(k, picked[-1]) is False:
+                    break
+            return picked
+        count = len(rids)
+        landing = [torch.empty(count, dtype=torch.int32).pin_memory() for _ in range(2)]
+        arrived = [torch.cuda.Event(), torch.cuda.Event()]
+        picked: list[list[int]] = []
+        previous: DecodeGraph | None = None
+        go_on = True
+        for k in range(n_steps):
+            # Only the first step's token ids are known here; later steps take theirs from the step before.
+            entries = [StepEntry(rid, [int(tokens[i]) if k == 0 else 0], [0]) for i, rid in enumerate(rids)]
+            self.validate(entries)
+            self.reserve(entries)
+            graph = self._graph_for(entries)
+            graph.run(self, entries, tokens_on_device=previous.ids if previous is not None else None)
+            for entry in entries:
+                self.cache.advance(entry.rid, self.cache.seq_len(entry.rid) + 1)
+            self.steps += 1
+            landing[k % 2].copy_(graph.ids, non_blocking=True)      # queued before the next replay overwrites the ids
+            arrived[k % 2].record()
+            if k > 0:
+                arrived[(k - 1) % 2].synchronize()
+                picked.append(landing[(k - 1) % 2].tolist())
+                if on_step is not None and on_step(k - 1, picked[-1]) is False:
+                    go_on = False
+            previous = graph
+            if not go_on:
+                break
+        last = len(picked)
+        arrived[last % 2].synchronize()
+        picked.append(landing[last % 2].tolist())
+        if on_step is not None and go_on:
+            on_step(last, picked[-1])
+        self._graph_result = None
+        return picked
+
+    def _graph_for(self, entries: list[StepEntry]) -> "DecodeGraph":
         longest = max(self.cache.seq_len(e.rid) for e in entries) + 1
         bucket = -(-longest // self.GRAPH_BUCKET) * self.GRAPH_BUCKET
         bucket = -(-bucket // self.cache.page_size) * self.cache.page_size
@@ -183,6 +242,10 @@ class Engine:
         if graph is None:
             graph = DecodeGraph(self, entries, bucket)      # its first eager run and the capture write the same
             self.graphs[key] = graph                         # keys and values the replay writes again
+        return graph
+
+    def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
+        graph = self._graph_for(entries)
         logits = graph.run(self, entries)
         self._graph_result = graph
         return logits
