@@ -5,6 +5,12 @@
 A step is one decode step of the whole batch.  The default run prefills 8 prompts of 2,048
 random ids and decodes from there; it also times a prefill of 2,048 tokens and decoding at
 batch 1 and 64, and prints one JSON line.
+
+    python bench.py --workload mixed-1.5b | prefix-7b
+
+runs a whole serving workload through the scheduler instead (64 requests at Qwen2.5-1.5B sizes
+with prompts of 128 to 2,048 ids and 256 new tokens each; 64 requests at Qwen2.5-7B sizes that
+share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for it.
 """
 from __future__ import annotations
 
@@ -26,6 +32,10 @@ QWEN2_0_5B = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "h
               "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
               "max_position_embeddings": 32768, "sliding_window": 32768, "use_sliding_window": False,
               "max_window_layers": 21, "hidden_act": "silu"}
+QWEN2_1_5B = dict(QWEN2_0_5B, num_hidden_layers=28, hidden_size=1536, num_attention_heads=12, num_key_value_heads=2,
+                  intermediate_size=8960, max_window_layers=21)
+QWEN2_7B = dict(QWEN2_0_5B, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+                intermediate_size=18944, vocab_size=152064, tie_word_embeddings=False, max_window_layers=28)
 FULL_LAYERS = 24
 PROMPT_LEN = 2048
 CONTEXT_LEN = 4096
@@ -126,6 +136,64 @@ def run_prefill(model, repeats: int = 3):
     return best
 
 
+def run_workload(name: str, layers: int | None, dtype: str) -> dict:
+    """A serving workload through the scheduler: every request is admitted, its prompt cut into portions under
+    the token budget beside the others' decode tokens, decoded greedily to its length, and freed."""
+    import numpy as np
+    import torch
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import Engine, GenerateParams, Generated, Scheduler, SchedulerConfig, random_model
+
+    rng = np.random.default_rng(7)
+    if name == "mixed-1.5b":
+        raw, new_tokens, prefix_cache = QWEN2_1_5B, 256, False
+        lengths = [int(n) for n in rng.integers(128, 2049, size=64)]
+        prompts = [[int(t) for t in rng.integers(0, raw["vocab_size"], size=n)] for n in lengths]
+    elif name == "prefix-7b":
+        raw, new_tokens, prefix_cache = QWEN2_7B, 512, True
+        shared = [int(t) for t in rng.integers(0, raw["vocab_size"], size=1024)]
+        prompts = [shared + [int(t) for t in rng.integers(0, raw["vocab_size"], size=512)] for _ in range(64)]
+    else:
+        raise SystemExit(f"unknown workload {name!r}")
+    full_layers = raw["num_hidden_layers"]
+    cfg = Qwen2Config.from_dict(dict(raw, num_hidden_layers=layers or full_layers))
+    log(f"building random weights ({cfg.num_hidden_layers} of {full_layers} layers, {dtype})")
+    model = random_model(cfg, seed=0, dtype=dtype, device="cuda:0")
+    pages = sum(-(-(len(p) + new_tokens) // 16) for p in prompts) + 16
+    engine = Engine(model, num_pages=pages, page_size=16, max_requests=64, prefix_cache=prefix_cache)
+    log(f"{name}: {len(prompts)} requests, {sum(len(p) for p in prompts)} prompt tokens, {new_tokens} new tokens each")
+    for attempt in ("warm-up", "timed"):        # the first pass captures the decode graphs and warms the library
+        sched = Scheduler(engine, SchedulerConfig(max_batch_size=64, max_waiting=64, num_blocks=pages,
+                                                  prefix_cache=prefix_cache, max_num_batched_tokens=2048))
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        ids = [sched.add_request(prompts[0], GenerateParams.greedy(new_tokens))]
+        if prefix_cache:
+            sched.step()                         # the first request's prompt is in the cache when the others arrive
+        ids += [sched.add_request(p, GenerateParams.greedy(new_tokens)) for p in prompts[1:]]
+        results = sched.run()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        done = [results[i] for i in ids]
+        assert all(isinstance(r, Generated) and r.completion_tokens == new_tokens for r in done)
+        sched.assert_idle()                      # also gives the cached prefix pages back: the timed pass starts cold
+        log(f"{attempt} pass: {elapsed:.3f} s")
+    generated = sum(r.completion_tokens for r in done)
+    stats = sched.stats
+    return {"metric": f"output tokens/s of the workload {name} through the scheduler", "value": round(generated / elapsed, 1),
+            "unit": "tokens/s", "n_gpus": 1, "seconds": round(elapsed, 3), "higher_is_better": True,
+            "dtype": "bf16" if dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform random ids)",
+            "config": {"model": name, "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+                       "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                       "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                       "requests": len(prompts), "prompt_tokens": sum(len(p) for p in prompts),
+                       "new_tokens_each": new_tokens, "token_budget": 2048, "prefix_cache": prefix_cache,
+                       "pages": pages, "page_size": 16},
+            "scheduler": {"steps": stats.steps, "tokens_forwarded": stats.tokens_forwarded, "max_running": stats.max_running,
+                          "preemptions": stats.preemptions, "peak_pages": stats.peak_blocks,
+                          "forwarded_tokens_per_s": round(stats.tokens_forwarded / elapsed, 1)}}
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -133,13 +201,20 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    parser.add_argument("--layers", type=int, default=FULL_LAYERS)
+    parser.add_argument("--layers", type=int, default=None)
+    parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "prefix-7b"],
+                        help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; runs with --gpus > 1 are not supported")
         return 2
+
+    if args.workload:
+        print(json.dumps(run_workload(args.workload, args.layers, args.dtype)), flush=True)
+        return 0
+    args.layers = args.layers or FULL_LAYERS
 
     import torch
     from tokenizer_amd.config import Qwen2Config

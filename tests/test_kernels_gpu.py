@@ -313,6 +313,24 @@ def linear_tol(out_dtype, x, w):
     return dict(rtol=base["rtol"], atol=max(base["atol"], 8 * k ** 0.5 * 2.0 ** -24 * typical))
 
 
+@pytest.mark.parametrize("shape", [(40, 200, 2304), (64, 96, 4864), (17, 1028, 2048), (33, 64, 2056)])
+def test_linear_with_k_cut_over_workgroups(ops, ref, shape):
+    """17 to 64 rows, a long K and few output tiles: the tiled kernel cuts K over workgroups and adds the parts
+    in a fixed order; the result is the same product, the same on every run."""
+    m, n, k = shape
+    assert ops._k_splits(m, n, k) > 1
+    x = rand((m, k), torch.bfloat16, 24)
+    w = rand((n, k), torch.bfloat16, 25, 0.1)
+    bias = rand((n,), torch.float32, 26)
+    for use_bias in (True, False):
+        for out_dtype in (torch.bfloat16, torch.float32):
+            got = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
+            want = ref.linear(x, w, bias if use_bias else None, out_dtype=torch.float64)
+            torch.testing.assert_close(got.double(), want, **linear_tol(out_dtype, x, w))
+            again = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
+            assert torch.equal(got, again)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(1, 100, 72), (37, 200, 136), (130, 260, 272), (300, 1000, 64), (64, 151, 896),
                                    (8, 384, 96), (513, 130, 40)])

@@ -11,10 +11,15 @@ __device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_out(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
 
 // BK: elements of K per step; rows in LDS are BK + 8 apart (padding against bank conflicts, still 16-byte aligned).
+//
+// Split K: blockIdx.z takes `k_chunk` elements of K (a multiple of BK) and, when there are several such blocks,
+// writes its float sums into its own slab of `partial` [splits, M, N]; `splitk_reduce` then adds the slabs in
+// their fixed order (and the bias) into C.  That is for products whose output is too small to fill the device
+// with tiles but whose K is long: every compute unit streams a share of the weights.
 template <int BM, int BN, int BK, typename OutT>
 __global__ void __launch_bounds__(256)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
-                 OutT* __restrict__ C, int M, int N, int K, int lda, int ldc) {
+                 OutT* __restrict__ C, int M, int N, int K, int lda, int ldc, int k_chunk, float* __restrict__ partial) {
   constexpr int WM = BM / 2, WN = BN / 2, TMI = WM / 32, TNI = WN / 32;
   constexpr int GB_BK = BK, GB_LDS = BK + 8, CPR = BK / 8;          // 16-byte chunks per row
   constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;   // chunks per thread and K step
@@ -26,6 +31,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int k_begin = blockIdx.z * k_chunk, k_end = min(K, k_begin + k_chunk);
   floatx16 acc[TMI][TNI];
 #pragma unroll
   for (int i = 0; i < TMI; ++i)
@@ -42,7 +48,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
       const int r = c / CPR, kc = (c % CPR) * 8;
       const int m = m0 + r, k = k0 + kc;
       a_reg[i] = make_uint4(0, 0, 0, 0);
-      if (m < M && k < K) a_reg[i] = *reinterpret_cast<const uint4*>(A + (size_t)m * lda + k);
+      if (m < M && k < k_end) a_reg[i] = *reinterpret_cast<const uint4*>(A + (size_t)m * lda + k);
     }
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
@@ -50,7 +56,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
       const int r = c / CPR, kc = (c % CPR) * 8;
       const int n = n0 + r, k = k0 + kc;
       w_reg[i] = make_uint4(0, 0, 0, 0);
-      if (n < N && k < K) w_reg[i] = *reinterpret_cast<const uint4*>(W + (size_t)n * K + k);
+      if (n < N && k < k_end) w_reg[i] = *reinterpret_cast<const uint4*>(W + (size_t)n * K + k);
     }
   };
   auto stash = [&](int buf) {
@@ -66,12 +72,12 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
     }
   };
 
-  fetch(0);
+  fetch(k_begin);
   stash(0);
   __syncthreads();
   int buf = 0;
-  for (int k0 = 0; k0 < K; k0 += GB_BK) {
-    const bool more = k0 + GB_BK < K;
+  for (int k0 = k_begin; k0 < k_end; k0 += GB_BK) {
+    const bool more = k0 + GB_BK < k_end;
     if (more) fetch(k0 + GB_BK);
 #pragma unroll
     for (int ks = 0; ks < GB_BK; ks += 16) {
@@ -99,26 +105,59 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
     for (int j = 0; j < TNI; ++j) {
       const int n = n0 + wn * WN + j * 32 + (lane & 31);
       if (n >= N) continue;
-      const float b = bias ? bias[n] : 0.f;
+      const float b = (bias && !partial) ? bias[n] : 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m < M) store_out(C + (size_t)m * ldc + n, acc[i][j][r] + b);
+        if (m >= M) continue;
+        if (partial) partial[((size_t)blockIdx.z * M + m) * N + n] = acc[i][j][r];
+        else store_out(C + (size_t)m * ldc + n, acc[i][j][r] + b);
       }
     }
 }
 
+// C[m, n] = sum over the slabs (in their order) + bias: four columns a thread (N is a multiple of 4 here).
+template <typename OutT>
+__global__ void splitk_reduce(const float* __restrict__ partial, const float* __restrict__ bias, OutT* __restrict__ C,
+                              int M, int N, int ldc, int splits) {
+  const size_t quad = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t per_row = N / 4;
+  if (quad >= (size_t)M * per_row) return;
+  const int m = (int)(quad / per_row), n = (int)(quad % per_row) * 4;
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s = 0; s < splits; ++s) {
+    const float4 v = *reinterpret_cast<const float4*>(partial + ((size_t)s * M + m) * N + n);
+    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  }
+  if (bias) { sum.x += bias[n]; sum.y += bias[n + 1]; sum.z += bias[n + 2]; sum.w += bias[n + 3]; }
+  OutT* dst = C + (size_t)m * ldc + n;
+  store_out(dst, sum.x); store_out(dst + 1, sum.y); store_out(dst + 2, sum.z); store_out(dst + 3, sum.w);
+}
+
 template <int BM, int BN, int BK>
 static int launch(const void* A, const void* W, const void* bias, void* C, int M, int N, int K, int lda,
-                  int ldc, int out_dtype, hipStream_t stream) {
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+                  int ldc, int out_dtype, hipStream_t stream, int splits = 1, void* partial = nullptr) {
+  const int k_chunk = splits > 1 ? ((K + splits - 1) / splits + BK - 1) / BK * BK : K;
+  if (splits > 1) splits = (K + k_chunk - 1) / k_chunk;      // no block without a step of its own
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM, splits);
+  float* slabs = splits > 1 ? (float*)partial : nullptr;
   if (out_dtype == DT_F32)
     gemm_bf16_kernel<BM, BN, BK, float><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (const float*)bias,
-                                                              (float*)C, M, N, K, lda, ldc);
+                                                              (float*)C, M, N, K, lda, ldc, k_chunk, slabs);
   else
     gemm_bf16_kernel<BM, BN, BK, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (const float*)bias,
-                                                               (bf16_t*)C, M, N, K, lda, ldc);
-  return LAUNCH_STATUS();
+                                                               (bf16_t*)C, M, N, K, lda, ldc, k_chunk, slabs);
+  int status = LAUNCH_STATUS();
+  if (status == 0 && splits > 1) {
+    const size_t quads = (size_t)M * (N / 4);
+    const int blocks = (int)((quads + 255) / 256);
+    if (out_dtype == DT_F32)
+      splitk_reduce<float><<<blocks, 256, 0, stream>>>(slabs, (const float*)bias, (float*)C, M, N, ldc, splits);
+    else
+      splitk_reduce<bf16_t><<<blocks, 256, 0, stream>>>(slabs, (const float*)bias, (bf16_t*)C, M, N, ldc, splits);
+    status = LAUNCH_STATUS();
+  }
+  return status;
 }
 
 // K and lda must be multiples of 8 and the pointers 16-byte aligned (the host checks).
@@ -133,4 +172,13 @@ extern "C" int ta_gemm_bf16(const void* A, const void* W, const void* bias, void
     return launch<64, 64, 32>(A, W, bias, C, M, N, K, lda, ldc, out_dtype, stream);
   }
   return launch<128, 128, 32>(A, W, bias, C, M, N, K, lda, ldc, out_dtype, stream);
+}
+
+// The same product with K cut into `splits` parts (at most; parts are multiples of 64) over 64 x 64 tiles, the
+// parts' float sums added afterwards in a fixed order.  partial: room for splits * M * N floats; N % 4 == 0.
+extern "C" int ta_gemm_bf16_splitk(const void* A, const void* W, const void* bias, void* C, void* partial, int M,
+                                   int N, int K, int lda, int ldc, int out_dtype, int splits, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if ((K & 7) || (lda & 7) || (N & 3) || splits < 1 || (splits > 1 && !partial)) return -1;
+  return launch<64, 64, 64>(A, W, bias, C, M, N, K, lda, ldc, out_dtype, stream, splits, partial);
 }

@@ -52,7 +52,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual",
                      "ta_argmax", "ta_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -270,14 +270,24 @@ class Ops:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+            splits = self._k_splits(m, n, k)
+            if splits > 1:
+                # Few output tiles and a long K (the down projection of a decode batch): K is cut over
+                # workgroups so that every compute unit streams a share of the weights.
+                partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
+                self._check(self.lib.ta_gemm_bf16_splitk(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(partial),
+                                                         m, n, k, lda, n, _code(out_dtype), splits, self._stream()),
+                            "linear")
+                return out
             if (self.use_library_gemm and bias is None and out_dtype == torch.bfloat16
                     and ((m > self.SKINNY_ROWS and ((k >= 2048 and m >= 128) or m * n * k >= 2 ** 32))
-                         or (m > self.FUSED_ROWS and k >= 2048 and n <= 4096))):
+                         or (m > self.FUSED_ROWS and ((k >= 2048 and n <= 4096) or n * k >= self.LIBRARY_WEIGHT)))):
                 # Large plain products go to the vendor's library (hipBLASLt through torch), as the
                 # reference's engine uses a library for its matrix products; it is faster there than
-                # the tiled kernel of this package.  So do products of 17 to 64 rows with a long K and few
-                # output columns: the weight-streaming kernel has too few tiles for them and the library
-                # splits K.
+                # the tiled kernel of this package.  So do products of 17 to 64 rows with a big weight
+                # matrix (every tile of the weight-streaming kernel reads all the rows again, which costs more
+                # than the weights once there are more than sixteen of them) or with a long K and few output
+                # columns (too few tiles; the library splits K).
                 torch.matmul(x, weight.t(), out=out)
                 return out
             if m <= self.FUSED_ROWS or (m <= self.SKINNY_ROWS and n < self.WIDE_OUTPUT):
@@ -289,6 +299,20 @@ class Ops:
         self._check(status, "linear")
         return out
 
+    use_split_k = True
+
+    def _k_splits(self, m: int, n: int, k: int) -> int:
+        """Into how many parts the tiled kernel cuts K: more than one for 17 to 64 rows with a long K and so few
+        output tiles of 64 x 64 that they would leave most of the device idle."""
+        if not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or k < 2048 or n % 4:
+            return 1
+        tiles = -(-m // 64) * -(-n // 64)
+        if tiles >= 256:
+            return 1
+        return max(1, min(-(-512 // tiles), k // 256))
+
+    LIBRARY_WEIGHT = 2 ** 21   # weight elements from which products of 17 to 64 rows go to the library
+    GATED_LIBRARY_WEIGHT = 2 ** 24   # ... and the gated product (its activation then is a kernel of its own)
     SKINNY_ROWS = 64    # up to this many rows the weight-streaming kernel runs ...
     WIDE_OUTPUT = 32768  # ... unless there are more than 16 rows and this many output columns (the vocabulary
     #                      projection): there the rows' re-reading per tile of 16 columns costs more than tiling
@@ -303,7 +327,9 @@ class Ops:
         if out is None:
             out = torch.empty((m, inner), dtype=x.dtype, device=x.device)
         _need(tuple(out.shape) == (m, inner) and out.dtype == x.dtype and out.is_contiguous(), "gated output shape")
-        if x.dtype == torch.bfloat16 and m <= self.SKINNY_ROWS:
+        if (x.dtype == torch.bfloat16 and m <= self.SKINNY_ROWS
+                and not (self.use_library_gemm and m > self.FUSED_ROWS
+                         and weight.shape[0] * weight.shape[1] >= self.GATED_LIBRARY_WEIGHT)):
             _need(x.is_cuda and weight.is_cuda and x.dim() == 2 and x.shape[1] == weight.shape[1], "linear shapes do not fit")
             _need(x.stride(1) == 1 and weight.is_contiguous() and weight.dtype == torch.bfloat16, "linear operands")
             k = x.shape[1]
