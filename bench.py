@@ -202,6 +202,8 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--layers", type=int, default=None)
+    parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
+                        help="layer sizes of the decode benchmark (the default is the one the record is for)")
     parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
@@ -214,13 +216,15 @@ def main() -> int:
     if args.workload:
         print(json.dumps(run_workload(args.workload, args.layers, args.dtype)), flush=True)
         return 0
-    args.layers = args.layers or FULL_LAYERS
+    sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
+    full_layers = sizes["num_hidden_layers"]
+    args.layers = args.layers or full_layers
 
     import torch
     from tokenizer_amd.config import Qwen2Config
     from tokenizer_amd.engine import random_model
 
-    cfg = Qwen2Config.from_dict(dict(QWEN2_0_5B, num_hidden_layers=args.layers))
+    cfg = Qwen2Config.from_dict(dict(sizes, num_hidden_layers=args.layers))
     log(f"building random weights ({args.layers} layers, {args.dtype})")
     model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
     itemsize = 2 if args.dtype == "bfloat16" else 4
@@ -239,11 +243,11 @@ def main() -> int:
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     record = {
-        "metric": "decode tokens/s (Qwen2.5-0.5B sizes, batch %d, context %d)" % (args.batch, CONTEXT_LEN),
+        "metric": "decode tokens/s (Qwen2.5-%s sizes, batch %d, context %d)" % (args.size.upper(), args.batch, CONTEXT_LEN),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform random ids)",
-        "config": {"model": "qwen2.5-0.5b-sizes", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+        "config": {"model": "qwen2.5-%s-sizes" % args.size, "layers": args.layers, "layers_of_model": full_layers,
                    "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch, "prompt_len": PROMPT_LEN,
