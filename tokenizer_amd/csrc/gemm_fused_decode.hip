@@ -385,9 +385,20 @@ static int compute_units() {
 }
 
 // Weight rows per workgroup for the rotation epilogue, where a block pairs rows half a head apart: 16, 8 or 4.
-static int rows_per_tile(int tiles16, int rows_override) {
+// Every workgroup reads and normalises all m input rows before its share of the weights, so the choice weighs
+// the bytes the busiest compute unit has to ask for: rounds of workgroups x (prologue + its weight rows).
+static int rows_per_tile(int n_q, int n_kv, int d, int m, int k, int rows_override) {
   if (rows_override == 16 || rows_override == 8 || rows_override == 4) return rows_override;
-  return tiles16 >= 256 ? 16 : tiles16 >= 128 ? 8 : 4;
+  const long units = compute_units();
+  const long prologue = (long)m * k * 8;                   // float rows and the norm weight, once per row
+  int best = 16;
+  long best_cost = -1;
+  for (int r = 16; r >= 4; r /= 2) {
+    const long tiles = (long)(n_q + n_kv) * (d / 2 / r) + (long)n_kv * d / r;
+    const long cost = ((tiles + units - 1) / units) * (prologue + 2L * r * k * 2);
+    if (best_cost < 0 || cost < best_cost) { best = r; best_cost = cost; }
+  }
+  return best;
 }
 
 // Weight rows per workgroup elsewhere: the matrix is cut into a multiple of the compute units' number of
@@ -415,7 +426,7 @@ extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_wei
   a.out = (bf16_t*)q_out; a.ldc = n_q * d;
   a.positions = (const int*)positions; a.cos_sin = (const float*)cos_sin; a.slots = (const int*)slots;
   a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
-  a.rows = rows_per_tile(a.n / 16, rows);
+  a.rows = rows_per_tile(n_q, n_kv, d, m, k, rows);
   const int tiles = (n_q + n_kv) * (d / 2 / a.rows) + n_kv * d / a.rows;
   return launch_rows<EPI_ROPE_STORE, true>(a, tiles, waves, stream);
 }
