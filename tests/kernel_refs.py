@@ -110,10 +110,16 @@ class PlainOps:
     def can_fuse_decode(self, rows, dtype, hidden=0):
         return 0 < rows <= self.fuse_rows
 
+    def fold_norm(self, hidden):
+        return hidden <= 80          # so that the CPU tests of the engine take both routes
+
     def fused_norm_qkv_rope(self, residual, norm_weight, eps, weight, bias, positions, cos_sin, slots,
                             k_pages, v_pages, n_q, n_kv, head_dim):
-        x = torch.empty(residual.shape, dtype=weight.dtype, device=residual.device)
-        self.add_rmsnorm(residual.clone(), None, norm_weight, eps, x)
+        if norm_weight is None:                                  # the rows are normalised already
+            x = residual
+        else:
+            x = torch.empty(residual.shape, dtype=weight.dtype, device=residual.device)
+            self.add_rmsnorm(residual.clone(), None, norm_weight, eps, x)
         qkv = (x.to(self.work) @ weight.to(self.work).t())
         if bias is not None:
             qkv = qkv + bias.to(self.work)
@@ -128,8 +134,11 @@ class PlainOps:
         return holder[:, :n_q * head_dim].to(weight.dtype).contiguous()
 
     def fused_norm_gated(self, residual, norm_weight, eps, weight):
-        x = torch.empty(residual.shape, dtype=weight.dtype, device=residual.device)
-        self.add_rmsnorm(residual.clone(), None, norm_weight, eps, x)
+        if norm_weight is None:
+            x = residual
+        else:
+            x = torch.empty(residual.shape, dtype=weight.dtype, device=residual.device)
+            self.add_rmsnorm(residual.clone(), None, norm_weight, eps, x)
         gate_up = x.to(self.work) @ weight.to(self.work).t()
         inner = weight.shape[0] // 2
         g, u = gate_up[:, :inner], gate_up[:, inner:]

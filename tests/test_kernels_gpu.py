@@ -383,7 +383,8 @@ def test_skinny_rows_agree_with_the_tiled_kernel(ops, shape):
     torch.testing.assert_close(skinny, tiled, **linear_tol(torch.float32, x, w))
 
 
-@pytest.mark.parametrize("geometry", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 16), (4, 4, 128, 520, 32), (20, 2, 96, 264, 16)])
+@pytest.mark.parametrize("geometry", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 16), (4, 4, 128, 520, 32), (20, 2, 96, 264, 16),
+                                      (2, 1, 64, 1280, 16), (4, 2, 32, 2304, 16)])
 @pytest.mark.parametrize("rows", [1, 8, 16])
 def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
     n_q, n_kv, d, hidden, page_size = geometry
@@ -416,9 +417,22 @@ def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
         torch.testing.assert_close(va.float(), vb.float(), **tolerance)
         if not store:
             assert float(ka.abs().max()) == 0 and float(va.abs().max()) == 0
+        # The same from rows that are normalised already (the route of wide models): rows of a wider buffer.
+        wide = torch.zeros((rows, hidden + 8), dtype=torch.bfloat16).cuda()
+        normed = wide[:, :hidden]
+        ref.add_rmsnorm(residual.clone(), None, norm_w, 1e-6, normed)
+        kc, vc = torch.zeros_like(ka), torch.zeros_like(va)
+        qc = ops.fused_norm_qkv_rope(normed, None, 1e-6, w, bias if use_bias else None, positions, table,
+                                     slots if store else None, kc, vc, n_q, n_kv, d)
+        torch.testing.assert_close(qc.float(), qb.float(), **tolerance)
+        torch.testing.assert_close(kc.float(), kb.float(), **tolerance)
+        torch.testing.assert_close(vc.float(), vb.float(), **tolerance)
 
 
-@pytest.mark.parametrize("shape", [(1, 4864, 896), (8, 272, 96), (16, 176, 80), (5, 136, 72)])
+# The last shapes: rows of 1,280 and 2,304 elements give the waves unequal shares of K in the kernels that ask for
+# a wave's whole share at once (some waves then have steps past the end, which must add nothing).
+@pytest.mark.parametrize("shape", [(1, 4864, 896), (8, 272, 96), (16, 176, 80), (5, 136, 72), (6, 1280, 2304),
+                                   (8, 2304, 1280)])
 def test_fused_norm_gated_and_linear_add(ops, ref, shape):
     rows, inner, hidden = shape
     residual = rand((rows, hidden), torch.float32, 50, 2.0)
@@ -427,6 +441,9 @@ def test_fused_norm_gated_and_linear_add(ops, ref, shape):
     got = ops.fused_norm_gated(residual, norm_w, 1e-5, w)
     want = ref.fused_norm_gated(residual, norm_w, 1e-5, w)
     torch.testing.assert_close(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    normed = torch.empty((rows, hidden), dtype=torch.bfloat16).cuda()
+    ref.add_rmsnorm(residual.clone(), None, norm_w, 1e-5, normed)
+    torch.testing.assert_close(ops.fused_norm_gated(normed, None, 1e-5, w).float(), want.float(), rtol=2e-2, atol=2e-2)
     # residual += act @ down.T + bias
     down = rand((hidden, inner), torch.bfloat16, 53, 0.05)
     bias = rand((hidden,), torch.float32, 54)

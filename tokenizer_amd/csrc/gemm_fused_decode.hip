@@ -223,8 +223,12 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
     if constexpr (ONE) {
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
-        if (step_of(wave, u) >= full_steps) continue;
-        const bf16x8 af = NORM ? load_a(step_of(wave, u) * 32) : af_one[u];
+        // A step past the end of K is multiplied all the same, with zeros for the rows: no matrix instruction
+        // sits behind a condition (it would run whatever a lane mask says, and whether the compiler masks
+        // or branches here is its choice).  The weights of such a step were read from a clamped, valid place.
+        const int step = step_of(wave, u);
+        bf16x8 af = NORM ? load_a(min(step, max(full_steps - 1, 0)) * 32) : af_one[u];
+        if (step >= full_steps) af = fz8();
 #pragma unroll
         for (int s = 0; s < SETS; ++s)
           acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[HELD - PASSES + ps][u][s], af, acc[s], 0, 0, 0);
@@ -238,11 +242,11 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
           wc[u][0] = wf[0][u][0];
           if (SETS == 2) wc[u][SETS - 1] = wf[0][u][SETS - 1];
           af[u] = load_a(min(step_of(pair, u), full_steps - 1) * 32);
+          if (step_of(pair, u) >= full_steps) af[u] = fz8();      // past the end of K: zeros, see above
         }
         if ((pair + (UN / 2) * NW) * 2 < full_steps) load_w(0, ps, pair + (UN / 2) * NW);
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-          if (step_of(pair, u) >= full_steps) continue;
 #pragma unroll
           for (int s = 0; s < SETS; ++s)
             acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[u][s], af[u], acc[s], 0, 0, 0);
@@ -250,9 +254,9 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
       }
       if (ps + 1 < PASSES) load_w(0, ps + 1, wave);          // the next block's first batch, before this one's sums
     }
-    if ((K & 31) && wave == 0) {                             // tail of K (a multiple of 8): zero-filled
+    if (K & 31) {                                            // tail of K (a multiple of 8): zero-filled; wave 0's
       const int k = full_steps * 32;
-      const bool ok = k + 8 * g < K;
+      const bool ok = wave == 0 && k + 8 * g < K;
       const bf16x8 af = ok ? load_a(k) : fz8();
       acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ok ? *reinterpret_cast<const bf16x8*>(w0[ps] + k) : fz8(), af, acc[0], 0, 0, 0);
       if (SETS == 2)
@@ -359,6 +363,7 @@ static int launch_rows(const FusedArgs& args, int tiles, int waves, hipStream_t 
   const int k_steps = (args.k + 31) / 32;
   const bool two = args.rows > 16;
   if (waves == 0) waves = (tiles >= 1024 || k_steps <= 8) ? 4 : (tiles >= 256 || k_steps <= 64 || NORM || two) ? 8 : 16;
+  if (EPI != EPI_RESIDUAL && waves > 8) waves = 8;           // two sets of weight registers: no room at 16 waves
   if constexpr (EPI != EPI_ROPE_STORE) {
     if (two) {
       if (waves == 4) return launch_one<4, EPI, NORM, 2>(args, tiles, stream);
@@ -367,7 +372,7 @@ static int launch_rows(const FusedArgs& args, int tiles, int waves, hipStream_t 
   }
   if (waves == 4) return launch_one<4, EPI, NORM, 1>(args, tiles, stream);
   if (waves == 8 || NORM) return launch_one<8, EPI, NORM, 1>(args, tiles, stream);
-  if constexpr (!NORM) return launch_one<16, EPI, false, 1>(args, tiles, stream);
+  if constexpr (EPI == EPI_RESIDUAL) return launch_one<16, EPI, false, 1>(args, tiles, stream);
   return -1;
 }
 
@@ -387,10 +392,10 @@ static int compute_units() {
 // Weight rows per workgroup for the rotation epilogue, where a block pairs rows half a head apart: 16, 8 or 4.
 // Every workgroup reads and normalises all m input rows before its share of the weights, so the choice weighs
 // the bytes the busiest compute unit has to ask for: rounds of workgroups x (prologue + its weight rows).
-static int rows_per_tile(int n_q, int n_kv, int d, int m, int k, int rows_override) {
+static int rows_per_tile(int n_q, int n_kv, int d, int m, int k, bool norm, int rows_override) {
   if (rows_override == 16 || rows_override == 8 || rows_override == 4) return rows_override;
   const long units = compute_units();
-  const long prologue = (long)m * k * 8;                   // float rows and the norm weight, once per row
+  const long prologue = (long)m * k * (norm ? 8 : 2);       // float rows and the norm weight per row, or bfloat16 rows
   int best = 16;
   long best_cost = -1;
   for (int r = 16; r >= 4; r /= 2) {
@@ -411,6 +416,22 @@ static int rows_per_workgroup(int n_rows, int rows_override) {
   return rows < 4 ? 4 : rows;
 }
 
+static int fused_qkv_rope(const FusedArgs& base, bool norm, const void* w, const void* bias, void* q_out,
+                          const void* positions, const void* cos_sin, const void* slots, void* k_pages, void* v_pages,
+                          int m, int k, int n_q, int n_kv, int d, int page_size, int rows, int waves, hipStream_t stream) {
+  if (m <= 0) return 0;
+  if (m > 16 || (k & 7) || (d & 31)) return -1;
+  FusedArgs a = base;
+  a.w = (const bf16_t*)w; a.bias = (const float*)bias; a.m = m; a.n = (n_q + 2 * n_kv) * d; a.k = k;
+  a.out = (bf16_t*)q_out; a.ldc = n_q * d;
+  a.positions = (const int*)positions; a.cos_sin = (const float*)cos_sin; a.slots = (const int*)slots;
+  a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
+  a.rows = rows_per_tile(n_q, n_kv, d, m, k, norm, rows);
+  const int tiles = (n_q + n_kv) * (d / 2 / a.rows) + n_kv * d / a.rows;
+  if (norm) return launch_rows<EPI_ROPE_STORE, true>(a, tiles, waves, stream);
+  return launch_rows<EPI_ROPE_STORE, false>(a, tiles, waves, stream);
+}
+
 // q/k/v projection of up to 16 rows read from the float residual (normalised on the fly): bias, rotation,
 // q into `q_out` [m, n_q * d], keys and values into their pages (slots null or negative: not stored).
 // rows / waves: 0 = the launcher's choice of weight rows per workgroup and waves sharing a workgroup's K.
@@ -418,17 +439,23 @@ extern "C" int ta_fused_norm_qkv_rope(const void* residual, const void* norm_wei
                                       const void* bias, void* q_out, const void* positions, const void* cos_sin,
                                       const void* slots, void* k_pages, void* v_pages, int m, int k, int n_q,
                                       int n_kv, int d, int page_size, int rows, int waves, hipStream_t stream) {
-  if (m <= 0) return 0;
-  if (m > 16 || (k & 7) || (d & 31)) return -1;
   FusedArgs a = {};
   a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
-  a.w = (const bf16_t*)w; a.bias = (const float*)bias; a.m = m; a.n = (n_q + 2 * n_kv) * d; a.k = k;
-  a.out = (bf16_t*)q_out; a.ldc = n_q * d;
-  a.positions = (const int*)positions; a.cos_sin = (const float*)cos_sin; a.slots = (const int*)slots;
-  a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
-  a.rows = rows_per_tile(n_q, n_kv, d, m, k, rows);
-  const int tiles = (n_q + n_kv) * (d / 2 / a.rows) + n_kv * d / a.rows;
-  return launch_rows<EPI_ROPE_STORE, true>(a, tiles, waves, stream);
+  return fused_qkv_rope(a, true, w, bias, q_out, positions, cos_sin, slots, k_pages, v_pages, m, k, n_q, n_kv, d,
+                        page_size, rows, waves, stream);
+}
+
+// The same from rows that are normalised already: x bfloat16 [m, k] with row stride lda.  For wide models, where
+// normalising all rows again in every workgroup costs more than one small kernel before this one.
+extern "C" int ta_fused_qkv_rope(const void* x, int lda, const void* w, const void* bias, void* q_out,
+                                 const void* positions, const void* cos_sin, const void* slots, void* k_pages,
+                                 void* v_pages, int m, int k, int n_q, int n_kv, int d, int page_size, int rows,
+                                 int waves, hipStream_t stream) {
+  if (lda & 7) return -1;
+  FusedArgs a = {};
+  a.a = (const bf16_t*)x; a.lda = lda;
+  return fused_qkv_rope(a, false, w, bias, q_out, positions, cos_sin, slots, k_pages, v_pages, m, k, n_q, n_kv, d,
+                        page_size, rows, waves, stream);
 }
 
 // out [m, n/2] = silu(x Wg^T) * (x Wu^T), x = the normalised residual rows, W = [Wg; Wu] of shape [n, k].
@@ -441,6 +468,18 @@ extern "C" int ta_fused_norm_gated(const void* residual, const void* norm_weight
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
   a.rows = rows_per_workgroup(n / 2, rows);
   return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
+}
+
+// The same from rows that are normalised already: x bfloat16 [m, k] with row stride lda.
+extern "C" int ta_fused_gated(const void* x, int lda, const void* w, void* out, int m, int n, int k, int rows,
+                              int waves, hipStream_t stream) {
+  if (m <= 0) return 0;
+  if (m > 16 || (k & 7) || (lda & 7) || (n & 1)) return -1;
+  FusedArgs a = {};
+  a.a = (const bf16_t*)x; a.lda = lda;
+  a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
+  a.rows = rows_per_workgroup(n / 2, rows);
+  return launch_rows<EPI_GATED, false>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
 }
 
 // residual [m, n] += x W^T (+ bias), x bfloat16 [m, k] with row stride lda.

@@ -94,9 +94,11 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af, acc[s][mb], 0, 0, 0);
     }
   }
-  if ((K & 31) && wave == full_steps % NW) {              // the tail of K (a multiple of 8), zero-filled
+  if (K & 31) {
+    // The tail of K (a multiple of 8), zero-filled, is one wave's; the others multiply zeros, so that no matrix
+    // instruction sits behind a condition on the wave (it would run whatever a lane mask says).
     const int k = full_steps * 32;
-    const bool k_ok = k + 8 * g < K;
+    const bool k_ok = wave == full_steps % NW && k + 8 * g < K;
     const bf16x8 wf0 = load8(w0 + k, k_ok);
     bf16x8 wf1;
     if (GATED) wf1 = load8(w1 + k, k_ok);

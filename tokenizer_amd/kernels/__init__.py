@@ -52,7 +52,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_argmax", "ta_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -354,16 +354,30 @@ class Ops:
         cache write, the gated activation and the residual add into the same kernel.  The norm prologue
         keeps sixteen normalised rows of `hidden` elements in LDS, which bounds `hidden`."""
         return (self.use_fused_decode and dtype == torch.bfloat16 and 0 < rows <= self.FUSED_ROWS
-                and 16 * (hidden + 8) * 2 <= self.FUSED_LDS_BYTES)
+                and (not self.fold_norm(hidden) or 16 * (hidden + 8) * 2 <= self.FUSED_LDS_BYTES))
+
+    FOLD_NORM_WIDTH = 2048    # up to this model width the decode products normalise their rows themselves
+
+    def fold_norm(self, hidden: int) -> bool:
+        """Whether the fused decode products should take the norm into their prologue: every workgroup then reads
+        and normalises all rows again, which pays for narrow models (one kernel fewer) and costs more than the
+        norm's own small kernel for wide ones."""
+        return hidden <= self.FOLD_NORM_WIDTH
 
     def fused_norm_qkv_rope(self, residual, norm_weight, eps, weight, bias, positions, cos_sin, slots,
                             k_pages, v_pages, n_q: int, n_kv: int, head_dim: int) -> torch.Tensor:
         """q, k, v = rmsnorm(residual) @ weight.T + bias; q and k rotated; k and v stored into their pages
-        (when `slots` is given); returns q [M, n_q * d] in bfloat16.  residual float32 [M, K]."""
-        _dev(residual, norm_weight, weight, bias, positions, cos_sin, slots, k_pages, v_pages)
+        (when `slots` is given); returns q [M, n_q * d] in bfloat16.  residual float32 [M, K]; or, with
+        `norm_weight` None, `residual` holds the normalised rows in bfloat16 already."""
+        _dev(norm_weight, weight, bias, positions, cos_sin, slots, k_pages, v_pages)
+        _need(residual.is_cuda and residual.dim() == 2, "the rows must live on the GPU")
         m, k = residual.shape
-        _need(residual.dtype == torch.float32 and norm_weight.dtype == torch.float32 and norm_weight.numel() == k,
-              "the residual and the norm weight are float32")
+        if norm_weight is None:
+            _need(residual.dtype == torch.bfloat16 and residual.stride(1) == 1 and residual.stride(0) % 8 == 0
+                  and residual.data_ptr() % 16 == 0, "normalised rows are bfloat16 with 16-byte aligned rows")
+        else:
+            _need(residual.dtype == torch.float32 and residual.is_contiguous() and norm_weight.dtype == torch.float32
+                  and norm_weight.numel() == k, "the residual and the norm weight are float32")
         _need(weight.dtype == torch.bfloat16 and tuple(weight.shape) == ((n_q + 2 * n_kv) * head_dim, k),
               "the joined q/k/v matrix has the wrong shape")
         _need(m <= self.FUSED_ROWS and k % 8 == 0 and head_dim % 32 == 0, "sizes the fused projection does not take")
@@ -378,26 +392,37 @@ class Ops:
             _need(k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16, "pages must be bfloat16")
             page_size = self._page_size(k_pages, v_pages, n_kv, head_dim)
         q = torch.empty((m, n_q * head_dim), dtype=torch.bfloat16, device=residual.device)
-        self._check(self.lib.ta_fused_norm_qkv_rope(
-            _ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(weight), _ptr(bias), _ptr(q), _ptr(positions),
-            _ptr(cos_sin), _ptr(slots), _ptr(k_pages if slots is not None else None),
-            _ptr(v_pages if slots is not None else None), m, k, n_q, n_kv, head_dim, page_size,
-            self.fused_rows, self.fused_waves, self._stream()),
-            "fused_norm_qkv_rope")
+        tail = (_ptr(weight), _ptr(bias), _ptr(q), _ptr(positions), _ptr(cos_sin), _ptr(slots),
+                _ptr(k_pages if slots is not None else None), _ptr(v_pages if slots is not None else None),
+                m, k, n_q, n_kv, head_dim, page_size, self.fused_rows, self.fused_waves, self._stream())
+        if norm_weight is None:
+            status = self.lib.ta_fused_qkv_rope(_ptr(residual), residual.stride(0) if m > 1 else k, *tail)
+        else:
+            status = self.lib.ta_fused_norm_qkv_rope(_ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), *tail)
+        self._check(status, "fused_norm_qkv_rope")
         return q
 
     def fused_norm_gated(self, residual, norm_weight, eps, weight) -> torch.Tensor:
-        """silu(x @ Wg.T) * (x @ Wu.T) with x = rmsnorm(residual), weight = [Wg; Wu]; bfloat16 [M, I]."""
-        _dev(residual, norm_weight, weight)
+        """silu(x @ Wg.T) * (x @ Wu.T) with x = rmsnorm(residual), weight = [Wg; Wu]; bfloat16 [M, I].  With
+        `norm_weight` None, `residual` holds the normalised rows in bfloat16 already."""
+        _dev(norm_weight, weight)
+        _need(residual.is_cuda and residual.dim() == 2, "the rows must live on the GPU")
         m, k = residual.shape
-        _need(residual.dtype == torch.float32 and norm_weight.dtype == torch.float32 and norm_weight.numel() == k,
-              "the residual and the norm weight are float32")
+        if norm_weight is None:
+            _need(residual.dtype == torch.bfloat16 and residual.stride(1) == 1 and residual.stride(0) % 8 == 0
+                  and residual.data_ptr() % 16 == 0, "normalised rows are bfloat16 with 16-byte aligned rows")
+        else:
+            _need(residual.dtype == torch.float32 and residual.is_contiguous() and norm_weight.dtype == torch.float32
+                  and norm_weight.numel() == k, "the residual and the norm weight are float32")
         _need(weight.dtype == torch.bfloat16 and weight.shape[1] == k and weight.shape[0] % 2 == 0, "gate/up matrix shape")
         _need(m <= self.FUSED_ROWS and k % 8 == 0, "sizes the fused product does not take")
         out = torch.empty((m, weight.shape[0] // 2), dtype=torch.bfloat16, device=residual.device)
-        self._check(self.lib.ta_fused_norm_gated(_ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(weight),
-                                                 _ptr(out), m, weight.shape[0], k, self.fused_rows, self.fused_waves,
-                                                 self._stream()), "fused_norm_gated")
+        tail = (_ptr(weight), _ptr(out), m, weight.shape[0], k, self.fused_rows, self.fused_waves, self._stream())
+        if norm_weight is None:
+            status = self.lib.ta_fused_gated(_ptr(residual), residual.stride(0) if m > 1 else k, *tail)
+        else:
+            status = self.lib.ta_fused_norm_gated(_ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), *tail)
+        self._check(status, "fused_norm_gated")
         return out
 
     def linear_add(self, x, weight, bias, residual) -> None:

@@ -70,7 +70,11 @@ class GQAttention(Mixer):
                  and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
             return super().forward_normed(residual, delta, norm, ctx, cache)
-        q = ops.fused_norm_qkv_rope(residual, norm.weight, norm.eps, self.w_qkv, self.b_qkv, ctx.positions,
+        if getattr(ops, "fold_norm", lambda hidden: True)(residual.shape[1]):
+            rows, norm_weight = residual, norm.weight
+        else:                       # a wide model: the norm's own kernel once, not again in every workgroup
+            rows, norm_weight = norm.apply(residual, None), None
+        q = ops.fused_norm_qkv_rope(rows, norm_weight, norm.eps, self.w_qkv, self.b_qkv, ctx.positions,
                                     self.position.table(), ctx.slots[cache.group] if cache.writes else None,
                                     cache.k_pages, cache.v_pages, self.n_q, self.n_kv, self.d)
         mixed = torch.empty((q.shape[0], self.n_q * self.d), dtype=q.dtype, device=q.device)

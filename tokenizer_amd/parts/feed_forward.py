@@ -40,7 +40,10 @@ class GatedDense(FeedForward):
                  and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
             return super().forward_normed(residual, delta, norm, ctx)
-        act = ops.fused_norm_gated(residual, norm.weight, norm.eps, self.w_gate_up)
+        if getattr(ops, "fold_norm", lambda hidden: True)(residual.shape[1]):
+            act = ops.fused_norm_gated(residual, norm.weight, norm.eps, self.w_gate_up)
+        else:                       # a wide model: the norm's own kernel once, not again in every workgroup
+            act = ops.fused_norm_gated(norm.apply(residual, None), None, norm.eps, self.w_gate_up)
         ops.linear_add(act, self.w_down, None, residual)
         return None
 
