@@ -44,12 +44,12 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int head_blocks = (group + 15) / 16;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int item = blockIdx.z;
-  const int t = rows ? rows[item] : item;
+  const int t = rows ? __builtin_amdgcn_readfirstlane(rows[item]) : item;   // the same for every lane: scalar
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int heads_here = min(16, group - hb * 16);
   const int head = kvh * group + hb * 16 + col;          // valid when col < heads_here
-  const int pos = positions[t];
+  const int pos = __builtin_amdgcn_readfirstlane(positions[t]);
   // entry_of_token null: every request has one token in the batch, request e is row e (one dependent load fewer).
   const int* table = block_table + (size_t)(entry_of_token ? entry_of_token[t] : t) * table_stride;
   const int lo = (window >= 0 && pos > window) ? pos - window : 0;

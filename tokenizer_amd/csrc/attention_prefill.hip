@@ -139,10 +139,14 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int heads_here = min(HG, group - hb * HG);
   const int head0 = kvh * group + hb * HG;
   const int tile_index = gridDim.x - 1 - blockIdx.x;      // late tiles see the most keys: start them first
-  const int entry = tiles[2 * tile_index], offset = tiles[2 * tile_index + 1];
-  const int row0 = cu_q[entry] + offset;
-  const int n_valid = min(16, cu_q[entry + 1] - row0);
-  const int p0 = first_position[entry] + offset;          // position of the tile's first token
+  // What describes the tile is the same for every lane; taken through readfirstlane so that all that is derived
+  // from it (which keys are visible, which blocks need no mask) lives in scalar registers and branches on it
+  // are scalar branches.
+  const int entry = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index]);
+  const int offset = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index + 1]);
+  const int row0 = __builtin_amdgcn_readfirstlane(cu_q[entry]) + offset;
+  const int n_valid = min(16, __builtin_amdgcn_readfirstlane(cu_q[entry + 1]) - row0);
+  const int p0 = __builtin_amdgcn_readfirstlane(first_position[entry]) + offset;   // position of the tile's first token
   const int my_pos = p0 + min(col, n_valid - 1);          // padded columns repeat the last token
   const int my_row = row0 + min(col, n_valid - 1);
   const int hi = p0 + n_valid - 1;                         // last key any token of the tile sees
