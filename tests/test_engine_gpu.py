@@ -112,6 +112,57 @@ def test_long_decoding(model_folders, oracle, name, dtype):
     close(got["long"], oracle(name, ids), dtype)
 
 
+_LONG_ORACLE: dict = {}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_thousands_of_tokens_of_context(tmp_path, dtype):
+    """A context far beyond the other tests' (5,200 tokens, a position limit of 8,192): the prompt in portions of
+    2,048 and less beside a second request that decodes, then single tokens across an end of a decode graph's
+    context bucket.  Page numbers, slots and key ranges are large here; two rows of the long request and every row
+    of the short one are compared with the plain implementation."""
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import StepEntry
+    raw = dict(TINY["A"][0], max_position_embeddings=8192, sliding_window=8192, rope_theta=1000000.0)
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 11, str(tmp_path / "long"))
+    cfg, tensors = plain.load_folder(folder)
+    long_ids, short_ids = random_ids(256, 5200, 31), random_ids(256, 60, 32)
+    if "long" not in _LONG_ORACLE:                                # the same weights for both dtypes: computed once
+        _LONG_ORACLE["long"] = plain.all_logits(cfg, tensors, long_ids)
+        _LONG_ORACLE["short"] = plain.all_logits(cfg, tensors, short_ids)
+    want_long, want_short = _LONG_ORACLE["long"], _LONG_ORACLE["short"]
+    eng = engine_for(folder, dtype, max_tokens=5200 + 64 + 64, max_requests=2)
+    eng.pools.poison()
+    eng.add_request("long"), eng.add_request("short")
+    got_long, got_short = {}, {}
+    at, short_at = 0, 0
+    for portion in (2048, 2048, 1000, 3, 64):                     # 5,163 tokens in portions, the short one beside them
+        entries = [StepEntry("long", long_ids[at:at + portion], [portion - 1])]
+        take = 20 if short_at == 0 else 1
+        entries.append(StepEntry("short", short_ids[short_at:short_at + take], list(range(take))))
+        logits = eng.step(entries).float().cpu()
+        got_long[at + portion - 1] = logits[0]
+        for i in range(take):
+            got_short[short_at + i] = logits[1 + i]
+        at, short_at = at + portion, short_at + take
+    while at < len(long_ids):                                      # single tokens, through position 5,120 = 10 x 512
+        entries = [StepEntry("long", [long_ids[at]], [0])]
+        if short_at < len(short_ids):
+            entries.append(StepEntry("short", [short_ids[short_at]], [0]))
+        logits = eng.step(entries).float().cpu()
+        got_long[at] = logits[0]
+        if short_at < len(short_ids):
+            got_short[short_at] = logits[1]
+            short_at += 1
+        at += 1
+    assert len(eng.graphs) >= 2 or not eng.use_graphs
+    close(torch.stack([got_long[p] for p in sorted(got_long)]), want_long[sorted(got_long)], dtype)
+    close(torch.stack([got_short[p] for p in sorted(got_short)]), want_short[sorted(got_short)], dtype)
+    eng.end_request("long"), eng.end_request("short")
+    eng.cache.check_invariants()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", list(TINY))
 def test_first_tokens_of_a_sequence(model_folders, oracle, name, dtype):
