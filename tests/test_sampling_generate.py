@@ -200,3 +200,23 @@ def test_parse_eos_token_ids():
     for bad in ('{"bos_token_id":1}', '{"eos_token_id":[]}', '{"eos_token_id":"x"}'):
         with pytest.raises(ValueError):
             parse_eos_token_ids(bad)
+
+
+def test_engine_queues_and_runs_generations(model_folders):
+    """The entry point in the reference's manner: requests with their parameters go to the engine, `run()` returns
+    what each generated; the same as generating each alone."""
+    from cpu_engine import cpu_engine
+    from tiny_configs import random_ids
+    from tokenizer_amd.engine import Engine, GenerateParams, Generated, generate, load_model
+    from kernel_refs import PlainOps
+    folder = model_folders["A"]
+    model = load_model(folder, "float32", "cpu", ops=PlainOps())
+    engine = Engine(model, num_blocks=32, max_batch_size=3, max_num_batched_tokens=24, prefix_cache=True)
+    assert engine.cache.num_pages == 32 and engine.cache.max_requests == 3
+    prompts = [random_ids(256, n, 300 + n) for n in (5, 30, 17, 2)]
+    ids = [engine.add_request(p, GenerateParams.greedy(4 + i)) for i, p in enumerate(prompts)]
+    results = engine.run()
+    for rid, prompt, n in zip(ids, prompts, range(4, 8)):
+        assert isinstance(results[rid], Generated)
+        assert results[rid].tokens == generate(cpu_engine(folder), prompt, GenerateParams.greedy(n)).tokens
+    engine.scheduler.assert_idle()

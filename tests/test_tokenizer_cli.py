@@ -87,3 +87,17 @@ def test_command_line_arguments():
         with pytest.raises(ArgError) as err:
             parse_args(bad)
         assert word in str(err.value)
+
+
+def test_generate_takes_text_with_a_tokenizer(model_folders):
+    """`generate(model, text, params, tokenizer=...)`: the text is encoded, the sampled ids are decoded."""
+    from cpu_engine import cpu_engine
+    from tokenizer_amd.engine import GenerateParams, generate
+    tok = Tokenizer.from_json(tiny_file())
+    engine = cpu_engine(model_folders["A"])                     # vocabulary 256: every byte is a token
+    from_text = generate(engine, "bbaa!", GenerateParams.greedy(5), tokenizer=tok)
+    from_ids = generate(cpu_engine(model_folders["A"]), tok.encode("bbaa!"), GenerateParams.greedy(5))
+    assert from_text.tokens == from_ids.tokens and len(from_text.tokens) == 5
+    assert from_text.text == tok.decode_bytes(from_text.tokens).decode("utf-8", errors="replace")
+    with pytest.raises(ValueError):
+        generate(engine, "abba", GenerateParams.greedy(1))

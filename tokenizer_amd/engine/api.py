@@ -82,7 +82,15 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
     return Generated(done.tokens, done.text, done.chunks, done.reason, done.completion_tokens, prefill, decode)
 
 
-def generate(engine, prompt: list[int], params: GenerateParams, token_bytes=_no_bytes) -> Generated:
+def generate(engine, prompt, params: GenerateParams, token_bytes=_no_bytes, tokenizer=None) -> Generated:
+    """Generate from token ids, or from text when a `tokenizer` (tokenizer_amd.Tokenizer) is given: the text is
+    encoded with it and the sampled ids are decoded with it.  `engine`: an `Engine` or a bare model."""
+    if isinstance(prompt, str):
+        if tokenizer is None:
+            raise ValueError("a text prompt needs a tokenizer")
+        prompt = tokenizer.encode(prompt)
+    if tokenizer is not None and token_bytes is _no_bytes:
+        token_bytes = lambda token: tokenizer.decode_bytes([token])
     return generate_with(engine, prompt, params, token_bytes, _go_on)
 
 

@@ -125,7 +125,15 @@ class Engine:
     GRAPH_BUCKET = 512      # decode graphs are captured per batch size and per this many tokens of context
 
     def __init__(self, model: Model, num_pages: int | None = None, page_size: int = 16, max_requests: int = 8,
-                 max_tokens: int | None = None, prefix_cache: bool = False, use_graphs: bool | None = None):
+                 max_tokens: int | None = None, prefix_cache: bool = False, use_graphs: bool | None = None,
+                 num_blocks: int | None = None, max_batch_size: int | None = None,
+                 max_num_batched_tokens: int = 2048):
+        """`num_blocks` and `max_batch_size` are the reference's names (qwen-server/src/lib.rs:33-56) for
+        `num_pages` and `max_requests`; `max_num_batched_tokens` is the token budget of `run()`."""
+        num_pages = num_blocks if num_pages is None else num_pages
+        max_requests = max_batch_size if max_batch_size is not None else max_requests
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self._scheduler = None
         if num_pages is None:
             if max_tokens is None:
                 raise ValueError("give num_pages or max_tokens")
@@ -251,8 +259,28 @@ class Engine:
         return logits
 
     # ------------------------------------------------------------------ requests
-    def add_request(self, rid) -> None:
-        self.cache.add_request(rid)
+    def add_request(self, rid, params=None, **callbacks):
+        """`add_request(rid)` makes `rid` a live request for `step()`.  `add_request(prompt_ids, GenerateParams)`
+        queues a generation for `run()` instead and returns its id (a scheduler over this engine is made at the
+        first such call; `token_bytes` and `on_chunk` may be passed on)."""
+        if params is None:
+            self.cache.add_request(rid)
+            return None
+        return self.scheduler.add_request(list(rid), params, **callbacks)
+
+    @property
+    def scheduler(self):
+        """The scheduler behind `add_request(prompt, params)` and `run()`."""
+        if self._scheduler is None:
+            from .scheduler import Scheduler, SchedulerConfig
+            self._scheduler = Scheduler(self, SchedulerConfig(
+                max_batch_size=self.cache.max_requests, num_blocks=self.cache.num_pages,
+                prefix_cache=self.cache.prefix_cache, max_num_batched_tokens=self.max_num_batched_tokens))
+        return self._scheduler
+
+    def run(self):
+        """Generate for everything queued with `add_request(prompt, params)`; results by request id."""
+        return self.scheduler.run()
 
     def end_request(self, rid) -> None:
         self.cache.release(rid)
