@@ -194,6 +194,35 @@ def run_workload(name: str, layers: int | None, dtype: str) -> dict:
                           "forwarded_tokens_per_s": round(stats.tokens_forwarded / elapsed, 1)}}
 
 
+def measure_peaks() -> dict:
+    """What this device reaches on the two yardsticks of the rooflines: reading a large buffer once (a library
+    reduction over 4 GiB) and a large square bf16 product through the library."""
+    import torch
+    out = {}
+    big = torch.empty(1 << 30, dtype=torch.float32, device="cuda:0").fill_(1.0)
+    for _ in range(2):
+        big.sum()
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(10):
+        big.sum()
+    torch.cuda.synchronize()
+    out["hbm_read_gbs"] = round(10 * big.numel() * 4 / (time.perf_counter() - started) / 1e9, 1)
+    del big
+    n = 8192
+    a = torch.randn(n, n, device="cuda:0").to(torch.bfloat16)
+    b = torch.randn(n, n, device="cuda:0").to(torch.bfloat16)
+    for _ in range(3):
+        a @ b
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(20):
+        a @ b
+    torch.cuda.synchronize()
+    out["bf16_gemm_tflops"] = round(20 * 2.0 * n ** 3 / (time.perf_counter() - started) / 1e12, 1)
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -204,6 +233,7 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None)
     parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
                         help="layer sizes of the decode benchmark (the default is the one the record is for)")
+    parser.add_argument("--peaks", action="store_true", help="measure what the device reaches in HBM reads and bf16 products")
     parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
@@ -213,6 +243,9 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; runs with --gpus > 1 are not supported")
         return 2
 
+    if args.peaks:
+        print(json.dumps(measure_peaks()), flush=True)
+        return 0
     if args.workload:
         print(json.dumps(run_workload(args.workload, args.layers, args.dtype)), flush=True)
         return 0
