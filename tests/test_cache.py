@@ -88,6 +88,13 @@ def test_bytes_per_token_and_the_51_sequences():
         seqs.append(length)
     assert len(seqs) == 51
     assert sum(seqs) * per_token == 94_666_752 and used * P * per_token == 99_090_432
+    # The pool that holds exactly those pages has that many bytes in float32 and half of them in bfloat16.
+    import torch
+    from tokenizer_amd.cache import CacheManager, CachePools
+    needs = [CacheNeed("full", 2, 64)] * 24
+    manager = CacheManager(needs, num_pages=used, page_size=P, max_requests=4)
+    assert CachePools(manager, needs, torch.float32, "cpu").bytes() == 99_090_432
+    assert CachePools(manager, needs, torch.bfloat16, "cpu").bytes() * 2 == 99_090_432
 
 
 def test_shared_prefix_uses_fewer_pages_than_two_copies():
