@@ -204,8 +204,8 @@ def test_trace_run_program(model_folders, oracle, tmp_path, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
-    # The same trace with and without graph replay: decode steps of changing batch size, with prompt
-    # portions (never captured) between them, each replay checked against the eager engine.
+    # The same trace with and without graph replay: decode steps of changing batch size, with a mixed step
+    # (captured from its third appearance) between them, each replay checked against the eager engine.
     from tokenizer_amd.engine import StepEntry
     name = "B"
     vocab = TINY[name][0]["vocab_size"]
@@ -237,6 +237,52 @@ def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
         torch.testing.assert_close(got[0][0], got[1][0], rtol=0, atol=0)
         assert got[0][1] == got[1][1]
     assert len(engines[0].graphs) >= 3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recurring_step_shapes_replay_graphs_and_equal_eager_steps(model_folders, dtype, monkeypatch):
+    """A step whose shape has come up before (a prompt cut into equal portions, the same mix of portions and
+    decoded tokens) replays a captured graph.  Every replay is checked against an engine without graphs, with
+    eager steps of other shapes and synchronisations between the replays; portions of 96 tokens take the
+    vendor library's products into the graph.  The oldest graph goes when too many are kept."""
+    from tokenizer_amd.engine import Engine, StepEntry
+    name = "C"
+    vocab = TINY[name][0]["vocab_size"]
+    monkeypatch.setattr(Engine, "STEP_GRAPHS", 3)
+    engines = [engine_for(model_folders[name], dtype, max_tokens=4096, max_requests=4, use_graphs=flag)
+               for flag in (True, False)]
+    ids = random_ids(vocab, 3000, 123)
+    at = [0]
+
+    def take(n):
+        at[0] += n
+        return ids[at[0] - n:at[0]]
+
+    def both(make_entries):
+        entries = make_entries()
+        got = [eng.step(entries).float().cpu().clone() for eng in engines]
+        torch.testing.assert_close(got[0], got[1], rtol=0, atol=0)
+        return got[0]
+
+    for eng in engines:
+        for rid in range(4):
+            eng.add_request(rid)
+    for _ in range(5):                                    # equal portions of one prompt: captured at the third
+        both(lambda: [StepEntry(0, take(96), [95])])
+    assert any(not isinstance(key[0], int) for key in engines[0].graphs)
+    both(lambda: [StepEntry(1, take(33), [32])])          # another shape, eager
+    for k in range(4):                                    # a portion beside decoded tokens
+        both(lambda: [StepEntry(0, take(1), [0]), StepEntry(2, take(80), [0, 79]), StepEntry(1, take(1), [0])])
+        both(lambda: [StepEntry(1, take(7 + k), [])])     # shapes that never recur stay eager
+    for _ in range(2):
+        both(lambda: [StepEntry(3, take(96), [95])])      # the first shape again, for another request
+    for n in (13, 14, 15, 16):                            # more shapes than graphs are kept
+        for _ in range(4):
+            both(lambda: [StepEntry(3, take(n), [n - 1])])
+    kept = [key for key in engines[0].graphs if not isinstance(key[0], int)]
+    assert len(kept) == 3 and ((16, 1),) in [key[0] for key in kept]
+    for eng in engines:
+        eng.cache.check_invariants()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

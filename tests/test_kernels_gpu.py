@@ -314,9 +314,10 @@ def linear_tol(out_dtype, x, w):
 
 
 @pytest.mark.parametrize("shape", [(40, 200, 2304), (64, 96, 4864), (17, 1028, 2048), (33, 64, 2056)])
-def test_linear_with_k_cut_over_workgroups(ops, ref, shape):
+def test_linear_with_k_cut_over_workgroups(ops, ref, shape, monkeypatch):
     """17 to 64 rows, a long K and few output tiles: the tiled kernel cuts K over workgroups and adds the parts
     in a fixed order; the result is the same product, the same on every run."""
+    monkeypatch.setattr(ops, "SPLIT_K_FROM", 2048)
     m, n, k = shape
     assert ops._k_splits(m, n, k) > 1
     x = rand((m, k), torch.bfloat16, 24)
@@ -329,6 +330,25 @@ def test_linear_with_k_cut_over_workgroups(ops, ref, shape):
             torch.testing.assert_close(got.double(), want, **linear_tol(out_dtype, x, w))
             again = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
             assert torch.equal(got, again)
+
+
+@pytest.mark.parametrize("shape", [(17, 1152, 896), (64, 896, 4864), (200, 264, 136), (2048, 1152, 896)])
+def test_linear_through_the_library_and_through_own_kernels(ops, ref, shape, monkeypatch):
+    """More than sixteen bfloat16 rows go to the vendor's library, with the bias in its accumulator when the
+    caller has an exact bfloat16 copy of it; the package's own kernels give the same product."""
+    m, n, k = shape
+    x = rand((m, k), torch.bfloat16, 27)
+    w = rand((n, k), torch.bfloat16, 28, 0.1)
+    bias = rand((n,), torch.bfloat16, 29).float()
+    want = ref.linear(x, w, bias, out_dtype=torch.float64)
+    monkeypatch.setattr(ops, "use_library_gemm", True)
+    through_library = ops.linear(x, w, bias, bias_lowp=bias.to(torch.bfloat16))
+    without_copy = ops.linear(x, w, bias)                 # no exact copy: the float32 bias and own kernels
+    monkeypatch.setattr(ops, "use_library_gemm", False)
+    own = ops.linear(x, w, bias, bias_lowp=bias.to(torch.bfloat16))
+    for got in (through_library, without_copy, own):
+        torch.testing.assert_close(got.double(), want, **linear_tol(torch.bfloat16, x, w))
+    assert torch.equal(without_copy, own)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -261,7 +261,10 @@ static int launch_prefill(const void* q, int q_stride, void* out, const void* k_
                           const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
                           float scale, int max_keys, int waves, hipStream_t stream) {
   if (waves == 0) {
-    const int reach = (window >= 0 && window + 16 < max_keys) ? window + 16 : max_keys;
+    // By the context rounded up to a multiple of 512 keys, so that a launch planned for a range of contexts
+    // (one recorded in a graph) and a launch for the exact context make the same choice.
+    const int planned = (max_keys + 511) / 512 * 512;
+    const int reach = (window >= 0 && window + 16 < planned) ? window + 16 : planned;
     waves = reach > 768 ? 4 : reach > 256 ? 2 : 1;
   }
 #define GO(NWV) launch_prefill_waves<D, HG, NWV>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \

@@ -16,16 +16,15 @@ __device__ __forceinline__ void store_out(bf16_t* p, float v) { p->bits = float_
 // writes its float sums into its own slab of `partial` [splits, M, N]; `splitk_reduce` then adds the slabs in
 // their fixed order (and the bias) into C.  That is for products whose output is too small to fill the device
 // with tiles but whose K is long: every compute unit streams a share of the weights.
-template <int BM, int BN, int BK, typename OutT>
+template <int BM, int BN, int BK, typename OutT, int AHEAD = 3>
 __global__ void __launch_bounds__(256)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias,
                  OutT* __restrict__ C, int M, int N, int K, int lda, int ldc, int k_chunk, float* __restrict__ partial) {
   constexpr int WM = BM / 2, WN = BN / 2, TMI = WM / 32, TNI = WN / 32;
   constexpr int GB_BK = BK, GB_LDS = BK + 8, CPR = BK / 8;          // 16-byte chunks per row
   constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;   // chunks per thread and K step
-  // Two LDS buffers: while one K step is multiplied, the next one's tiles (already requested from
-  // memory into registers) are written into the other, so a step costs one barrier and the loads of
-  // step k+1 are in flight during the products of step k.
+  // Two LDS buffers: while one K step is multiplied, the next one's tiles (already in registers) are
+  // written into the other, so a step costs one barrier.
   __shared__ __attribute__((aligned(16))) uint16_t a_s[2][BM * GB_LDS];
   __shared__ __attribute__((aligned(16))) uint16_t w_s[2][BN * GB_LDS];
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
@@ -40,63 +39,79 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  uint4 a_reg[A_CHUNKS], w_reg[W_CHUNKS];
-  auto fetch = [&](int k0) {
+  // AHEAD steps of K are on their way from memory into registers at any time: a step's products take far less
+  // time than a trip to memory, so with one step in flight a tile's walk over K would be a chain of such trips.
+  uint4 a_reg[AHEAD][A_CHUNKS], w_reg[AHEAD][W_CHUNKS];
+  // Loads are unconditional (a row past the end reads the last row, a step past the end of K the last
+  // chunk of the row: both are valid addresses), so that the compiler can count them and wait only for the
+  // step it is about to use; what lies past the end of K is replaced by zeros on its way into LDS, and rows
+  // past the end are never stored.
+  auto fetch = [&](int k0, uint4 (&a_now)[A_CHUNKS], uint4 (&w_now)[W_CHUNKS]) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int c = tid + i * 256;
-      const int r = c / CPR, kc = (c % CPR) * 8;
-      const int m = m0 + r, k = k0 + kc;
-      a_reg[i] = make_uint4(0, 0, 0, 0);
-      if (m < M && k < k_end) a_reg[i] = *reinterpret_cast<const uint4*>(A + (size_t)m * lda + k);
+      const int m = min(m0 + c / CPR, M - 1), k = min(k0 + (c % CPR) * 8, K - 8);
+      a_now[i] = *reinterpret_cast<const uint4*>(A + (size_t)m * lda + k);
     }
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
       const int c = tid + i * 256;
-      const int r = c / CPR, kc = (c % CPR) * 8;
-      const int n = n0 + r, k = k0 + kc;
-      w_reg[i] = make_uint4(0, 0, 0, 0);
-      if (n < N && k < k_end) w_reg[i] = *reinterpret_cast<const uint4*>(W + (size_t)n * K + k);
+      const int n = min(n0 + c / CPR, N - 1), k = min(k0 + (c % CPR) * 8, K - 8);
+      w_now[i] = *reinterpret_cast<const uint4*>(W + (size_t)n * K + k);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, int k0, const uint4 (&a_now)[A_CHUNKS], const uint4 (&w_now)[W_CHUNKS]) {
+    const uint4 zero = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int c = tid + i * 256;
-      *reinterpret_cast<uint4*>(a_s[buf] + (c / CPR) * GB_LDS + (c % CPR) * 8) = a_reg[i];
+      const bool inside = k0 + (c % CPR) * 8 < k_end;
+      uint4 v = a_now[i];
+      if (!inside) v = zero;
+      *reinterpret_cast<uint4*>(a_s[buf] + (c / CPR) * GB_LDS + (c % CPR) * 8) = v;
     }
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
       const int c = tid + i * 256;
-      *reinterpret_cast<uint4*>(w_s[buf] + (c / CPR) * GB_LDS + (c % CPR) * 8) = w_reg[i];
+      const bool inside = k0 + (c % CPR) * 8 < k_end;
+      uint4 v = w_now[i];
+      if (!inside) v = zero;
+      *reinterpret_cast<uint4*>(w_s[buf] + (c / CPR) * GB_LDS + (c % CPR) * 8) = v;
     }
   };
 
-  fetch(k_begin);
-  stash(0);
+#pragma unroll
+  for (int j = 0; j < AHEAD; ++j) fetch(k_begin + j * GB_BK, a_reg[j], w_reg[j]);
+  stash(0, k_begin, a_reg[0], w_reg[0]);
   __syncthreads();
   int buf = 0;
-  for (int k0 = k_begin; k0 < k_end; k0 += GB_BK) {
-    const bool more = k0 + GB_BK < k_end;
-    if (more) fetch(k0 + GB_BK);
+  for (int k_round = k_begin; k_round < k_end; k_round += AHEAD * GB_BK) {
 #pragma unroll
-    for (int ks = 0; ks < GB_BK; ks += 16) {
-      bf16x8 af[TMI], bf[TNI];
+    for (int j = 0; j < AHEAD; ++j) {          // step k0 was fetched into registers j and sits in LDS buffer `buf`
+      const int k0 = k_round + j * GB_BK;
+      if (k0 < k_end) {                        // (no `break`: the register sets keep their fixed indices)
+        fetch(k0 + AHEAD * GB_BK, a_reg[j], w_reg[j]);
 #pragma unroll
-      for (int i = 0; i < TMI; ++i)
-        af[i] = *reinterpret_cast<const bf16x8*>(a_s[buf] + (wm * WM + i * 32 + (lane & 31)) * GB_LDS + ks + 8 * (lane >> 5));
+        for (int ks = 0; ks < GB_BK; ks += 16) {
+          bf16x8 af[TMI], bf[TNI];
 #pragma unroll
-      for (int j = 0; j < TNI; ++j)
-        bf[j] = *reinterpret_cast<const bf16x8*>(w_s[buf] + (wn * WN + j * 32 + (lane & 31)) * GB_LDS + ks + 8 * (lane >> 5));
+          for (int i = 0; i < TMI; ++i)
+            af[i] = *reinterpret_cast<const bf16x8*>(a_s[buf] + (wm * WM + i * 32 + (lane & 31)) * GB_LDS + ks + 8 * (lane >> 5));
 #pragma unroll
-      for (int i = 0; i < TMI; ++i)
+          for (int jn = 0; jn < TNI; ++jn)
+            bf[jn] = *reinterpret_cast<const bf16x8*>(w_s[buf] + (wn * WN + jn * 32 + (lane & 31)) * GB_LDS + ks + 8 * (lane >> 5));
 #pragma unroll
-        for (int j = 0; j < TNI; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+          for (int i = 0; i < TMI; ++i)
+#pragma unroll
+            for (int jn = 0; jn < TNI; ++jn)
+              acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[jn], acc[i][jn], 0, 0, 0);
+        }
+        // Nobody reads the other buffer now: its last readers passed the previous barrier.
+        if (k0 + GB_BK < k_end) stash(buf ^ 1, k0 + GB_BK, a_reg[(j + 1) % AHEAD], w_reg[(j + 1) % AHEAD]);
+        __syncthreads();
+        buf ^= 1;
+      }
     }
-    if (more) stash(buf ^ 1);      // nobody reads that buffer now: its last readers passed the previous barrier
-    __syncthreads();
-    buf ^= 1;
   }
   // Lane l holds column l%32 and rows 8*(r/4) + 4*(l/32) + r%4 of each 32x32 tile.
 #pragma unroll

@@ -64,9 +64,10 @@ def random_model(config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:
 
 
 class DecodeGraph:
-    """One captured HIP graph of a decode step: `n_entries` requests with one token each, contexts of up
-    to `bucket` tokens.  The batch's tables live in fixed buffers that are refilled before every replay;
-    the graph ends with the greedy pick, so ids are ready without a further launch."""
+    """One captured HIP graph of a step of one shape: so many entries with so many tokens and wanted places
+    each (a decode step: one token each), contexts of up to `bucket` tokens.  The batch's tables live in
+    fixed buffers that are refilled before every replay; the graph ends with the greedy pick, so ids are
+    ready without a further launch."""
 
     def __init__(self, engine: "Engine", entries: list[StepEntry], bucket: int):
         self.bucket = bucket
@@ -91,7 +92,7 @@ class DecodeGraph:
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph, pool=engine.graph_pool):
             self.logits = engine.model.decoder.forward(self.ctx, engine.layer_caches)
-            self.ids = ops.argmax(self.logits)
+            self.ids = ops.argmax(self.logits) if self.logits.shape[0] else None
         self.uploaded = None
 
     def run(self, engine: "Engine", entries: list[StepEntry], tokens_on_device: torch.Tensor | None = None) -> torch.Tensor:
@@ -122,7 +123,11 @@ class Engine:
     entries and of each entry's `want`.
     """
 
-    GRAPH_BUCKET = 512      # decode graphs are captured per batch size and per this many tokens of context
+    GRAPH_BUCKET = 512      # graphs are captured per shape of the step and per this many tokens of context
+    STEP_GRAPHS = 32        # how many graphs of other steps than plain decode steps are kept (the oldest goes)
+    GRAPH_TOKENS = 2048     # steps with more tokens than this are not captured: the device is the slower side
+    GRAPH_AFTER = 3         # a shape is captured when it comes up for this many times ...
+    SHAPES_REMEMBERED = 64  # ... among this many shapes seen last
 
     def __init__(self, model: Model, num_pages: int | None = None, page_size: int = 16, max_requests: int = 8,
                  max_tokens: int | None = None, prefix_cache: bool = False, use_graphs: bool | None = None,
@@ -154,6 +159,7 @@ class Engine:
         self.use_graphs = (model.device.type == "cuda") if use_graphs is None else use_graphs
         self.use_graphs = self.use_graphs and model.decoder.graph_safe
         self.graphs: dict[tuple, DecodeGraph] = {}
+        self._shapes_seen: dict[tuple, int] = {}
         self.graph_pool = torch.cuda.graph_pool_handle() if self.use_graphs else None
         self._graph_result: DecodeGraph | None = None
 
@@ -165,7 +171,7 @@ class Engine:
     def argmax(self, logits: torch.Tensor, rows: list[int] | None = None) -> list[int]:
         """Greedy ids of the given rows of a step's logits, picked on the device."""
         graph = self._graph_result
-        if graph is not None and logits is graph.logits:
+        if graph is not None and logits is graph.logits and graph.ids is not None:
             picked = graph.ids.cpu().tolist()           # the graph already picked them
         else:
             picked = self.model.runtime.ops.argmax(logits).cpu().tolist()
@@ -241,16 +247,49 @@ class Engine:
         self._graph_result = None
         return picked
 
-    def _graph_for(self, entries: list[StepEntry]) -> "DecodeGraph":
-        longest = max(self.cache.seq_len(e.rid) for e in entries) + 1
+    @staticmethod
+    def _shape_of(entries: list[StepEntry]):
+        """What fixes the layout of a step's tables and the sizes of its launches: the number of entries for a
+        plain decode step, else the tokens and wanted places of every entry in order."""
+        if all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            return len(entries)
+        return tuple((len(e.tokens), len(e.want)) for e in entries)
+
+    def _graph_key(self, entries: list[StepEntry]) -> tuple:
+        longest = max(self.cache.seq_len(e.rid) + len(e.tokens) for e in entries)
         bucket = -(-longest // self.GRAPH_BUCKET) * self.GRAPH_BUCKET
         bucket = -(-bucket // self.cache.page_size) * self.cache.page_size
-        key = (len(entries), bucket)
+        return (self._shape_of(entries), bucket)
+
+    def _graph_for(self, entries: list[StepEntry]) -> "DecodeGraph":
+        key = self._graph_key(entries)
         graph = self.graphs.get(key)
         if graph is None:
-            graph = DecodeGraph(self, entries, bucket)      # its first eager run and the capture write the same
+            others = [k for k in self.graphs if not isinstance(k[0], int)]
+            if not isinstance(key[0], int) and len(others) >= self.STEP_GRAPHS:
+                del self.graphs[others[0]]                   # dicts keep the order of insertion: the oldest
+            graph = DecodeGraph(self, entries, key[1])       # its first eager run and the capture write the same
             self.graphs[key] = graph                         # keys and values the replay writes again
         return graph
+
+    def _replays(self, entries: list[StepEntry]) -> bool:
+        """Whether this step replays a captured graph.  Plain decode steps always do.  Other steps (portions of
+        prompts, mixed batches) do once their shape has come up `GRAPH_AFTER` times among the last
+        `SHAPES_REMEMBERED` shapes: for short steps the host's launches, not the device, set the pace, and some
+        shapes recur at once (a prompt cut into equal portions, a full token budget of equal prompts), while
+        most mixes of a busy server never come again and are not worth a capture."""
+        if not self.use_graphs:
+            return False
+        key = self._graph_key(entries)
+        if isinstance(key[0], int) or key in self.graphs:
+            return True
+        if sum(len(e.tokens) for e in entries) > self.GRAPH_TOKENS:
+            return False
+        seen = self._shapes_seen.pop(key, 0) + 1              # back in at the young end
+        self._shapes_seen[key] = seen
+        if len(self._shapes_seen) > self.SHAPES_REMEMBERED:
+            del self._shapes_seen[next(iter(self._shapes_seen))]
+        return seen >= self.GRAPH_AFTER
 
     def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
         graph = self._graph_for(entries)
@@ -323,7 +362,7 @@ class Engine:
         self.validate(entries)
         self.reserve(entries)
         self._graph_result = None
-        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+        if self._replays(entries):
             logits = self._graph_step(entries)
         else:
             ctx = build_context(entries, self.cache, self.model.device)

@@ -214,6 +214,7 @@ class Ops:
     prefill_waves = 0          # waves that share a tile's keys in the prompt kernel: 0 lets the launcher choose
     prefill_heads_per_wave = 0    # 0: the kernel's own choice for the head size
     target_workgroups = 1024      # what the split of the key range aims at
+    PLAN_KEYS = 512               # launch shapes depend on the context only through its multiple of this
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                           n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None,
@@ -221,6 +222,9 @@ class Ops:
         """Matrix-core attention of single tokens with the key range split over workgroups."""
         n_items = qkv.shape[0] if rows is None else rows.numel()
         max_keys = (block_table.shape[1] * page_size) if max_position is None else max_position + 1
+        # The split is planned for the context rounded up to a multiple of 512 keys: a step that replays a
+        # graph captured for a whole range of contexts then splits exactly as the same step run on its own.
+        max_keys = -(-max_keys // self.PLAN_KEYS) * self.PLAN_KEYS
         if window is not None:
             max_keys = min(max_keys, window + 32)
         head_blocks = -(-(n_q // n_kv) // 16)
@@ -242,8 +246,11 @@ class Ops:
 
     # --------------------------------------------------------------------- linear
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        """out = x @ weight.T (+ bias).  x [M, K] (rows may be strided); weight [N, K]; bias float32 [N].
+               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+               bias_lowp: torch.Tensor | None = None) -> torch.Tensor:
+        """out = x @ weight.T (+ bias).  x [M, K] (rows may be strided); weight [N, K]; bias float32 [N];
+        bias_lowp: the same bias in bfloat16, given only if that copy is exact (it lets a biased product take
+        the library's path).
 
         float32 operands run on plain multiply-adds; bfloat16 operands on the matrix cores with
         float accumulation and a bfloat16 or float32 result.
@@ -272,23 +279,31 @@ class Ops:
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
             splits = self._k_splits(m, n, k)
             if splits > 1:
-                # Few output tiles and a long K (the down projection of a decode batch): K is cut over
-                # workgroups so that every compute unit streams a share of the weights.
+                # Few rows and a very long K (the down projection of a decode batch in a wide model): K is cut
+                # over workgroups so that every compute unit streams a share of the weights.
                 partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
                 self._check(self.lib.ta_gemm_bf16_splitk(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(partial),
                                                          m, n, k, lda, n, _code(out_dtype), splits, self._stream()),
                             "linear")
                 return out
-            if (self.use_library_gemm and bias is None and out_dtype == torch.bfloat16
-                    and ((m > self.SKINNY_ROWS and ((k >= 2048 and m >= 128) or m * n * k >= 2 ** 32))
+            if (self.use_library_gemm and out_dtype == torch.bfloat16 and (bias is None or bias_lowp is not None)
+                    and (m > self.SKINNY_ROWS
                          or (m > self.FUSED_ROWS and ((k >= 2048 and n <= 4096) or n * k >= self.LIBRARY_WEIGHT)))):
-                # Large plain products go to the vendor's library (hipBLASLt through torch), as the
-                # reference's engine uses a library for its matrix products; it is faster there than
-                # the tiled kernel of this package.  So do products of 17 to 64 rows with a big weight
-                # matrix (every tile of the weight-streaming kernel reads all the rows again, which costs more
-                # than the weights once there are more than sixteen of them) or with a long K and few output
-                # columns (too few tiles; the library splits K).
-                torch.matmul(x, weight.t(), out=out)
+                # Plain products of more than 64 rows go to the vendor's library (hipBLASLt through torch), as
+                # the reference's engine uses a library for its matrix products: on the device's own clock
+                # (launches recorded in a graph, weights cold) it is ahead of the tiled kernel of this package
+                # for nearly every shape of the 0.5B to 7B models.  So do products of 17 to 64 rows with a big
+                # weight matrix (every tile of the weight-streaming kernel reads all the rows again, which costs
+                # more than the weights once there are more than sixteen of them) or with a long K and few
+                # output columns (too few tiles; the library cuts K).  The bias goes into the library's
+                # accumulator as well, which takes it in bfloat16: the caller passes such a copy only if it
+                # holds the float32 bias exactly.
+                if bias is None:
+                    torch.matmul(x, weight.t(), out=out)
+                else:
+                    _need(bias_lowp.dtype == torch.bfloat16 and bias_lowp.numel() == n and bias_lowp.is_cuda,
+                          "bias_lowp must be bfloat16 [N]")
+                    torch.addmm(bias_lowp, x, weight.t(), out=out)
                 return out
             if m <= self.FUSED_ROWS or (m <= self.SKINNY_ROWS and n < self.WIDE_OUTPUT):
                 status = self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, m, n, k,
@@ -302,14 +317,16 @@ class Ops:
     use_split_k = True
 
     def _k_splits(self, m: int, n: int, k: int) -> int:
-        """Into how many parts the tiled kernel cuts K: more than one for 17 to 64 rows with a long K and so few
-        output tiles of 64 x 64 that they would leave most of the device idle."""
-        if not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or k < 2048 or n % 4:
+        """Into how many parts the tiled kernel cuts K: more than one for 17 to 64 rows with a K so long, and so
+        few output tiles of 64 x 64, that the library (which cuts K as well) falls behind."""
+        if not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or k < self.SPLIT_K_FROM or n % 4:
             return 1
         tiles = -(-m // 64) * -(-n // 64)
         if tiles >= 256:
             return 1
         return max(1, min(-(-512 // tiles), k // 256))
+
+    SPLIT_K_FROM = 8192        # the shortest K that is cut (shorter ones are the library's, or the weight-streaming kernel's)
 
     LIBRARY_WEIGHT = 2 ** 21   # weight elements from which products of 17 to 64 rows go to the library
     GATED_LIBRARY_WEIGHT = 2 ** 24   # ... and the gated product (its activation then is a kernel of its own)
