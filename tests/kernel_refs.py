@@ -87,7 +87,7 @@ class PlainOps:
             out[t] = torch.einsum("hk,khd->hd", probs, v).reshape(-1).to(out.dtype)
         return out
 
-    def linear(self, x, weight, bias=None, out=None, out_dtype=None, bias_lowp=None):
+    def linear(self, x, weight, bias=None, out=None, out_dtype=None):
         y = x.to(self.work) @ weight.to(self.work).t()
         if bias is not None:
             y = y + bias.to(self.work)

@@ -244,11 +244,15 @@ def test_recurring_step_shapes_replay_graphs_and_equal_eager_steps(model_folders
     """A step whose shape has come up before (a prompt cut into equal portions, the same mix of portions and
     decoded tokens) replays a captured graph.  Every replay is checked against an engine without graphs, with
     eager steps of other shapes and synchronisations between the replays; portions of 96 tokens take the
-    vendor library's products into the graph.  The oldest graph goes when too many are kept."""
+    vendor library's products into the graph.  When as many graphs are kept as may be, one that has not been
+    replayed for a while makes room; if none is that old, the new shape runs eagerly."""
     from tokenizer_amd.engine import Engine, StepEntry
     name = "C"
     vocab = TINY[name][0]["vocab_size"]
     monkeypatch.setattr(Engine, "STEP_GRAPHS", 3)
+    monkeypatch.setattr(Engine, "GRAPH_IDLE_STEPS", 6)
+    from tokenizer_amd.kernels import get_ops
+    monkeypatch.setattr(get_ops(), "EAGER_LIBRARY_WORK", 0)     # eager steps choose their kernels as captured ones do
     engines = [engine_for(model_folders[name], dtype, max_tokens=4096, max_requests=4, use_graphs=flag)
                for flag in (True, False)]
     ids = random_ids(vocab, 3000, 123)
@@ -279,8 +283,14 @@ def test_recurring_step_shapes_replay_graphs_and_equal_eager_steps(model_folders
     for n in (13, 14, 15, 16):                            # more shapes than graphs are kept
         for _ in range(4):
             both(lambda: [StepEntry(3, take(n), [n - 1])])
-    kept = [key for key in engines[0].graphs if not isinstance(key[0], int)]
-    assert len(kept) == 3 and ((16, 1),) in [key[0] for key in kept]
+    kept = [key[0] for key in engines[0].graphs if not isinstance(key[0], int)]
+    assert sorted(kept) == [((14, 1),), ((15, 1),), ((16, 1),)]          # the idle ones made room
+    for n in (14, 15, 16):
+        both(lambda: [StepEntry(1, take(n), [n - 1])])    # all three in use again ...
+    for _ in range(3):
+        both(lambda: [StepEntry(1, take(17), [16])])      # ... so a further shape finds no room and runs eagerly
+    kept = [key[0] for key in engines[0].graphs if not isinstance(key[0], int)]
+    assert sorted(kept) == [((14, 1),), ((15, 1),), ((16, 1),)]
     for eng in engines:
         eng.cache.check_invariants()
 

@@ -334,21 +334,23 @@ def test_linear_with_k_cut_over_workgroups(ops, ref, shape, monkeypatch):
 
 @pytest.mark.parametrize("shape", [(17, 1152, 896), (64, 896, 4864), (200, 264, 136), (2048, 1152, 896)])
 def test_linear_through_the_library_and_through_own_kernels(ops, ref, shape, monkeypatch):
-    """More than sixteen bfloat16 rows go to the vendor's library, with the bias in its accumulator when the
-    caller has an exact bfloat16 copy of it; the package's own kernels give the same product."""
+    """More than sixteen bfloat16 rows may go to the vendor's library, the float32 bias in its accumulator; the
+    package's own kernels give the same product.  Rows of the input may be strided."""
     m, n, k = shape
-    x = rand((m, k), torch.bfloat16, 27)
+    wide = rand((m, k + 24), torch.bfloat16, 27)
+    x = wide[:, 8:8 + k]                                 # strided rows, 16-byte aligned
     w = rand((n, k), torch.bfloat16, 28, 0.1)
-    bias = rand((n,), torch.bfloat16, 29).float()
-    want = ref.linear(x, w, bias, out_dtype=torch.float64)
-    monkeypatch.setattr(ops, "use_library_gemm", True)
-    through_library = ops.linear(x, w, bias, bias_lowp=bias.to(torch.bfloat16))
-    without_copy = ops.linear(x, w, bias)                 # no exact copy: the float32 bias and own kernels
-    monkeypatch.setattr(ops, "use_library_gemm", False)
-    own = ops.linear(x, w, bias, bias_lowp=bias.to(torch.bfloat16))
-    for got in (through_library, without_copy, own):
-        torch.testing.assert_close(got.double(), want, **linear_tol(torch.bfloat16, x, w))
-    assert torch.equal(without_copy, own)
+    bias = rand((n,), torch.float32, 29)
+    for use_bias in (True, False):
+        b = bias if use_bias else None
+        want = ref.linear(x, w, b, out_dtype=torch.float64)
+        monkeypatch.setattr(ops, "use_library_gemm", True)
+        monkeypatch.setattr(ops, "LIBRARY_WEIGHT", 0)    # every product of more than sixteen rows
+        through_library = ops.linear(x, w, b)
+        monkeypatch.setattr(ops, "use_library_gemm", False)
+        own = ops.linear(x, w, b)
+        for got in (through_library, own):
+            torch.testing.assert_close(got.double(), want, **linear_tol(torch.bfloat16, x, w))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

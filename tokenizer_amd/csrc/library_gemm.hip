@@ -1,0 +1,107 @@
+// C[M,N] = A[M,K] * W[N,K]^T (+ bias) in bfloat16 with float accumulation through the vendor's library
+// (hipBLASLt), called directly: the description of a product and the algorithm the library's heuristic picks
+// for it are made once per shape and kept, so that a call costs the host a few microseconds.  The reference's
+// engine uses a library for its matrix products as well.  No device code here.
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <cstdint>
+#include <mutex>
+#include <unordered_map>
+
+namespace {
+
+struct Shape {
+  int device, m, n, k, lda, ldc, bias;
+  bool operator==(const Shape& o) const {
+    return device == o.device && m == o.m && n == o.n && k == o.k && lda == o.lda && ldc == o.ldc && bias == o.bias;
+  }
+};
+struct ShapeHash {
+  size_t operator()(const Shape& s) const {
+    uint64_t h = 1469598103934665603ull;
+    for (int v : {s.device, s.m, s.n, s.k, s.lda, s.ldc, s.bias}) h = (h ^ (uint64_t)(uint32_t)v) * 1099511628211ull;
+    return (size_t)h;
+  }
+};
+struct Plan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t w = nullptr, x = nullptr, c = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+  bool usable = false;
+};
+
+std::mutex guard;
+std::unordered_map<int, hipblasLtHandle_t> handles;       // one per device
+std::unordered_map<Shape, Plan, ShapeHash> plans;
+
+// Row-major C = A W^T is, in the library's column-major terms, C^T [N x M] = op(W) [N x K] * A^T [K x M]:
+// W as stored is a K x N column-major matrix (transposed by the operation), A as stored a K x M one.
+Plan make_plan(hipblasLtHandle_t handle, const Shape& s, size_t workspace_bytes) {
+  Plan p;
+  if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return p;
+  const hipblasOperation_t trans = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+  hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &trans, sizeof(trans));
+  hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain));
+  if (s.bias) {
+    const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+    const hipDataType bias_type = HIP_R_32F;
+    const void* placeholder = nullptr;       // the pointer is set at every call
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue));
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type));
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &placeholder, sizeof(placeholder));
+  }
+  if (hipblasLtMatrixLayoutCreate(&p.w, HIP_R_16BF, s.k, s.n, s.k) != HIPBLAS_STATUS_SUCCESS) return p;
+  if (hipblasLtMatrixLayoutCreate(&p.x, HIP_R_16BF, s.k, s.m, s.lda) != HIPBLAS_STATUS_SUCCESS) return p;
+  if (hipblasLtMatrixLayoutCreate(&p.c, HIP_R_16BF, s.n, s.m, s.ldc) != HIPBLAS_STATUS_SUCCESS) return p;
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
+  hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
+                                        sizeof(workspace_bytes));
+  hipblasLtMatmulHeuristicResult_t found[1];
+  int count = 0;
+  const hipblasStatus_t status =
+      hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, 1, found, &count);
+  hipblasLtMatmulPreferenceDestroy(pref);
+  if (status == HIPBLAS_STATUS_SUCCESS && count > 0 && found[0].workspaceSize <= workspace_bytes) {
+    p.algo = found[0].algo;
+    p.workspace = found[0].workspaceSize;
+    p.usable = true;
+  }
+  return p;
+}
+
+}  // namespace
+
+// A, W, C bfloat16 (rows of A `lda` apart, of C `ldc`), bias float32 [N] or null; `workspace`: device memory
+// the library may use (the same for every call; products on one stream follow one another).
+// Returns 0; -3 if the library offers no algorithm for the shape (the caller uses a kernel of its own);
+// -1 for arguments that make no sense; 1000 + the library's status for its errors.
+extern "C" int ta_library_gemm_bf16(const void* A, const void* W, const void* bias, void* C, int M, int N, int K,
+                                    int lda, int ldc, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldc < N || !A || !W || !C) return -1;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return -1;
+  std::lock_guard<std::mutex> lock(guard);
+  auto handle_at = handles.find(device);
+  if (handle_at == handles.end()) {
+    hipblasLtHandle_t handle = nullptr;
+    const hipblasStatus_t status = hipblasLtCreate(&handle);
+    if (status != HIPBLAS_STATUS_SUCCESS) return 1000 + (int)status;
+    handle_at = handles.emplace(device, handle).first;
+  }
+  const Shape shape{device, M, N, K, lda, ldc, bias ? 1 : 0};
+  auto plan_at = plans.find(shape);
+  if (plan_at == plans.end()) plan_at = plans.emplace(shape, make_plan(handle_at->second, shape, workspace_bytes)).first;
+  Plan& plan = plan_at->second;
+  if (!plan.usable || plan.workspace > workspace_bytes) return -3;
+  if (bias)
+    hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+  const float one = 1.f, zero = 0.f;
+  const hipblasStatus_t status =
+      hipblasLtMatmul(handle_at->second, plan.desc, &one, W, plan.w, A, plan.x, &zero, C, plan.c, C, plan.c,
+                      &plan.algo, workspace, workspace_bytes, stream);
+  return status == HIPBLAS_STATUS_SUCCESS ? 0 : 1000 + (int)status;
+}

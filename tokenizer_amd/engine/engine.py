@@ -83,17 +83,23 @@ class DecodeGraph:
         self.ctx = build_context(entries, engine.cache, device, table_width=self.width, into=(self.host, self.dev))
         self.ctx.max_position = bucket - 1          # what the kernels' launch sizes are planned for
         ops = engine.model.runtime.ops
-        side = torch.cuda.Stream(device=device)
-        side.wait_stream(torch.cuda.current_stream(device))
-        with torch.cuda.stream(side):               # one eager run first, so that nothing is set up under capture
-            engine.model.decoder.forward(self.ctx, engine.layer_caches)
-        torch.cuda.current_stream(device).wait_stream(side)
-        torch.cuda.synchronize(device)
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, pool=engine.graph_pool):
-            self.logits = engine.model.decoder.forward(self.ctx, engine.layer_caches)
-            self.ids = ops.argmax(self.logits) if self.logits.shape[0] else None
+        before = getattr(ops, "capturing", False)
+        ops.capturing = True                        # kernels are chosen by their time on the device alone
+        try:
+            side = torch.cuda.Stream(device=device)
+            side.wait_stream(torch.cuda.current_stream(device))
+            with torch.cuda.stream(side):           # one eager run first, so that nothing is set up under capture
+                engine.model.decoder.forward(self.ctx, engine.layer_caches)
+            torch.cuda.current_stream(device).wait_stream(side)
+            torch.cuda.synchronize(device)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, pool=engine.graph_pool):
+                self.logits = engine.model.decoder.forward(self.ctx, engine.layer_caches)
+                self.ids = ops.argmax(self.logits) if self.logits.shape[0] else None
+        finally:
+            ops.capturing = before
         self.uploaded = None
+        self.last_used = 0
 
     def run(self, engine: "Engine", entries: list[StepEntry], tokens_on_device: torch.Tensor | None = None) -> torch.Tensor:
         """Pack the batch's description into the fixed buffers again and replay.  `tokens_on_device`: the token
@@ -124,7 +130,8 @@ class Engine:
     """
 
     GRAPH_BUCKET = 512      # graphs are captured per shape of the step and per this many tokens of context
-    STEP_GRAPHS = 32        # how many graphs of other steps than plain decode steps are kept (the oldest goes)
+    STEP_GRAPHS = 64        # how many graphs of other steps than plain decode steps are kept
+    GRAPH_IDLE_STEPS = 2000  # a kept graph makes room for another only after this many steps without a replay
     GRAPH_TOKENS = 2048     # steps with more tokens than this are not captured: the device is the slower side
     GRAPH_AFTER = 3         # a shape is captured when it comes up for this many times ...
     SHAPES_REMEMBERED = 64  # ... among this many shapes seen last
@@ -265,12 +272,23 @@ class Engine:
         key = self._graph_key(entries)
         graph = self.graphs.get(key)
         if graph is None:
-            others = [k for k in self.graphs if not isinstance(k[0], int)]
-            if not isinstance(key[0], int) and len(others) >= self.STEP_GRAPHS:
-                del self.graphs[others[0]]                   # dicts keep the order of insertion: the oldest
             graph = DecodeGraph(self, entries, key[1])       # its first eager run and the capture write the same
             self.graphs[key] = graph                         # keys and values the replay writes again
+        graph.last_used = self.steps
         return graph
+
+    def _room_for_a_graph(self) -> bool:
+        """Graphs of other steps than plain decode steps are kept up to `STEP_GRAPHS`; beyond that one makes room
+        only if it has not been replayed for `GRAPH_IDLE_STEPS` steps (else a cycle of more shapes than graphs
+        would capture every one of them again and again, which costs far more than running them eagerly)."""
+        others = [key for key in self.graphs if not isinstance(key[0], int)]
+        if len(others) < self.STEP_GRAPHS:
+            return True
+        oldest = min(others, key=lambda key: self.graphs[key].last_used)
+        if self.steps - self.graphs[oldest].last_used < self.GRAPH_IDLE_STEPS:
+            return False
+        del self.graphs[oldest]
+        return True
 
     def _replays(self, entries: list[StepEntry]) -> bool:
         """Whether this step replays a captured graph.  Plain decode steps always do.  Other steps (portions of
@@ -289,7 +307,7 @@ class Engine:
         self._shapes_seen[key] = seen
         if len(self._shapes_seen) > self.SHAPES_REMEMBERED:
             del self._shapes_seen[next(iter(self._shapes_seen))]
-        return seen >= self.GRAPH_AFTER
+        return seen >= self.GRAPH_AFTER and self._room_for_a_graph()
 
     def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
         graph = self._graph_for(entries)

@@ -29,6 +29,10 @@ def _code(dtype: torch.dtype) -> int:
         raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
 
 
+def _raw_stream(device_index: int) -> int:
+    return torch._C._cuda_getCurrentRawStream(device_index)
+
+
 def _ptr(tensor: torch.Tensor | None) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
 
@@ -53,12 +57,26 @@ class Ops:
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
-                     "ta_argmax", "ta_sample"):
+                     "ta_argmax", "ta_sample", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
+        self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
+            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        self._workspaces: dict[int, torch.Tensor] = {}
 
     @staticmethod
     def _stream() -> ctypes.c_void_p:
-        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        """The current HIP stream of the current device (the raw handle, which costs far less to ask for
+        than a stream object; every launch asks)."""
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
+
+    LIBRARY_WORKSPACE = 32 << 20       # bytes the vendor's matrix library may use per device
+
+    def _workspace(self, device: torch.device) -> torch.Tensor:
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        space = self._workspaces.get(index)
+        if space is None:
+            space = self._workspaces[index] = torch.empty(self.LIBRARY_WORKSPACE, dtype=torch.uint8, device=device)
+        return space
 
     @staticmethod
     def _check(status: int, what: str) -> None:
@@ -246,11 +264,8 @@ class Ops:
 
     # --------------------------------------------------------------------- linear
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
-               bias_lowp: torch.Tensor | None = None) -> torch.Tensor:
-        """out = x @ weight.T (+ bias).  x [M, K] (rows may be strided); weight [N, K]; bias float32 [N];
-        bias_lowp: the same bias in bfloat16, given only if that copy is exact (it lets a biased product take
-        the library's path).
+               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        """out = x @ weight.T (+ bias).  x [M, K] (rows may be strided); weight [N, K]; bias float32 [N].
 
         float32 operands run on plain multiply-adds; bfloat16 operands on the matrix cores with
         float accumulation and a bfloat16 or float32 result.
@@ -286,25 +301,28 @@ class Ops:
                                                          m, n, k, lda, n, _code(out_dtype), splits, self._stream()),
                             "linear")
                 return out
-            if (self.use_library_gemm and out_dtype == torch.bfloat16 and (bias is None or bias_lowp is not None)
-                    and (m > self.SKINNY_ROWS
-                         or (m > self.FUSED_ROWS and ((k >= 2048 and n <= 4096) or n * k >= self.LIBRARY_WEIGHT)))):
-                # Plain products of more than 64 rows go to the vendor's library (hipBLASLt through torch), as
-                # the reference's engine uses a library for its matrix products: on the device's own clock
-                # (launches recorded in a graph, weights cold) it is ahead of the tiled kernel of this package
-                # for nearly every shape of the 0.5B to 7B models.  So do products of 17 to 64 rows with a big
-                # weight matrix (every tile of the weight-streaming kernel reads all the rows again, which costs
-                # more than the weights once there are more than sixteen of them) or with a long K and few
-                # output columns (too few tiles; the library cuts K).  The bias goes into the library's
-                # accumulator as well, which takes it in bfloat16: the caller passes such a copy only if it
-                # holds the float32 bias exactly.
-                if bias is None:
-                    torch.matmul(x, weight.t(), out=out)
-                else:
-                    _need(bias_lowp.dtype == torch.bfloat16 and bias_lowp.numel() == n and bias_lowp.is_cuda,
-                          "bias_lowp must be bfloat16 [N]")
-                    torch.addmm(bias_lowp, x, weight.t(), out=out)
-                return out
+            if m > self.SKINNY_ROWS:
+                to_library = self.capturing or m * n * k >= self.EAGER_LIBRARY_WORK
+            else:
+                to_library = m > self.FUSED_ROWS and ((k >= 2048 and n <= 4096) or n * k >= self.LIBRARY_WEIGHT)
+            if to_library and self.use_library_gemm and out_dtype == torch.bfloat16:
+                # Plain products of more than 64 rows go to the vendor's library (hipBLASLt, called from
+                # library_gemm.hip), as the reference's engine uses a library for its matrix products: on the
+                # device's own clock (launches recorded in a graph, weights cold) it is ahead of the tiled
+                # kernel of this package for nearly every shape of the 0.5B to 7B models.  So do products of 17
+                # to 64 rows with a big weight matrix (every tile of the weight-streaming kernel reads all the
+                # rows again, which costs more than the weights once there are more than sixteen of them) or
+                # with a long K and few output columns (too few tiles; the library cuts K).  The float32 bias
+                # joins the library's float accumulator as it joins the kernels' own.  A launch of the library
+                # costs the host some 15 us against 4 us for a kernel of this package: outside graph capture,
+                # products of more than 64 rows that are over on the device in about that time stay with the
+                # tiled kernel (steps of small models with few tokens are bound by the host's launches).
+                space = self._workspace(x.device)
+                status = self.lib.ta_library_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
+                                                       _ptr(space), space.numel(), self._stream())
+                if status != -3:                  # -3: no algorithm for this shape, the kernels below take it
+                    self._check(status, "linear (vendor library)")
+                    return out
             if m <= self.FUSED_ROWS or (m <= self.SKINNY_ROWS and n < self.WIDE_OUTPUT):
                 status = self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, m, n, k,
                                                       _code(out_dtype), 0, self._stream())
@@ -328,6 +346,8 @@ class Ops:
 
     SPLIT_K_FROM = 8192        # the shortest K that is cut (shorter ones are the library's, or the weight-streaming kernel's)
 
+    EAGER_LIBRARY_WORK = 2 ** 30   # multiply-adds from which a product launched eagerly goes to the library
+    capturing = False          # set while a graph is recorded (and in the run that warms it up): launches are free then
     LIBRARY_WEIGHT = 2 ** 21   # weight elements from which products of 17 to 64 rows go to the library
     GATED_LIBRARY_WEIGHT = 2 ** 24   # ... and the gated product (its activation then is a kernel of its own)
     SKINNY_ROWS = 64    # up to this many rows the weight-streaming kernel runs ...

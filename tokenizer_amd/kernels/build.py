@@ -32,6 +32,11 @@ HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
                "-Wno-unused-command-line-argument"]
 
 
+# The vendor's matrix library, for the plain products that go to it (library_gemm.hip).
+ROCM_LIB_DIR = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
+LINK_FLAGS = [f"-L{ROCM_LIB_DIR}", "-lhipblaslt", f"-Wl,-rpath,{ROCM_LIB_DIR}"]
+
+
 def _say(message: str) -> None:
     print(f"[tokenizer_amd build] {message}", file=sys.stderr, flush=True)
 
@@ -107,7 +112,7 @@ def build_library(verbose: bool = True) -> str:
                 if verbose:
                     _say(f"  {name} done in {seconds:.1f} s ({time.time() - started:.0f} s elapsed)")
         partial = target + f".{os.getpid()}.tmp"
-        proc = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objects, "-o", partial],
+        proc = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objects, *LINK_FLAGS, "-o", partial],
                               capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"linking the kernel library failed:\n{proc.stderr[-4000:]}")

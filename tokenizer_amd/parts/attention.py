@@ -6,7 +6,7 @@ import math
 import torch
 
 from .base import can_fuse_decode as _can_fuse
-from .base import MIXERS, POSITIONS, Mixer, Runtime, exact_lowp
+from .base import MIXERS, POSITIONS, Mixer, Runtime
 from .norm import RMSNorm
 from .position import NoPosition, RotaryHalfSplit
 from .spec import CacheNeed, MixerSpec, PositionSpec, TensorSpec
@@ -37,7 +37,6 @@ class GQAttention(Mixer):
                                     tensors["v_proj.bias"]], dim=0).contiguous()
         self.w_o = tensors["o_proj.weight"]
         self.b_o = tensors.get("o_proj.bias") if spec.out_bias else None
-        self.b_qkv_lowp, self.b_o_lowp = exact_lowp(self.b_qkv, runtime.dtype), exact_lowp(self.b_o, runtime.dtype)
         self.scale = float(spec.scale) if spec.scale is not None else 1.0 / math.sqrt(self.d)
         self.window = spec.window
         position = spec.position or PositionSpec("none")
@@ -87,10 +86,10 @@ class GQAttention(Mixer):
 
     def forward(self, x, ctx, cache):
         ops = self.runtime.ops
-        qkv = ops.linear(x, self.w_qkv, self.b_qkv, bias_lowp=self.b_qkv_lowp)   # bias joins the float accumulator
+        qkv = ops.linear(x, self.w_qkv, self.b_qkv)   # bias joins the float accumulator
         self.position.encode_and_store(qkv, None, self.n_q, self.n_kv, self.d, ctx, cache)
         mixed = torch.empty((x.shape[0], self.n_q * self.d), dtype=x.dtype, device=x.device)
         ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
                             ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
                             self.scale, max_position=ctx.max_position, batch=ctx)
-        return ops.linear(mixed, self.w_o, self.b_o, bias_lowp=self.b_o_lowp)
+        return ops.linear(mixed, self.w_o, self.b_o)

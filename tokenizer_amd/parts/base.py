@@ -123,16 +123,6 @@ class Block:
         raise NotImplementedError
 
 
-def exact_lowp(vector, dtype):
-    """A copy of a float32 vector (a bias) in the compute dtype if that copy holds the same numbers, else None.
-    Kernel libraries whose matrix products take a bias only in the operands' dtype may use it; a bias that
-    was stored in more precision keeps the float32 path."""
-    if vector is None or dtype == vector.dtype:
-        return None
-    copy = vector.to(dtype)
-    return copy if torch.equal(copy.to(vector.dtype), vector) else None
-
-
 def can_fuse_decode(ops, residual, dtype) -> bool:
     """Whether the kernel library offers its fused decode products for these rows of the residual stream
     (few bfloat16 rows of a width whose normalised copy fits in LDS); a library without them says no."""
