@@ -125,7 +125,7 @@ template <int D, int HG, int NWV>
 __global__ void __launch_bounds__(NWV * WAVE)
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
-                         const int* __restrict__ tiles, const int* __restrict__ cu_q,
+                         const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
                          const int* __restrict__ first_position, const int* __restrict__ block_table,
                          int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
   constexpr int KS = (D + 31) / 32;
@@ -135,10 +135,16 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int col = lane & 15, g = lane >> 4;
   const int group = n_q / n_kv;
   const int head_blocks = (group + HG - 1) / HG;
-  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  // The launch is one line of workgroups, all head blocks of the last tile first, then those of the tile before
+  // it and so on: late tiles see the most keys, and every one of them should be under way before the short
+  // ones fill the device (ordered by head block instead, half of the long tiles would start only when the
+  // first half of the launch had drained, and the kernel would end with them alone on the device).
+  const int per_tile = n_kv * head_blocks;
+  const int which = blockIdx.x % per_tile;
+  const int kvh = which / head_blocks, hb = which % head_blocks;
   const int heads_here = min(HG, group - hb * HG);
   const int head0 = kvh * group + hb * HG;
-  const int tile_index = gridDim.x - 1 - blockIdx.x;      // late tiles see the most keys: start them first
+  const int tile_index = n_tiles - 1 - blockIdx.x / per_tile;
   // What describes the tile is the same for every lane; taken through readfirstlane so that all that is derived
   // from it (which keys are visible, which blocks need no mask) lives in scalar registers and branches on it
   // are scalar branches.
@@ -246,10 +252,11 @@ static int launch_prefill_waves(const void* q, int q_stride, void* out, const vo
                                 const void* block_table, int table_stride, int n_q, int n_kv, int page_size,
                                 int window, float scale, hipStream_t stream) {
   const int group = n_q / n_kv;
-  dim3 grid(n_tiles, n_kv * ((group + HG - 1) / HG));
-  prefill_attention_kernel<D, HG, NWV><<<grid, NWV * WAVE, 0, stream>>>(
+  const long workgroups = (long)n_tiles * n_kv * ((group + HG - 1) / HG);
+  if (workgroups > 0x7fffffffL) return -1;
+  prefill_attention_kernel<D, HG, NWV><<<(unsigned)workgroups, NWV * WAVE, 0, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
-      (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
+      n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
       window, scale * 1.4426950408889634f);
   return LAUNCH_STATUS();
 }
