@@ -59,14 +59,18 @@ Plan make_plan(hipblasLtHandle_t handle, const Shape& s, size_t workspace_bytes)
   if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
   hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
                                         sizeof(workspace_bytes));
-  hipblasLtMatmulHeuristicResult_t found[1];
+  // The heuristic's first choice may want more workspace than it was told there is: the first that fits is taken.
+  constexpr int CANDIDATES = 8;
+  hipblasLtMatmulHeuristicResult_t found[CANDIDATES];
   int count = 0;
   const hipblasStatus_t status =
-      hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, 1, found, &count);
+      hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, CANDIDATES, found, &count);
   hipblasLtMatmulPreferenceDestroy(pref);
-  if (status == HIPBLAS_STATUS_SUCCESS && count > 0 && found[0].workspaceSize <= workspace_bytes) {
-    p.algo = found[0].algo;
-    p.workspace = found[0].workspaceSize;
+  if (status != HIPBLAS_STATUS_SUCCESS) return p;
+  for (int i = 0; i < count && !p.usable; ++i) {
+    if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > workspace_bytes) continue;
+    p.algo = found[i].algo;
+    p.workspace = found[i].workspaceSize;
     p.usable = true;
   }
   return p;

@@ -69,7 +69,8 @@ class Ops:
         than a stream object; every launch asks)."""
         return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
 
-    LIBRARY_WORKSPACE = 32 << 20       # bytes the vendor's matrix library may use per device
+    LIBRARY_WORKSPACE = 128 << 20      # bytes the vendor's matrix library may use per device (its first choice for
+    #                                    the widest products of a 7B model wants some 60 MB)
 
     def _workspace(self, device: torch.device) -> torch.Tensor:
         index = device.index if device.index is not None else torch.cuda.current_device()
