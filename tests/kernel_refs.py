@@ -150,7 +150,7 @@ class PlainOps:
             y = y + bias.to(self.work)
         residual.add_(y.to(torch.float32))
 
-    def sample(self, logits, temperature, top_p, uniform, out=None):
+    def sample(self, logits, temperature, top_p, uniform, out=None, any_cut=True):
         from plain import qwen2_plain as plain
         result = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device) if out is None else out
         for row in range(logits.shape[0]):

@@ -545,6 +545,64 @@ def test_sampling_kernel_follows_the_reference_rules(ops, ref):
     assert ops.sample(torch.full((1, 50), float("-inf")).cuda(), ones[:1], ones[:1], us[:1]).item() == 0
 
 
+@pytest.mark.parametrize("vocab", [151936, 50257, 33])
+def test_sampling_kernel_over_large_and_tiny_vocabularies(ops, ref, vocab):
+    """A row is cut into slices that are summed by workgroups of their own, round after round: vocabularies that
+    fill every slice, that leave the last slice short, and that leave most slices empty; peaked rows (a nucleus
+    of a few tokens) and flat ones (the crossing deep in the bulk, among many tokens in one range of keys); rows
+    with and without a nucleus cut in one batch; the same draw on every run."""
+    import numpy as np
+    rng = np.random.default_rng(vocab)
+    rows, temps, tops = [], [], []
+    for case in range(12):
+        scale = [0.05, 1.0, 4.0][case % 3]
+        row = rng.normal(size=vocab).astype(np.float32) * scale
+        if case % 4 == 1:
+            row[rng.integers(0, vocab, size=5)] += 12.0            # a few tokens hold nearly all the mass
+        if case % 4 == 2:
+            row[vocab // 3:vocab // 3 + 20] = row.max()             # equal maxima: the index order decides
+        if case == 11:
+            row[:] = -np.inf
+            row[vocab - 1] = 0.5                                    # a single token that can be drawn, in the last slice
+        rows.append(row)
+        temps.append([0.6, 1.0, 1.5][case % 3])
+        tops.append([0.9, 1.0, 0.5, 1.0][case % 4])
+    logits = torch.tensor(np.stack(rows)).cuda()
+    temperature, top_p = torch.tensor(temps).cuda(), torch.tensor(tops).cuda()
+    uniform = torch.tensor(rng.random(12).astype(np.float32)).cuda()
+    got = ops.sample(logits, temperature, top_p, uniform).cpu().tolist()
+    assert got == ops.sample(logits, temperature, top_p, uniform).cpu().tolist()
+    want = ref.sample(logits, temperature, top_p, uniform).cpu().tolist()
+
+    def agree(got, want):
+        # The two may differ by how float32 sums of `vocab` weights round (the reference adds them one after the
+        # other in falling order, where the small ones at the end are partly lost; here slices are summed apart):
+        # the target, a share of the whole mass, moves by that.  In the reference's order the running mass (in
+        # float64 here) at the two tokens must lie closer together than such a sum can be off; and a token that
+        # weighs far more than that must be drawn by both.
+        heavy = 0
+        for row, (a, b) in enumerate(zip(got, want)):
+            order = np.lexsort((np.arange(vocab), -rows[row].astype(np.float64)))
+            weights = np.exp((rows[row][order].astype(np.float64) - float(rows[row].max())) / temps[row])
+            running = np.cumsum(weights)
+            place = np.empty(vocab, dtype=np.int64)
+            place[order] = np.arange(vocab)
+            slack = vocab * 2.0 ** -24 * running[-1]
+            assert abs(running[place[a]] - running[place[b]]) <= slack, (row, a, b)
+            if weights[place[b]] > 10 * slack:
+                heavy += 1
+                assert a == b, (row, a, b)
+        assert heavy >= 2
+
+    agree(got, want)
+    assert got[11] == vocab - 1
+    # Without any cut in the batch the rounds of the nucleus are not launched at all.
+    ones = torch.ones(12).cuda()
+    free = ops.sample(logits, temperature, ones, uniform, any_cut=False).cpu().tolist()
+    assert free == ops.sample(logits, temperature, ones, uniform, any_cut=True).cpu().tolist()
+    agree(free, ref.sample(logits, temperature, ones, uniform).cpu().tolist())
+
+
 @pytest.mark.parametrize("rows", [1, 3, 4, 7, 16, 19, 32])
 @pytest.mark.parametrize("waves", [0, 4, 8, 16])
 def test_fused_products_for_every_cut(ops, ref, rows, waves):

@@ -84,9 +84,16 @@ extern "C" int ta_argmax(const void* logits, void* out, void* partial_v, void* p
 // prefix whose probability reaches top_p, and walks that prefix with a uniform number until the mass is
 // used up.  Both questions are "where does the running mass, in that order, cross a value": answered here
 // by narrowing an order-preserving 32-bit key of the logit four bits at a time, each round summing the
-// weights exp((l - max) / T) of the sixteen candidate ranges (fixed summation order, so the result does not
-// change from run to run), and then counting indices among the tokens whose logit equals the crossing one.
-#define SAMPLE_THREADS 1024
+// weights exp((l - max) / T) of the sixteen candidate ranges, and then counting indices among the tokens
+// whose logit equals the crossing one.
+//
+// A row is cut into SAMPLE_PIECES slices with a workgroup each, and every round is a launch of its own: a
+// round's workgroups first add up what the round before left for their row (in the fixed order of the slices,
+// so the result does not change from run to run, and every workgroup of a row comes to the same decision),
+// then sum their slice for the next round.  Some twenty small launches replace one workgroup walking a
+// vocabulary of 150,000 twenty times on its own.
+#define SAMPLE_THREADS 256
+#define SAMPLE_PIECES 32
 
 __device__ __forceinline__ uint32_t order_key(float v) {
   // Larger float -> larger key; NaN is treated as the smallest value.
@@ -94,171 +101,416 @@ __device__ __forceinline__ uint32_t order_key(float v) {
   const uint32_t b = __float_as_uint(v);
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
-
-// Sums `vals[0..n)` over the block; every thread gets all n results in `vals`.  n <= 16.
-__device__ __forceinline__ void block_sums(float* vals, int n, float (*scratch)[16]) {
-  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-  for (int i = 0; i < n; ++i) vals[i] = wave_sum(vals[i]);
-  __syncthreads();
-  if (lane == 0)
-    for (int i = 0; i < n; ++i) scratch[wave][i] = vals[i];
-  __syncthreads();
-  for (int i = 0; i < n; ++i) {
-    float total = 0.f;
-    for (int w = 0; w < SAMPLE_THREADS / WAVE; ++w) total += scratch[w][i];
-    vals[i] = total;
-  }
+__device__ __forceinline__ float key_value(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
 }
 
-struct Crossing {
-  uint32_t key;     // key of the token at which the running mass crosses the target
-  float above;      // mass of all tokens with a larger key
-  float each;       // weight of one token with this key
-  int rank;         // how many tokens with this key (in index order) lie before the crossing one
+// What a row keeps between launches (floats and ints of one array, SAMPLE_ROW_WORDS per row).
+enum {
+  SW_MAX = 0,                                   // [PIECES] maximum of each slice
+  SW_MASS = SW_MAX + SAMPLE_PIECES,             // [PIECES] mass of each slice
+  SW_PART = SW_MASS + SAMPLE_PIECES,            // [2][PIECES][16] masses of the sixteen ranges, by round parity
+  SW_COUNT = SW_PART + 2 * SAMPLE_PIECES * 16,  // [PIECES] tokens with the picked key in each slice
+  SW_STATE = SW_COUNT + SAMPLE_PIECES,          // [2][2] (prefix, above) by round parity
+  SW_CUT = SW_STATE + 4,                        // cut_key, cut_rank, kept
+  SW_PICK = SW_CUT + 4,                         // pick_key, pick_rank
+  SAMPLE_ROW_WORDS = SW_PICK + 4
 };
 
-// Finds where the mass, taken in falling key order, first exceeds `target` (target < total mass).
-__device__ Crossing find_crossing(const float* __restrict__ row, int vocab, float max_logit, float inv_t,
-                                  float target, float (*scratch)[16]) {
-  uint32_t prefix = 0;
-  float above = 0.f;
-  for (int shift = 28; shift >= 0; shift -= 4) {
-    float part[16];
-#pragma unroll
-    for (int n = 0; n < 16; ++n) part[n] = 0.f;
-    const uint32_t mask = (shift == 28) ? 0u : (0xffffffffu << (shift + 4));
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-      const float v = row[i];
-      const uint32_t key = order_key(v);
-      if ((key & mask) != prefix) continue;
-      const float w = (v != v) ? 0.f : expf((v - max_logit) * inv_t);
-      const uint32_t nib = (key >> shift) & 15u;
-#pragma unroll
-      for (int n = 0; n < 16; ++n) part[n] += (nib == (uint32_t)n) ? w : 0.f;
-    }
-    block_sums(part, 16, scratch);
-    // Walk the ranges from the largest keys down.  If rounding leaves the target at or past the whole mass,
-    // the crossing is in the last range that holds anything.
-    int pick = -1, last = 0;
-    float run = above, run_at_last = above;
-    for (int n = 15; n >= 0; --n) {
-      if (part[n] > 0.f) { last = n; run_at_last = run; }
-      if (target < run + part[n]) { pick = n; break; }
-      run += part[n];
-    }
-    if (pick < 0) { pick = last; run = run_at_last; }
-    above = run;
-    prefix |= (uint32_t)pick << shift;
-  }
-  Crossing c;
-  c.key = prefix;
-  c.above = above;
-  c.each = 0.f;
-  c.rank = 0;
-  return c;
+struct RowFacts {
+  float max_logit, mass, inv_t;
+  bool weighable;       // a finite maximum and a finite positive mass: else the greedy choice
+};
+
+// Block-wide sum in a fixed order; every thread gets it.  `scratch`: SAMPLE_THREADS / WAVE floats.
+__device__ __forceinline__ float sample_block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & (WAVE - 1)) == 0) scratch[threadIdx.x / WAVE] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < SAMPLE_THREADS / WAVE; ++w) total += scratch[w];
+  return total;
 }
 
-// One workgroup per row.  temperature > 0.  out[row] = sampled index.
+// What the launches before left for the row, fetched into LDS by the whole workgroup at once (one trip to
+// memory instead of a chain of them): the slices' maxima and masses, and the range masses of one round
+// (`parity`, or none for -1) added up over the slices in their order.
+struct RowCopy {
+  float max_of[SAMPLE_PIECES], mass_of[SAMPLE_PIECES];
+  float part[SAMPLE_PIECES * 16];
+  float total[16];
+  float kept[SAMPLE_ROW_WORDS - SW_STATE];      // the settled state, the cut and the pick, as stored
+};
+
+__device__ __forceinline__ void fetch_row(const float* work, RowCopy& copy, int parity) {
+  constexpr int PER_THREAD = SAMPLE_PIECES * 16 / SAMPLE_THREADS;
+  static_assert(SAMPLE_PIECES * 16 % SAMPLE_THREADS == 0 && 2 * SAMPLE_PIECES <= SAMPLE_THREADS, "fetch_row's split");
+  float held[PER_THREAD], summary = 0.f;
+  if (threadIdx.x < 2 * SAMPLE_PIECES) summary = work[SW_MAX + threadIdx.x];          // maxima, then masses
+  if (parity >= 0) {
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j)
+      held[j] = work[SW_PART + parity * SAMPLE_PIECES * 16 + j * SAMPLE_THREADS + threadIdx.x];
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) copy.part[j * SAMPLE_THREADS + threadIdx.x] = held[j];
+  }
+  constexpr int KEPT = SAMPLE_ROW_WORDS - SW_STATE;
+  static_assert(2 * SAMPLE_PIECES + KEPT <= SAMPLE_THREADS, "fetch_row's split");
+  if (threadIdx.x >= 2 * SAMPLE_PIECES && threadIdx.x < 2 * SAMPLE_PIECES + KEPT)
+    copy.kept[threadIdx.x - 2 * SAMPLE_PIECES] = work[SW_STATE + threadIdx.x - 2 * SAMPLE_PIECES];
+  if (threadIdx.x < SAMPLE_PIECES) copy.max_of[threadIdx.x] = summary;
+  else if (threadIdx.x < 2 * SAMPLE_PIECES) copy.mass_of[threadIdx.x - SAMPLE_PIECES] = summary;
+  __syncthreads();
+  if (parity >= 0) {
+    if (threadIdx.x < 16) {
+      float t = 0.f;
+#pragma unroll
+      for (int g = 0; g < SAMPLE_PIECES; ++g) t += copy.part[g * 16 + threadIdx.x];
+      copy.total[threadIdx.x] = t;
+    }
+    __syncthreads();
+  }
+}
+
+__device__ __forceinline__ RowFacts row_facts(const RowCopy& copy, float temperature, bool with_mass) {
+  RowFacts f;
+  f.inv_t = 1.0f / temperature;
+  f.max_logit = -INFINITY;
+  for (int g = 0; g < SAMPLE_PIECES; ++g) f.max_logit = fmaxf(f.max_logit, copy.max_of[g]);
+  f.mass = 0.f;
+  if (with_mass)
+    for (int g = 0; g < SAMPLE_PIECES; ++g) f.mass += copy.mass_of[g];
+  f.weighable = (f.max_logit > -INFINITY) && (f.max_logit < INFINITY) && (f.mass > 0.f) && (f.mass < INFINITY);
+  return f;
+}
+
+__device__ __forceinline__ float weight_of(float v, const RowFacts& f) {
+  return (v != v) ? 0.f : expf((v - f.max_logit) * f.inv_t);
+}
+
+// One round's decision: the masses of the sixteen ranges under `prefix` (`total`, summed over the slices in their
+// order) are walked from the largest keys down until the running mass exceeds `target`.  If rounding leaves the
+// target at or past the whole mass, the crossing is in the last range that holds anything.
+__device__ __forceinline__ void walk_round(const float* total, float target, int shift, uint32_t& prefix, float& above) {
+  float held[16];
+#pragma unroll
+  for (int n = 0; n < 16; ++n) held[n] = total[n];
+  int pick = -1, last = 0;
+  float run = above, run_at_last = above;
+#pragma unroll
+  for (int n = 15; n >= 0; --n) {
+    if (pick < 0) {
+      if (held[n] > 0.f) { last = n; run_at_last = run; }
+      if (target < run + held[n]) pick = n;
+      else run += held[n];
+    }
+  }
+  if (pick < 0) { pick = last; run = run_at_last; }
+  above = run;
+  prefix |= (uint32_t)pick << shift;
+}
+
+// Where a crossing ended: the key, and how many tokens with that key (in index order) lie before the crossing one.
+__device__ __forceinline__ int rank_at(uint32_t key, float above, float target, const RowFacts& f, float& each) {
+  each = expf((key_value(key) - f.max_logit) * f.inv_t);
+  const int rank = (each > 0.f) ? (int)floorf((target - above) / each) : 0;
+  return max(rank, 0);
+}
+
+__device__ __forceinline__ void slice_of(int vocab, int& begin, int& end) {
+  const int per = (vocab + SAMPLE_PIECES - 1) / SAMPLE_PIECES;
+  begin = min(vocab, (int)blockIdx.x * per);
+  end = min(vocab, begin + per);
+}
+
+// Calls use(value, index) for every token of the slice [begin, end), each thread taking every SAMPLE_THREADS-th
+// one.  SAMPLE_BATCH loads are requested before the first is used: a slice is a few trips to memory, not one
+// per token.
+#define SAMPLE_BATCH 16
+template <typename Use>
+__device__ __forceinline__ void for_slice(const float* __restrict__ row, int begin, int end, Use use) {
+  for (int base = begin + threadIdx.x; base < end; base += SAMPLE_BATCH * SAMPLE_THREADS) {
+    float v[SAMPLE_BATCH];
+#pragma unroll
+    for (int j = 0; j < SAMPLE_BATCH; ++j) {
+      const int i = base + j * SAMPLE_THREADS;
+      v[j] = row[min(i, end - 1)];
+    }
+#pragma unroll
+    for (int j = 0; j < SAMPLE_BATCH; ++j) {
+      const int i = base + j * SAMPLE_THREADS;
+      if (i < end) use(v[j], i);
+    }
+  }
+}
+
+// Launch 1: the maximum of every slice (fmaxf skips NaN).
 __global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
-              const float* __restrict__ top_p, const float* __restrict__ uniform, int* __restrict__ out, int vocab) {
-  __shared__ float scratch[SAMPLE_THREADS / WAVE][16];
-  __shared__ int count_s[SAMPLE_THREADS];
-  __shared__ int found_s;
-  const int r = blockIdx.x;
-  const float* row = logits + (size_t)r * vocab;
-  const float inv_t = 1.0f / temperature[r];
-  // maximum
+sample_max(const float* __restrict__ logits, float* __restrict__ workspace, int vocab) {
+  __shared__ float scratch[SAMPLE_THREADS / WAVE];
+  const float* row = logits + (size_t)blockIdx.y * vocab;
+  float* work = workspace + (size_t)blockIdx.y * SAMPLE_ROW_WORDS;
+  int begin, end;
+  slice_of(vocab, begin, end);
   float mx = -INFINITY;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) mx = fmaxf(mx, row[i]);   // fmaxf skips NaN
+  for_slice(row, begin, end, [&](float v, int) { mx = fmaxf(mx, v); });
   mx = wave_max(mx);
-  __syncthreads();
-  if ((threadIdx.x & (WAVE - 1)) == 0) scratch[threadIdx.x / WAVE][0] = mx;
-  __syncthreads();
-  for (int w = 0; w < SAMPLE_THREADS / WAVE; ++w) mx = fmaxf(mx, scratch[w][0]);
-  // total mass
-  float total[1] = {0.f};
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-    const float v = row[i];
-    total[0] += (v != v) ? 0.f : expf((v - mx) * inv_t);
-  }
-  block_sums(total, 1, scratch);
-  const float mass = total[0];
-  uint32_t pick_key;
-  int pick_rank;
-  if (!(mx > -INFINITY) || !(mx < INFINITY) || !(mass > 0.f) || !(mass < INFINITY)) {
-    // Nothing to weigh (all -inf or NaN, or an infinite logit): the greedy choice, first maximum.
-    pick_key = order_key(mx);
-    pick_rank = 0;
-  } else {
-    // Nucleus: the kept prefix ends where the mass reaches top_p * total (at least the top token).
-    float kept = mass;
-    uint32_t cut_key = 0;
-    int cut_rank = 0x7fffffff;                       // tokens with key == cut_key kept: ranks 0..cut_rank
-    const float p = top_p[r];
-    if (p < 1.0f) {
-      // The reference stops at the first token with cumulative >= top_p: the crossing of a target just
-      // below top_p * mass in the "exceeds" sense.
-      const float target = fmaxf(0.f, nextafterf(p * mass, 0.f));
-      Crossing c = find_crossing(row, vocab, mx, inv_t, target, scratch);
-      const float each = expf((__uint_as_float((c.key & 0x80000000u) ? (c.key & 0x7fffffffu) : ~c.key) - mx) * inv_t);
-      int rank = (each > 0.f) ? (int)floorf((target - c.above) / each) : 0;
-      rank = max(rank, 0);
-      cut_key = c.key;
-      cut_rank = rank;
-      kept = c.above + (float)(rank + 1) * each;
-    }
-    const float target = uniform[r] * kept;
-    Crossing c = find_crossing(row, vocab, mx, inv_t, target, scratch);
-    const float each = expf((__uint_as_float((c.key & 0x80000000u) ? (c.key & 0x7fffffffu) : ~c.key) - mx) * inv_t);
-    int rank = (each > 0.f) ? (int)floorf((target - c.above) / each) : 0;
-    rank = max(rank, 0);
-    pick_key = c.key;
-    pick_rank = rank;
-    if (pick_key < cut_key || (pick_key == cut_key && pick_rank > cut_rank)) {   // past the kept prefix: its last token
-      pick_key = cut_key;
-      pick_rank = cut_rank;
-    }
-  }
-  // The pick_rank-th lowest index among the tokens whose key is pick_key (the last of them if there are fewer).
-  const int chunk = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int begin = threadIdx.x * chunk, end = min(vocab, begin + chunk);
-  int mine = 0;
-  for (int i = begin; i < end; ++i) mine += (order_key(row[i]) == pick_key) ? 1 : 0;
-  count_s[threadIdx.x] = mine;
-  if (threadIdx.x == 0) found_s = 0;
+  if ((threadIdx.x & (WAVE - 1)) == 0) scratch[threadIdx.x / WAVE] = mx;
   __syncthreads();
   if (threadIdx.x == 0) {
-    int seen = 0, all = 0;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) all += count_s[t];
-    const int want = min(pick_rank, max(all - 1, 0));
-    int owner = 0;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) {
-      if (seen + count_s[t] > want) { owner = t; break; }
-      seen += count_s[t];
-    }
-    count_s[0] = owner;           // thread that holds the token
-    found_s = want - seen;        // its rank inside that thread's chunk
-  }
-  __syncthreads();
-  const int owner = count_s[0];
-  if (threadIdx.x == owner) {
-    int left = found_s, answer = 0;
-    for (int i = begin; i < end; ++i) {
-      if (order_key(row[i]) == pick_key) {
-        if (left == 0) { answer = i; break; }
-        --left;
-      }
-    }
-    out[r] = answer;
+    for (int w = 1; w < SAMPLE_THREADS / WAVE; ++w) mx = fmaxf(mx, scratch[w]);
+    work[SW_MAX + blockIdx.x] = mx;
   }
 }
 
+// Launch 2: the mass of every slice under the row's maximum.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_mass(const float* __restrict__ logits, const float* __restrict__ temperature, float* __restrict__ workspace,
+            int vocab) {
+  __shared__ float scratch[SAMPLE_THREADS / WAVE];
+  __shared__ RowCopy copy;
+  const float* row = logits + (size_t)blockIdx.y * vocab;
+  float* work = workspace + (size_t)blockIdx.y * SAMPLE_ROW_WORDS;
+  fetch_row(work, copy, -1);
+  const RowFacts f = row_facts(copy, temperature[blockIdx.y], false);
+  int begin, end;
+  slice_of(vocab, begin, end);
+  float sum = 0.f;
+  for_slice(row, begin, end, [&](float v, int) { sum += weight_of(v, f); });
+  sum = sample_block_sum(sum, scratch);
+  if (threadIdx.x == 0) work[SW_MASS + blockIdx.x] = sum;
+}
+
+// The crossing a round belongs to: the nucleus cut (the kept prefix ends where the mass reaches top_p * total;
+// the reference stops at the first token with cumulative >= top_p, which is the crossing of a target just
+// below top_p * mass in the "exceeds" sense) or the pick (the uniform number times the kept mass).
+enum { CROSS_CUT = 0, CROSS_PICK = 1 };
+
+// What the rounds before this one have settled for the row: every workgroup of the row works it out for itself
+// (the same numbers in the same order give the same result); workgroup 0 stores it for the next launch.
+// `round` 0..7 of crossing `cross`; a round's shift is 28 - 4 * round.  Returns the crossing's target.
+__device__ float settle(float* work, const RowCopy& copy, const RowFacts& f, float top_p, float uniform, int cross,
+                        int round, bool had_cut, uint32_t& prefix, float& above) {
+  const bool writer = blockIdx.x == 0 && threadIdx.x == 0;
+  float kept = f.mass;
+  if (cross == CROSS_PICK && had_cut && top_p < 1.0f) {
+    if (round == 0) {
+      // The cut crossing's last round ended in the launch before: finish it.
+      uint32_t cut_prefix = __float_as_uint(copy.kept[2 * 1 + 0]);     // state before round 7 (odd parity)
+      float cut_above = copy.kept[2 * 1 + 1];
+      const float cut_target = fmaxf(0.f, nextafterf(top_p * f.mass, 0.f));
+      walk_round(copy.total, cut_target, 0, cut_prefix, cut_above);
+      float each;
+      const int rank = rank_at(cut_prefix, cut_above, cut_target, f, each);
+      kept = cut_above + (float)(rank + 1) * each;
+      if (writer) {
+        work[SW_CUT + 0] = __uint_as_float(cut_prefix);
+        work[SW_CUT + 1] = __int_as_float(rank);
+        work[SW_CUT + 2] = kept;
+      }
+    } else {
+      kept = copy.kept[SW_CUT - SW_STATE + 2];
+    }
+  }
+  const float target = cross == CROSS_CUT ? fmaxf(0.f, nextafterf(top_p * f.mass, 0.f)) : uniform * kept;
+  prefix = 0;
+  above = 0.f;
+  if (round > 0) {
+    // State before round - 1 (stored under that round's parity), then that round's walk.
+    const int before = (round - 1) & 1;
+    if (round > 1) {
+      prefix = __float_as_uint(copy.kept[2 * before + 0]);
+      above = copy.kept[2 * before + 1];
+    }
+    walk_round(copy.total, target, 28 - 4 * (round - 1), prefix, above);
+    if (writer) {
+      work[SW_STATE + 2 * (round & 1) + 0] = __uint_as_float(prefix);
+      work[SW_STATE + 2 * (round & 1) + 1] = above;
+    }
+  }
+  return target;
+}
+
+// Launches 3..: one round of a crossing.  Sums the masses of the sixteen ranges under the settled prefix over
+// this workgroup's slice.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_round(const float* __restrict__ logits, const float* __restrict__ temperature, const float* __restrict__ top_p,
+             const float* __restrict__ uniform, float* __restrict__ workspace, int vocab, int cross, int round,
+             int had_cut) {
+  __shared__ float bins[16][SAMPLE_THREADS + 1];            // a row one longer: the reduction's reads spread over the banks
+  __shared__ float segment[16][16];
+  __shared__ RowCopy copy;
+  const int r = blockIdx.y;
+  const float* row = logits + (size_t)r * vocab;
+  float* work = workspace + (size_t)r * SAMPLE_ROW_WORDS;
+  // The round before this one left its range masses under its parity; the pick's first round finishes the cut.
+  fetch_row(work, copy, round > 0 ? (round - 1) & 1 : (cross == CROSS_PICK && had_cut) ? 1 : -1);
+  const RowFacts f = row_facts(copy, temperature[r], true);
+  if (!f.weighable) return;                                 // the greedy choice, made at the end
+  if (cross == CROSS_CUT && !(top_p[r] < 1.0f)) return;     // everything is kept
+  uint32_t prefix;
+  float above;
+  settle(work, copy, f, top_p[r], uniform[r], cross, round, had_cut != 0, prefix, above);
+  const int shift = 28 - 4 * round;
+  const uint32_t mask = (round == 0) ? 0u : (0xffffffffu << (shift + 4));
+#pragma unroll
+  for (int n = 0; n < 16; ++n) bins[n][threadIdx.x] = 0.f;
+  int begin, end;
+  slice_of(vocab, begin, end);
+  for_slice(row, begin, end, [&](float v, int) {
+    const uint32_t key = order_key(v);
+    if ((key & mask) == prefix) bins[(key >> shift) & 15u][threadIdx.x] += weight_of(v, f);   // a thread's own column
+  });
+  // Every range's sum over the workgroup, in a fixed order: thread (n, s) adds sixteen neighbouring threads' sums
+  // of range n, then thread n adds the sixteen segments.
+  __syncthreads();
+  {
+    static_assert(SAMPLE_THREADS == 256, "sixteen ranges times sixteen segments of sixteen threads");
+    const int n = threadIdx.x & 15, seg = threadIdx.x >> 4;
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) t += bins[n][seg * 16 + k];
+    segment[n][seg] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    float total = 0.f;
+#pragma unroll
+    for (int seg = 0; seg < 16; ++seg) total += segment[threadIdx.x][seg];
+    work[SW_PART + (round & 1) * SAMPLE_PIECES * 16 + blockIdx.x * 16 + threadIdx.x] = total;
+  }
+}
+
+// After the last round of the pick: the key and rank of the drawn token (held back to the end of the kept prefix),
+// and how many tokens of each slice have that key.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_count(const float* __restrict__ logits, const float* __restrict__ temperature, const float* __restrict__ top_p,
+             const float* __restrict__ uniform, float* __restrict__ workspace, int vocab, int had_cut) {
+  __shared__ float scratch[SAMPLE_THREADS / WAVE];
+  __shared__ RowCopy copy;
+  const int r = blockIdx.y;
+  const float* row = logits + (size_t)r * vocab;
+  float* work = workspace + (size_t)r * SAMPLE_ROW_WORDS;
+  fetch_row(work, copy, 1);                                 // the pick's last round
+  const RowFacts f = row_facts(copy, temperature[r], true);
+  uint32_t pick_key;
+  int pick_rank = 0;
+  if (!f.weighable) {
+    pick_key = order_key(f.max_logit);        // nothing to weigh (all -inf or NaN, or an infinite logit): first maximum
+  } else {
+    const bool cut = had_cut && top_p[r] < 1.0f;
+    const float kept = cut ? copy.kept[SW_CUT - SW_STATE + 2] : f.mass;
+    const float target = uniform[r] * kept;
+    uint32_t prefix = __float_as_uint(copy.kept[2 * 1 + 0]);     // state before round 7
+    float above = copy.kept[2 * 1 + 1];
+    walk_round(copy.total, target, 0, prefix, above);
+    float each;
+    pick_rank = rank_at(prefix, above, target, f, each);
+    pick_key = prefix;
+    if (cut) {
+      const uint32_t cut_key = __float_as_uint(copy.kept[SW_CUT - SW_STATE + 0]);
+      const int cut_rank = __float_as_int(copy.kept[SW_CUT - SW_STATE + 1]);
+      if (pick_key < cut_key || (pick_key == cut_key && pick_rank > cut_rank)) {   // past the kept prefix: its last token
+        pick_key = cut_key;
+        pick_rank = cut_rank;
+      }
+    }
+  }
+  int begin, end;
+  slice_of(vocab, begin, end);
+  float mine = 0.f;                                          // counts stay exact in float (a slice is far below 2^24)
+  for_slice(row, begin, end, [&](float v, int) { mine += (order_key(v) == pick_key) ? 1.f : 0.f; });
+  mine = sample_block_sum(mine, scratch);
+  if (threadIdx.x == 0) {
+    work[SW_COUNT + blockIdx.x] = mine;
+    if (blockIdx.x == 0) {
+      work[SW_PICK + 0] = __uint_as_float(pick_key);
+      work[SW_PICK + 1] = __int_as_float(pick_rank);
+    }
+  }
+}
+
+// Last launch: the pick_rank-th lowest index among the tokens whose key is pick_key (the last of them if there
+// are fewer); the workgroup whose slice holds it writes it.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_locate(const float* __restrict__ logits, const float* __restrict__ workspace, int* __restrict__ out, int vocab) {
+  __shared__ int wave_count[SAMPLE_THREADS / WAVE];
+  const int r = blockIdx.y;
+  const float* row = logits + (size_t)r * vocab;
+  const float* work = workspace + (size_t)r * SAMPLE_ROW_WORDS;
+  const uint32_t pick_key = __float_as_uint(work[SW_PICK + 0]);
+  const int pick_rank = __float_as_int(work[SW_PICK + 1]);
+  __shared__ int count_of[SAMPLE_PIECES];
+  if (threadIdx.x < SAMPLE_PIECES) count_of[threadIdx.x] = (int)work[SW_COUNT + threadIdx.x];
+  __syncthreads();
+  int all = 0, before = 0;
+  for (int g = 0; g < SAMPLE_PIECES; ++g) {
+    if (g < (int)blockIdx.x) before += count_of[g];
+    all += count_of[g];
+  }
+  const int here = count_of[blockIdx.x];
+  if (all == 0) {                                           // no token has the key (cannot be, but never leave out[r] unset)
+    if (blockIdx.x == 0 && threadIdx.x == 0) out[r] = 0;
+    return;
+  }
+  const int want = min(pick_rank, all - 1);
+  if (want < before || want >= before + here) return;      // another slice's
+  int left = want - before;                                 // matches of this slice to pass over
+  int begin, end;
+  slice_of(vocab, begin, end);
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  for (int batch = begin; batch < end; batch += SAMPLE_BATCH * SAMPLE_THREADS) {
+    float v[SAMPLE_BATCH];
+#pragma unroll
+    for (int j = 0; j < SAMPLE_BATCH; ++j) v[j] = row[min(batch + j * SAMPLE_THREADS + (int)threadIdx.x, end - 1)];
+#pragma unroll 1
+    for (int j = 0; j < SAMPLE_BATCH; ++j) {                 // 256 consecutive tokens at a time, in order
+      const int base = batch + j * SAMPLE_THREADS;
+      if (base >= end) return;
+      const int i = base + threadIdx.x;
+      float mine = v[0];
+#pragma unroll
+      for (int q = 1; q < SAMPLE_BATCH; ++q) mine = (q == j) ? v[q] : mine;     // registers have no index
+      const bool match = i < end && order_key(mine) == pick_key;
+      const unsigned long long votes = __ballot(match);
+      __syncthreads();
+      if (lane == 0) wave_count[wave] = __popcll(votes);
+      __syncthreads();
+      int in_block = 0, before_wave = 0;
+      for (int w = 0; w < SAMPLE_THREADS / WAVE; ++w) {
+        if (w < wave) before_wave += wave_count[w];
+        in_block += wave_count[w];
+      }
+      if (left < in_block) {
+        const int my_place = before_wave + __popcll(votes & ((1ull << lane) - 1ull));
+        if (match && my_place == left) out[r] = i;
+        return;
+      }
+      left -= in_block;
+    }
+  }
+}
+
+// Floats of workspace a row needs.
+extern "C" int ta_sample_workspace_words() { return SAMPLE_ROW_WORDS; }
+
+// workspace: n_rows * ta_sample_workspace_words() floats.  any_cut: 0 if no row has top_p < 1 (the rounds of the
+// nucleus cut are then left out).
 extern "C" int ta_sample(const void* logits, const void* temperature, const void* top_p, const void* uniform,
-                         void* out, int n_rows, int vocab, hipStream_t stream) {
+                         void* out, void* workspace, int n_rows, int vocab, int any_cut, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (vocab < 1) return -1;
-  sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>((const float*)logits, (const float*)temperature,
-                                                      (const float*)top_p, (const float*)uniform, (int*)out, vocab);
+  if (vocab < 1 || !workspace) return -1;
+  const dim3 grid(SAMPLE_PIECES, n_rows);
+  const float* lg = (const float*)logits;
+  const float *t = (const float*)temperature, *p = (const float*)top_p, *u = (const float*)uniform;
+  float* work = (float*)workspace;
+  sample_max<<<grid, SAMPLE_THREADS, 0, stream>>>(lg, work, vocab);
+  sample_mass<<<grid, SAMPLE_THREADS, 0, stream>>>(lg, t, work, vocab);
+  for (int cross = any_cut ? CROSS_CUT : CROSS_PICK; cross <= CROSS_PICK; ++cross)
+    for (int round = 0; round < 8; ++round)
+      sample_round<<<grid, SAMPLE_THREADS, 0, stream>>>(lg, t, p, u, work, vocab, cross, round, any_cut);
+  sample_count<<<grid, SAMPLE_THREADS, 0, stream>>>(lg, t, p, u, work, vocab, any_cut);
+  sample_locate<<<grid, SAMPLE_THREADS, 0, stream>>>(lg, work, (int*)out, vocab);
   return LAUNCH_STATUS();
 }

@@ -192,7 +192,7 @@ class Engine:
         picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=device)]
         as_tensor = lambda values: torch.tensor(values, dtype=torch.float32, device=device)
         ids = self.model.runtime.ops.sample(picked.contiguous(), as_tensor(temperature), as_tensor(top_p),
-                                            as_tensor(uniform))
+                                            as_tensor(uniform), any_cut=any(p < 1.0 for p in top_p))
         return [int(v) for v in ids.cpu().tolist()]
 
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):

@@ -57,7 +57,7 @@ class Ops:
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
-                     "ta_argmax", "ta_sample", "ta_library_gemm_bf16"):
+                     "ta_argmax", "ta_sample", "ta_sample_workspace_words", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
@@ -496,10 +496,12 @@ class Ops:
 
 
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniform: torch.Tensor,
-               out: torch.Tensor | None = None) -> torch.Tensor:
+               out: torch.Tensor | None = None, any_cut: bool = True) -> torch.Tensor:
         """Temperature / nucleus draw per row with the reference's rules (tokens by falling logit, lower
         index first among equals; the shortest prefix reaching top_p; the uniform number walks its mass).
-        logits float32 [B, V]; temperature (> 0), top_p, uniform: float32 [B]; returns int32 [B]."""
+        logits float32 [B, V]; temperature (> 0), top_p, uniform: float32 [B]; returns int32 [B].
+        `any_cut=False` promises that no row has top_p < 1: the rounds that look for the nucleus's end are
+        then not launched."""
         _dev(logits, temperature, top_p, uniform, out)
         _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [B, V]")
         n_rows = logits.shape[0]
@@ -508,8 +510,11 @@ class Ops:
         if out is None:
             out = torch.empty(n_rows, dtype=torch.int32, device=logits.device)
         _need(out.dtype == torch.int32 and out.numel() == n_rows, "sample output must be int32 [B]")
+        workspace = torch.empty(max(1, n_rows) * self.lib.ta_sample_workspace_words(), dtype=torch.float32,
+                                device=logits.device)
         self._check(self.lib.ta_sample(_ptr(logits), _ptr(temperature), _ptr(top_p), _ptr(uniform), _ptr(out),
-                                       n_rows, logits.shape[1], self._stream()), "sample")
+                                       _ptr(workspace), n_rows, logits.shape[1], 1 if any_cut else 0, self._stream()),
+                    "sample")
         return out
 
 
