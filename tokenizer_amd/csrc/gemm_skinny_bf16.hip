@@ -60,18 +60,21 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     for (int mb = 0; mb < MB; ++mb) acc[s][mb] = (floatx4){0.f, 0.f, 0.f, 0.f};
 
   const int full_steps = K / 32;
-  // Four steps at a time, all loads first, so that many are in flight per lane.
+  // UN steps at a time, all loads first, so that many are in flight per lane.  A wave's last batch may reach
+  // past the end of K: such steps load nothing and multiply zeros (no matrix instruction sits behind a
+  // condition), so that a wave's share of K is as few trips to memory as can be, never one trip per step.
   constexpr int UN = (SETS * MB > 4) ? 2 : 4;
-  int ks = wave;
-  for (; ks + (UN - 1) * NW < full_steps; ks += UN * NW) {
+  for (int ks = wave; ks < full_steps; ks += UN * NW) {
     bf16x8 wf[UN][SETS], af[UN][MB];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int k = (ks + u * NW) * 32;
-      wf[u][0] = *reinterpret_cast<const bf16x8*>(w0 + k);
-      if (GATED) wf[u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + k);
+      const int step = ks + u * NW;
+      const bool valid = step < full_steps;
+      const int k = min(step, full_steps - 1) * 32;
+      wf[u][0] = load8(w0 + k, valid);
+      if (GATED) wf[u][SETS - 1] = load8(w1 + k, valid);
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) af[u][mb] = load8(a_row[mb] + k, a_ok[mb]);
+      for (int mb = 0; mb < MB; ++mb) af[u][mb] = load8(a_row[mb] + k, valid && a_ok[mb]);
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u)
@@ -80,19 +83,6 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 #pragma unroll
         for (int s = 0; s < SETS; ++s)
           acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][s], af[u][mb], acc[s][mb], 0, 0, 0);
-  }
-  for (; ks < full_steps; ks += NW) {
-    const int k = ks * 32;
-    bf16x8 wf[SETS];
-    wf[0] = *reinterpret_cast<const bf16x8*>(w0 + k);
-    if (GATED) wf[SETS - 1] = *reinterpret_cast<const bf16x8*>(w1 + k);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const bf16x8 af = load8(a_row[mb] + k, a_ok[mb]);
-#pragma unroll
-      for (int s = 0; s < SETS; ++s)
-        acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af, acc[s][mb], 0, 0, 0);
-    }
   }
   if (K & 31) {
     // The tail of K (a multiple of 8), zero-filled, is one wave's; the others multiply zeros, so that no matrix

@@ -190,9 +190,10 @@ class Engine:
         number per row (from the request's own generator)."""
         device = logits.device
         picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=device)]
-        as_tensor = lambda values: torch.tensor(values, dtype=torch.float32, device=device)
-        ids = self.model.runtime.ops.sample(picked.contiguous(), as_tensor(temperature), as_tensor(top_p),
-                                            as_tensor(uniform), any_cut=any(p < 1.0 for p in top_p))
+        # One copy to the device for the three vectors.
+        packed = torch.tensor([temperature, top_p, uniform], dtype=torch.float32).to(device, non_blocking=True)
+        ids = self.model.runtime.ops.sample(picked.contiguous(), packed[0], packed[1], packed[2],
+                                            any_cut=any(p < 1.0 for p in top_p))
         return [int(v) for v in ids.cpu().tolist()]
 
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):
@@ -359,7 +360,7 @@ class Engine:
                 raise KeyError(f"request {entry.rid!r} is not live")
             if not entry.tokens:
                 raise ValueError(f"request {entry.rid!r} brings no tokens")
-            if any((not 0 <= int(t) < vocab) for t in entry.tokens):
+            if not (0 <= min(entry.tokens) and max(entry.tokens) < vocab):
                 raise ValueError(f"request {entry.rid!r} has a token id outside 0..{vocab - 1}")
             end = self.cache.seq_len(entry.rid) + len(entry.tokens)
             if end > limit:
