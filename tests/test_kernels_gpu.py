@@ -318,6 +318,7 @@ def test_linear_with_k_cut_over_workgroups(ops, ref, shape, monkeypatch):
     """17 to 64 rows, a long K and few output tiles: the tiled kernel cuts K over workgroups and adds the parts
     in a fixed order; the result is the same product, the same on every run."""
     monkeypatch.setattr(ops, "SPLIT_K_FROM", 2048)
+    monkeypatch.setattr(ops, "split_k_kind", "tiled")
     m, n, k = shape
     assert ops._k_splits(m, n, k) > 1
     x = rand((m, k), torch.bfloat16, 24)
@@ -330,6 +331,23 @@ def test_linear_with_k_cut_over_workgroups(ops, ref, shape, monkeypatch):
             torch.testing.assert_close(got.double(), want, **linear_tol(out_dtype, x, w))
             again = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
             assert torch.equal(got, again)
+
+
+@pytest.mark.parametrize("shape", [(40, 200, 2304), (64, 96, 4864), (17, 1028, 2048), (33, 64, 2056), (20, 52, 4104)])
+def test_linear_with_k_cut_over_streaming_workgroups(ops, ref, shape):
+    """The same for the weight-streaming kernel (K of 2,048 up to 8,192): parts that are no multiple of 32 long in
+    all, a last part with a tail of K, output columns that do not fill the last tile of sixteen."""
+    m, n, k = shape
+    assert ops._streaming_splits(m, n, k) > 1
+    x = rand((m, k), torch.bfloat16, 24)
+    w = rand((n, k), torch.bfloat16, 25, 0.1)
+    bias = rand((n,), torch.float32, 26)
+    for use_bias in (True, False):
+        for out_dtype in (torch.bfloat16, torch.float32):
+            got = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
+            want = ref.linear(x, w, bias if use_bias else None, out_dtype=torch.float64)
+            torch.testing.assert_close(got.double(), want, **linear_tol(out_dtype, x, w))
+            assert torch.equal(got, ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype))
 
 
 @pytest.mark.parametrize("shape", [(17, 1152, 896), (64, 896, 4864), (200, 264, 136), (2048, 1152, 896)])

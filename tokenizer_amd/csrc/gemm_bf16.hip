@@ -2,13 +2,12 @@
 // (v_mfma_f32_32x32x16_bf16), output bfloat16 or float.  Tiles are staged through LDS; one block of
 // four waves owns a BM x BN tile of C, each wave a quarter of it.
 #include "common.h"
+#include "splitk_reduce.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 
-__device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
-__device__ __forceinline__ void store_out(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
 
 // BK: elements of K per step; rows in LDS are BK + 8 apart (padding against bank conflicts, still 16-byte aligned).
 //
@@ -131,24 +130,6 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, con
     }
 }
 
-// C[m, n] = sum over the slabs (in their order) + bias: four columns a thread (N is a multiple of 4 here).
-template <typename OutT>
-__global__ void splitk_reduce(const float* __restrict__ partial, const float* __restrict__ bias, OutT* __restrict__ C,
-                              int M, int N, int ldc, int splits) {
-  const size_t quad = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t per_row = N / 4;
-  if (quad >= (size_t)M * per_row) return;
-  const int m = (int)(quad / per_row), n = (int)(quad % per_row) * 4;
-  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int s = 0; s < splits; ++s) {
-    const float4 v = *reinterpret_cast<const float4*>(partial + ((size_t)s * M + m) * N + n);
-    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
-  }
-  if (bias) { sum.x += bias[n]; sum.y += bias[n + 1]; sum.z += bias[n + 2]; sum.w += bias[n + 3]; }
-  OutT* dst = C + (size_t)m * ldc + n;
-  store_out(dst, sum.x); store_out(dst + 1, sum.y); store_out(dst + 2, sum.z); store_out(dst + 3, sum.w);
-}
-
 template <int BM, int BN, int BK>
 static int launch(const void* A, const void* W, const void* bias, void* C, int M, int N, int K, int lda,
                   int ldc, int out_dtype, hipStream_t stream, int splits = 1, void* partial = nullptr) {
@@ -163,15 +144,7 @@ static int launch(const void* A, const void* W, const void* bias, void* C, int M
     gemm_bf16_kernel<BM, BN, BK, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (const float*)bias,
                                                                (bf16_t*)C, M, N, K, lda, ldc, k_chunk, slabs);
   int status = LAUNCH_STATUS();
-  if (status == 0 && splits > 1) {
-    const size_t quads = (size_t)M * (N / 4);
-    const int blocks = (int)((quads + 255) / 256);
-    if (out_dtype == DT_F32)
-      splitk_reduce<float><<<blocks, 256, 0, stream>>>(slabs, (const float*)bias, (float*)C, M, N, ldc, splits);
-    else
-      splitk_reduce<bf16_t><<<blocks, 256, 0, stream>>>(slabs, (const float*)bias, (bf16_t*)C, M, N, ldc, splits);
-    status = LAUNCH_STATUS();
-  }
+  if (status == 0 && splits > 1) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
   return status;
 }
 

@@ -4,6 +4,7 @@
 // element is loaded once, 16 bytes per lane.  The waves of a workgroup split K between them and add up
 // through LDS.  With GATED the kernel computes silu(A Wg^T) * (A Wu^T) for W = [Wg; Wu] in one pass.
 #include "common.h"
+#include "splitk_reduce.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -29,10 +30,14 @@ __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store1(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
 
 // grid.x: tiles of 16 output columns (of N, or of N/2 with GATED).  NW waves per workgroup.
+// grid.y: parts of K of `k_chunk` elements (a multiple of 32) each: with more than one, a workgroup writes the
+// float sums of its part into its slab of `partial` [parts, M, N] and `splitk_reduce` finishes the product.  That is
+// for few output tiles and a long K (the down projection of a decode batch): every compute unit gets a share.
 template <int MB, int NW, bool GATED, typename OutT>
 __global__ void __launch_bounds__(NW * WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
-                   const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K) {
+                   const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K_all,
+                   int k_chunk, float* __restrict__ partial) {
   constexpr int SETS = GATED ? 2 : 1;
   __shared__ float red[NW][SETS * MB * 4][WAVE];
   const int lane = threadIdx.x & 63, wave = wave_index();
@@ -41,8 +46,10 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int n0 = blockIdx.x * 16;
   // Rows past the end are clamped, not masked: they only feed outputs that are never stored.
   const int wrow = min(n0 + col, n_out - 1);
-  const bf16_t* w0 = W + (size_t)wrow * K + 8 * g;
-  const bf16_t* w1 = W + (size_t)(wrow + n_out) * K + 8 * g;     // the `up` rows when GATED
+  const int k_lo = blockIdx.y * k_chunk;
+  const int K = min(K_all, k_lo + k_chunk) - k_lo;                // this workgroup's part of K
+  const bf16_t* w0 = W + (size_t)wrow * K_all + k_lo + 8 * g;
+  const bf16_t* w1 = W + (size_t)(wrow + n_out) * K_all + k_lo + 8 * g;     // the `up` rows when GATED
   // Lanes of activation rows past M load nothing and hold zeros: a load costs the memory pipeline by its
   // active lanes, and with few rows most of a block's lanes are such.
   const bf16_t* a_row[MB];
@@ -50,7 +57,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     a_ok[mb] = mb * 16 + col < M;
-    a_row[mb] = A + (size_t)min(mb * 16 + col, M - 1) * lda + 8 * g;
+    a_row[mb] = A + (size_t)min(mb * 16 + col, M - 1) * lda + k_lo + 8 * g;
   }
 
   floatx4 acc[SETS][MB];
@@ -121,8 +128,12 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         sum0 += red[w][mb * 4 + r][ln];
         if (GATED) sum1 += red[w][(MB + mb) * 4 + r][ln];
       }
-      if (bias && n + r < n_out) sum0 += bias[n + r];
+      if (bias && !partial && n + r < n_out) sum0 += bias[n + r];
       v[r] = GATED ? sum0 / (1.0f + __expf(-sum0)) * sum1 : sum0;
+    }
+    if (partial) {                                              // (never GATED; N is a multiple of 4)
+      store4(partial + ((size_t)blockIdx.y * M + m) * n_out + n, v);
+      continue;
     }
     OutT* dst = C + (size_t)m * ldc + n;
     if (n + 3 < n_out && (ldc & 3) == 0) {
@@ -137,16 +148,21 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 
 template <int MB, int NW, bool GATED>
 static int launch_skinny(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
-                         int K, int out_dtype, hipStream_t stream) {
+                         int K, int out_dtype, hipStream_t stream, int splits = 1, void* partial = nullptr) {
   const int n_out = GATED ? N / 2 : N;
-  const int tiles = (n_out + 15) / 16;
+  const int k_chunk = splits > 1 ? ((K + splits - 1) / splits + 31) / 32 * 32 : K;
+  if (splits > 1) splits = (K + k_chunk - 1) / k_chunk;          // no part without a step of its own
+  const dim3 grid((n_out + 15) / 16, splits);
+  float* slabs = splits > 1 ? (float*)partial : nullptr;
   if (out_dtype == DT_F32)
-    skinny_gemm_kernel<MB, NW, GATED, float><<<tiles, NW * WAVE, 0, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (float*)C, ldc, M, N, K);
+    skinny_gemm_kernel<MB, NW, GATED, float><<<grid, NW * WAVE, 0, stream>>>(
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (float*)C, ldc, M, N, K, k_chunk, slabs);
   else
-    skinny_gemm_kernel<MB, NW, GATED, bf16_t><<<tiles, NW * WAVE, 0, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)C, ldc, M, N, K);
-  return LAUNCH_STATUS();
+    skinny_gemm_kernel<MB, NW, GATED, bf16_t><<<grid, NW * WAVE, 0, stream>>>(
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)C, ldc, M, N, K, k_chunk, slabs);
+  int status = LAUNCH_STATUS();
+  if (status == 0 && splits > 1) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
+  return status;
 }
 
 template <int MB, bool GATED>
@@ -171,6 +187,24 @@ extern "C" int ta_gemm_skinny_bf16(const void* A, int lda, const void* W, const 
 #define GO(MBV) (gated ? pick_waves<MBV, true>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream) \
                        : pick_waves<MBV, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream))
   switch (mb) {
+    case 1: return GO(1);
+    case 2: return GO(2);
+    case 3: return GO(3);
+    default: return GO(4);
+  }
+#undef GO
+}
+
+// The same product (not gated) with K cut into `splits` parts (at most; parts are multiples of 32) over the
+// workgroups, the parts' float sums added afterwards in a fixed order.  partial: room for splits * M * N floats;
+// N % 4 == 0; M <= 64.
+extern "C" int ta_gemm_skinny_bf16_splitk(const void* A, int lda, const void* W, const void* bias, void* C, int ldc,
+                                          void* partial, int M, int N, int K, int out_dtype, int splits,
+                                          hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || (K & 7) || (lda & 7) || (N & 3) || splits < 1 || (splits > 1 && !partial)) return -1;
+#define GO(MBV) launch_skinny<MBV, 8, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, splits, partial)
+  switch ((M + 15) / 16) {
     case 1: return GO(1);
     case 2: return GO(2);
     case 3: return GO(3);

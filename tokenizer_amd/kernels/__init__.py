@@ -56,7 +56,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_gemm_skinny_bf16_splitk", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_argmax", "ta_sample", "ta_sample_workspace_words", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
@@ -293,10 +293,19 @@ class Ops:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+            streaming_splits = self._streaming_splits(m, n, k)
+            if streaming_splits > 1 and self.split_k_kind == "streaming":
+                # 17 to 64 rows, a long K and few output columns (the down projection of a decode batch): the
+                # weight-streaming kernel with K cut over workgroups, so that every compute unit streams a share
+                # of the weights; the parts are added in a fixed order by a second small kernel.
+                partial = torch.empty((streaming_splits, m, n), dtype=torch.float32, device=x.device)
+                self._check(self.lib.ta_gemm_skinny_bf16_splitk(
+                    _ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, _ptr(partial), m, n, k, _code(out_dtype),
+                    streaming_splits, self._stream()), "linear")
+                return out
             splits = self._k_splits(m, n, k)
             if splits > 1:
-                # Few rows and a very long K (the down projection of a decode batch in a wide model): K is cut
-                # over workgroups so that every compute unit streams a share of the weights.
+                # The same with the tiled kernel.
                 partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
                 self._check(self.lib.ta_gemm_bf16_splitk(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(partial),
                                                          m, n, k, lda, n, _code(out_dtype), splits, self._stream()),
@@ -345,7 +354,24 @@ class Ops:
             return 1
         return max(1, min(-(-512 // tiles), k // 256))
 
-    SPLIT_K_FROM = 8192        # the shortest K that is cut (shorter ones are the library's, or the weight-streaming kernel's)
+    split_k_kind = "streaming"     # which kernel cuts K for 17 to 64 rows ("tiled": only the tiled one)
+
+    def _streaming_splits(self, m: int, n: int, k: int) -> int:
+        """Into how many parts the weight-streaming kernel cuts K for 17 to 64 rows and a K of 2,048 up to where
+        the tiled kernel takes over: so many that its tiles of sixteen output columns times the parts give every
+        compute unit a workgroup, each part at least 512 long.  (Measured with cold weights for the down
+        projections of the 0.5B to 7B models: one of the two beats the library at every row count from 17 to 64,
+        the streaming kernel while a part is a few steps per wave, the tiled one, which reads the rows a quarter
+        as often, for longer K.)"""
+        if (not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or n % 4
+                or not (2048 <= k < self.SPLIT_K_FROM)):
+            return 1
+        tiles = -(-n // 16)
+        if tiles >= 128:
+            return 1
+        return max(1, min(-(-256 // tiles), k // 512))
+
+    SPLIT_K_FROM = 8192        # the shortest K that the tiled kernel cuts (shorter ones are the weight-streaming kernel's)
 
     EAGER_LIBRARY_WORK = 2 ** 30   # multiply-adds from which a product launched eagerly goes to the library
     capturing = False          # set while a graph is recorded (and in the run that warms it up): launches are free then
