@@ -321,8 +321,8 @@ class Ops:
                 # device's own clock (launches recorded in a graph, weights cold) it is ahead of the tiled
                 # kernel of this package for nearly every shape of the 0.5B to 7B models.  So do products of 17
                 # to 64 rows with a big weight matrix (every tile of the weight-streaming kernel reads all the
-                # rows again, which costs more than the weights once there are more than sixteen of them) or
-                # with a long K and few output columns (too few tiles; the library cuts K).  The float32 bias
+                # rows again, which costs more than the weights once there are more than sixteen of them), and
+                # those with a long K and few output columns that the kernels above did not take.  The float32 bias
                 # joins the library's float accumulator as it joins the kernels' own.  A launch of the library
                 # costs the host some 15 us against 4 us for a kernel of this package: outside graph capture,
                 # products of more than 64 rows that are over on the device in about that time stay with the
