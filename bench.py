@@ -94,7 +94,9 @@ def run_decode(model, batch: int, steps: int, warmup: int):
     last = []
     for rid, prompt in enumerate(prompts):
         engine.add_request(rid)
-        logits = engine.step([StepEntry(rid, prompt, [len(prompt) - 1])])
+        for at in range(0, len(prompt), 2048):                  # long prompts in portions
+            portion = prompt[at:at + 2048]
+            logits = engine.step([StepEntry(rid, portion, [len(portion) - 1] if at + 2048 >= len(prompt) else [])])
         last.append(engine.argmax(logits)[0])
 
     # Greedy decode steps back to back: each step's ids feed the next on the device and reach the host one
@@ -238,7 +240,14 @@ def main() -> int:
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
+    parser.add_argument("--prompt-len", type=int, default=None,
+                        help="tokens of every prompt before decoding (default 2,048, the record's; the context the "
+                             "record names is then twice that, else the prompt plus the decoded tokens)")
     args = parser.parse_args()
+    if args.prompt_len:
+        global PROMPT_LEN, CONTEXT_LEN
+        PROMPT_LEN = args.prompt_len
+        CONTEXT_LEN = -(-(args.prompt_len + args.warmup + max(args.steps, 64) + 1) // 16) * 16
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; runs with --gpus > 1 are not supported")
         return 2
