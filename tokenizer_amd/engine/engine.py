@@ -63,7 +63,7 @@ def random_model(config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:
     return Model(config, tensors, dtype, device, ops)
 
 
-class DecodeGraph:
+class StepGraph:
     """One captured HIP graph of a step of one shape: so many entries with so many tokens and wanted places
     each (a decode step: one token each), contexts of up to `bucket` tokens.  The batch's tables live in
     fixed buffers that are refilled before every replay; the graph ends with the greedy pick, so ids are
@@ -161,14 +161,14 @@ class Engine:
                                                 v_pages=v_pages, state=self.pools.states.get(source),
                                                 writes=entry.cache_of is None))
         self.steps = 0
-        # Decode steps (one token per request, its logits wanted) replay a captured graph; the logits of a
-        # step stay valid until the next step.
+        # Decode steps (one token per request, its logits wanted) and other steps whose shape recurs replay a
+        # captured graph; the logits of a step stay valid until the next step.
         self.use_graphs = (model.device.type == "cuda") if use_graphs is None else use_graphs
         self.use_graphs = self.use_graphs and model.decoder.graph_safe
-        self.graphs: dict[tuple, DecodeGraph] = {}
+        self.graphs: dict[tuple, StepGraph] = {}
         self._shapes_seen: dict[tuple, int] = {}
         self.graph_pool = torch.cuda.graph_pool_handle() if self.use_graphs else None
-        self._graph_result: DecodeGraph | None = None
+        self._graph_result: StepGraph | None = None
 
     @property
     def max_positions(self) -> int:
@@ -225,7 +225,7 @@ class Engine:
         landing = [torch.empty(count, dtype=torch.int32).pin_memory() for _ in range(2)]
         arrived = [torch.cuda.Event(), torch.cuda.Event()]
         picked: list[list[int]] = []
-        previous: DecodeGraph | None = None
+        previous: StepGraph | None = None
         go_on = True
         for k in range(n_steps):
             # Only the first step's token ids are known here; later steps take theirs from the step before.
@@ -269,11 +269,11 @@ class Engine:
         bucket = -(-bucket // self.cache.page_size) * self.cache.page_size
         return (self._shape_of(entries), bucket)
 
-    def _graph_for(self, entries: list[StepEntry]) -> "DecodeGraph":
+    def _graph_for(self, entries: list[StepEntry]) -> "StepGraph":
         key = self._graph_key(entries)
         graph = self.graphs.get(key)
         if graph is None:
-            graph = DecodeGraph(self, entries, key[1])       # its first eager run and the capture write the same
+            graph = StepGraph(self, entries, key[1])       # its first eager run and the capture write the same
             self.graphs[key] = graph                         # keys and values the replay writes again
         graph.last_used = self.steps
         return graph
