@@ -110,6 +110,9 @@ class PlainOps:
     def can_fuse_decode(self, rows, dtype, hidden=0):
         return 0 < rows <= self.fuse_rows
 
+    def can_rope_store(self, rows, dtype):
+        return self.fuse_rows < rows <= 64
+
     def fold_norm(self, hidden):
         return hidden <= 80          # so that the CPU tests of the engine take both routes
 

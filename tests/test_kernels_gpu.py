@@ -425,8 +425,10 @@ def test_skinny_rows_agree_with_the_tiled_kernel(ops, shape):
 
 @pytest.mark.parametrize("geometry", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 16), (4, 4, 128, 520, 32), (20, 2, 96, 264, 16),
                                       (2, 1, 64, 1280, 16), (4, 2, 32, 2304, 16)])
-@pytest.mark.parametrize("rows", [1, 8, 16])
+@pytest.mark.parametrize("rows", [1, 8, 16, 17, 40, 64])
 def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
+    # Up to 16 rows: the fused decode kernel, from the residual or from normalised rows; 17 to 64 rows: the
+    # weight-streaming kernel with the same epilogue, from normalised rows.
     n_q, n_kv, d, hidden, page_size = geometry
     n_pages, max_pos = 7, 300
     gen = torch.Generator().manual_seed(40)
@@ -447,16 +449,17 @@ def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
         kb, vb = ka.clone(), va.clone()
         args = (residual, norm_w, 1e-6, w, bias if use_bias else None, positions, table, slots if store else None)
         before = residual.clone()
-        qa = ops.fused_norm_qkv_rope(*args, ka, va, n_q, n_kv, d)
         qb = ref.fused_norm_qkv_rope(*args, kb, vb, n_q, n_kv, d)
-        assert torch.equal(residual, before)
         # The norm's output is rounded to bfloat16 in both; what differs is the summation order.
         tolerance = dict(rtol=2e-2, atol=2e-2)
-        torch.testing.assert_close(qa.float(), qb.float(), **tolerance)
-        torch.testing.assert_close(ka.float(), kb.float(), **tolerance)
-        torch.testing.assert_close(va.float(), vb.float(), **tolerance)
-        if not store:
-            assert float(ka.abs().max()) == 0 and float(va.abs().max()) == 0
+        if rows <= 16:
+            qa = ops.fused_norm_qkv_rope(*args, ka, va, n_q, n_kv, d)
+            assert torch.equal(residual, before)
+            torch.testing.assert_close(qa.float(), qb.float(), **tolerance)
+            torch.testing.assert_close(ka.float(), kb.float(), **tolerance)
+            torch.testing.assert_close(va.float(), vb.float(), **tolerance)
+            if not store:
+                assert float(ka.abs().max()) == 0 and float(va.abs().max()) == 0
         # The same from rows that are normalised already (the route of wide models): rows of a wider buffer.
         wide = torch.zeros((rows, hidden + 8), dtype=torch.bfloat16).cuda()
         normed = wide[:, :hidden]
@@ -467,6 +470,8 @@ def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
         torch.testing.assert_close(qc.float(), qb.float(), **tolerance)
         torch.testing.assert_close(kc.float(), kb.float(), **tolerance)
         torch.testing.assert_close(vc.float(), vb.float(), **tolerance)
+        if not store:
+            assert float(kc.abs().max()) == 0 and float(vc.abs().max()) == 0
 
 
 # The last shapes: rows of 1,280 and 2,304 elements give the waves unequal shares of K in the kernels that ask for

@@ -33,23 +33,40 @@ __device__ __forceinline__ void store1(bf16_t* p, float v) { p->bits = float_to_
 // grid.y: parts of K of `k_chunk` elements (a multiple of 32) each: with more than one, a workgroup writes the
 // float sums of its part into its slab of `partial` [parts, M, N] and `splitk_reduce` finishes the product.  That is
 // for few output tiles and a long K (the down projection of a decode batch): every compute unit gets a share.
-template <int MB, int NW, bool GATED, typename OutT>
+//
+// ROPE (with GATED's two sets of weight rows): the product is the joined q/k/v projection.  A tile is sixteen
+// elements of the first half of a head and the sixteen half a head further on, which the half-split rotation
+// pairs; the epilogue adds the bias, rotates query and key heads by the row's position and writes queries to
+// C [M, n_q * d], keys and values into their pages (values transposed inside a page).
+struct RopeStore {
+  const int* positions; const float* cos_sin; const int* slots;
+  bf16_t* k_pages; bf16_t* v_pages;
+  int n_q, n_kv, d, page_size;
+};
+
+template <int MB, int NW, bool GATED, typename OutT, bool ROPE = false>
 __global__ void __launch_bounds__(NW * WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
                    const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K_all,
-                   int k_chunk, float* __restrict__ partial) {
+                   int k_chunk, float* __restrict__ partial, const RopeStore rope = RopeStore()) {
+  static_assert(!ROPE || GATED, "the rotation uses the two sets of weight rows");
   constexpr int SETS = GATED ? 2 : 1;
   __shared__ float red[NW][SETS * MB * 4][WAVE];
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
-  const int n_out = GATED ? N / 2 : N;
-  const int n0 = blockIdx.x * 16;
+  const int n_out = ROPE ? N : GATED ? N / 2 : N;
+  // ROPE: tile t is block t % (d/32) of sixteen elements in the first half of head t / (d/32).
+  const int rope_half = ROPE ? rope.d / 2 : 0;
+  const int rope_head = ROPE ? blockIdx.x / (rope_half / 16) : 0;
+  const int rope_first = ROPE ? (blockIdx.x % (rope_half / 16)) * 16 : 0;      // first element of the tile in its head
+  const int n0 = ROPE ? rope_head * rope.d + rope_first : blockIdx.x * 16;
   // Rows past the end are clamped, not masked: they only feed outputs that are never stored.
   const int wrow = min(n0 + col, n_out - 1);
   const int k_lo = blockIdx.y * k_chunk;
   const int K = min(K_all, k_lo + k_chunk) - k_lo;                // this workgroup's part of K
   const bf16_t* w0 = W + (size_t)wrow * K_all + k_lo + 8 * g;
-  const bf16_t* w1 = W + (size_t)(wrow + n_out) * K_all + k_lo + 8 * g;     // the `up` rows when GATED
+  // The second set: the `up` rows when GATED, the rows half a head further on with ROPE.
+  const bf16_t* w1 = W + (size_t)(wrow + (ROPE ? rope_half : n_out)) * K_all + k_lo + 8 * g;
   // Lanes of activation rows past M load nothing and hold zeros: a load costs the memory pipeline by its
   // active lanes, and with few rows most of a block's lanes are such.
   const bf16_t* a_row[MB];
@@ -119,7 +136,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     const int m = mb * 16 + (ln & 15);
     const int n = n0 + 4 * (ln >> 4);
     if (m >= M || n >= n_out) continue;
-    float v[4];
+    float v[4], v2[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float sum0 = 0.f, sum1 = 0.f;
@@ -128,8 +145,47 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         sum0 += red[w][mb * 4 + r][ln];
         if (GATED) sum1 += red[w][(MB + mb) * 4 + r][ln];
       }
+      if (ROPE) {
+        v[r] = sum0 + (bias ? bias[n + r] : 0.f);
+        v2[r] = sum1 + (bias ? bias[n + rope_half + r] : 0.f);
+        continue;
+      }
       if (bias && !partial && n + r < n_out) sum0 += bias[n + r];
       v[r] = GATED ? sum0 / (1.0f + __expf(-sum0)) * sum1 : sum0;
+    }
+    if constexpr (ROPE) {
+      const int d = rope.d, i = rope_first + 4 * (ln >> 4);          // elements i..i+3 of the head, and i + half
+      if (rope_head < rope.n_q + rope.n_kv && rope.cos_sin) {
+        const float* cs = rope.cos_sin + (size_t)rope.positions[m] * d;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float c = cs[i + r], sn = cs[rope_half + i + r], x1 = v[r], x2 = v2[r];
+          v[r] = x1 * c - x2 * sn;
+          v2[r] = x2 * c + x1 * sn;
+        }
+      }
+      if (rope_head < rope.n_q) {
+        bf16_t* dst = reinterpret_cast<bf16_t*>(C) + (size_t)m * ldc + (size_t)rope_head * d + i;
+        store4(dst, v);
+        store4(dst + rope_half, v2);
+        continue;
+      }
+      const int slot = rope.slots ? rope.slots[m] : -1;
+      if (slot < 0) continue;                                     // this row's keys and values are not stored
+      const int page = slot / rope.page_size, off = slot % rope.page_size;
+      if (rope_head < rope.n_q + rope.n_kv) {
+        bf16_t* dst = rope.k_pages + (((size_t)page * rope.n_kv + (rope_head - rope.n_q)) * rope.page_size + off) * d + i;
+        store4(dst, v);
+        store4(dst + rope_half, v2);
+      } else {
+        bf16_t* dst = rope.v_pages + (((size_t)page * rope.n_kv + (rope_head - rope.n_q - rope.n_kv)) * d + i) * rope.page_size + off;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          store1(dst + (size_t)r * rope.page_size, v[r]);
+          store1(dst + (size_t)(rope_half + r) * rope.page_size, v2[r]);
+        }
+      }
+      continue;
     }
     if (partial) {                                              // (never GATED; N is a multiple of 4)
       store4(partial + ((size_t)blockIdx.y * M + m) * n_out + n, v);
@@ -211,4 +267,33 @@ extern "C" int ta_gemm_skinny_bf16_splitk(const void* A, int lda, const void* W,
     default: return GO(4);
   }
 #undef GO
+}
+
+// The joined q/k/v projection of 17 to 64 rows with bias, rotation and the cache write in its epilogue (see
+// RopeStore): x bfloat16 [M, K] (row stride lda), W [(n_q + 2 n_kv) d, K], bias float32 or null; queries go to
+// q_out [M, n_q d]; cos_sin float32 [positions, d] or null (no rotation); slots int32 [M] or null (nothing is
+// stored; a negative slot skips its row).  d a multiple of 32.
+extern "C" int ta_gemm_skinny_qkv_rope(const void* x, int lda, const void* W, const void* bias, void* q_out,
+                                       const void* positions, const void* cos_sin, const void* slots, void* k_pages,
+                                       void* v_pages, int M, int K, int n_q, int n_kv, int d, int page_size,
+                                       hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (M > 64 || (K & 7) || (lda & 7) || (d & 31) || n_q <= 0 || n_kv <= 0 || page_size <= 0 || !positions) return -1;
+  if (slots && (!k_pages || !v_pages)) return -1;
+  RopeStore rope;
+  rope.positions = (const int*)positions; rope.cos_sin = (const float*)cos_sin; rope.slots = (const int*)slots;
+  rope.k_pages = (bf16_t*)k_pages; rope.v_pages = (bf16_t*)v_pages;
+  rope.n_q = n_q; rope.n_kv = n_kv; rope.d = d; rope.page_size = page_size;
+  const int N = (n_q + 2 * n_kv) * d;
+  const dim3 grid((n_q + 2 * n_kv) * (d / 32), 1);
+#define GO(MBV) skinny_gemm_kernel<MBV, 8, true, bf16_t, true><<<grid, 8 * WAVE, 0, stream>>>( \
+    (const bf16_t*)x, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)q_out, n_q * d, M, N, K, K, nullptr, rope)
+  switch ((M + 15) / 16) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 3: GO(3); break;
+    default: GO(4); break;
+  }
+#undef GO
+  return LAUNCH_STATUS();
 }

@@ -56,7 +56,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_gemm_skinny_bf16_splitk", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_argmax", "ta_sample", "ta_sample_workspace_words", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
@@ -444,7 +444,9 @@ class Ops:
                   and norm_weight.numel() == k, "the residual and the norm weight are float32")
         _need(weight.dtype == torch.bfloat16 and tuple(weight.shape) == ((n_q + 2 * n_kv) * head_dim, k),
               "the joined q/k/v matrix has the wrong shape")
-        _need(m <= self.FUSED_ROWS and k % 8 == 0 and head_dim % 32 == 0, "sizes the fused projection does not take")
+        _need(k % 8 == 0 and head_dim % 32 == 0
+              and (m <= self.FUSED_ROWS or (norm_weight is None and m <= self.SKINNY_ROWS)),
+              "sizes the fused projection does not take")
         _need(positions.dtype == torch.int32 and positions.numel() == m, "positions must be int32 [M]")
         if bias is not None:
             _need(bias.dtype == torch.float32 and bias.numel() == weight.shape[0], "bias must be float32")
@@ -459,12 +461,20 @@ class Ops:
         tail = (_ptr(weight), _ptr(bias), _ptr(q), _ptr(positions), _ptr(cos_sin), _ptr(slots),
                 _ptr(k_pages if slots is not None else None), _ptr(v_pages if slots is not None else None),
                 m, k, n_q, n_kv, head_dim, page_size, self.fused_rows, self.fused_waves, self._stream())
-        if norm_weight is None:
+        if m > self.FUSED_ROWS:
+            # 17 to 64 rows: the weight-streaming kernel with the same epilogue.
+            status = self.lib.ta_gemm_skinny_qkv_rope(_ptr(residual), residual.stride(0), *tail[:-3], self._stream())
+        elif norm_weight is None:
             status = self.lib.ta_fused_qkv_rope(_ptr(residual), residual.stride(0) if m > 1 else k, *tail)
         else:
             status = self.lib.ta_fused_norm_qkv_rope(_ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), *tail)
         self._check(status, "fused_norm_qkv_rope")
         return q
+
+    def can_rope_store(self, rows: int, dtype: torch.dtype) -> bool:
+        """Whether `fused_norm_qkv_rope` takes this many normalised bfloat16 rows (17 to 64 go through the
+        weight-streaming kernel, which then needs no rotation kernel after it)."""
+        return self.use_fused_decode and dtype == torch.bfloat16 and self.FUSED_ROWS < rows <= self.SKINNY_ROWS
 
     def fused_norm_gated(self, residual, norm_weight, eps, weight) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with x = rmsnorm(residual), weight = [Wg; Wu]; bfloat16 [M, I].  With

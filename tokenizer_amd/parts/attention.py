@@ -86,8 +86,16 @@ class GQAttention(Mixer):
 
     def forward(self, x, ctx, cache):
         ops = self.runtime.ops
-        qkv = ops.linear(x, self.w_qkv, self.b_qkv)   # bias joins the float accumulator
-        self.position.encode_and_store(qkv, None, self.n_q, self.n_kv, self.d, ctx, cache)
+        can = getattr(ops, "can_rope_store", None)
+        if (can and can(x.shape[0], self.runtime.dtype) and type(self.position) in (NoPosition, RotaryHalfSplit)
+                and self.d % 32 == 0 and cache.group is not None):
+            # A few dozen rows: bias, rotation and the cache write ride in the projection's epilogue.
+            qkv = ops.fused_norm_qkv_rope(x, None, 0.0, self.w_qkv, self.b_qkv, ctx.positions, self.position.table(),
+                                          ctx.slots[cache.group] if cache.writes else None, cache.k_pages,
+                                          cache.v_pages, self.n_q, self.n_kv, self.d)
+        else:
+            qkv = ops.linear(x, self.w_qkv, self.b_qkv)   # bias joins the float accumulator
+            self.position.encode_and_store(qkv, None, self.n_q, self.n_kv, self.d, ctx, cache)
         mixed = torch.empty((x.shape[0], self.n_q * self.d), dtype=x.dtype, device=x.device)
         ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
                             ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
