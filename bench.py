@@ -138,7 +138,7 @@ def run_prefill(model, repeats: int = 3):
     return best
 
 
-def run_workload(name: str, layers: int | None, dtype: str) -> dict:
+def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0) -> dict:
     """A serving workload through the scheduler: every request is admitted, its prompt cut into portions under
     the token budget beside the others' decode tokens, decoded greedily to its length, and freed."""
     import numpy as np
@@ -169,10 +169,12 @@ def run_workload(name: str, layers: int | None, dtype: str) -> dict:
                                                   prefix_cache=prefix_cache, max_num_batched_tokens=2048))
         torch.cuda.synchronize()
         started = time.perf_counter()
-        ids = [sched.add_request(prompts[0], GenerateParams.greedy(new_tokens))]
+        params = lambda i: (GenerateParams.greedy(new_tokens) if temperature == 0 else
+                            GenerateParams(max_tokens=new_tokens, temperature=temperature, top_p=0.95, seed=i))
+        ids = [sched.add_request(prompts[0], params(0))]
         if prefix_cache:
             sched.step()                         # the first request's prompt is in the cache when the others arrive
-        ids += [sched.add_request(p, GenerateParams.greedy(new_tokens)) for p in prompts[1:]]
+        ids += [sched.add_request(p, params(i + 1)) for i, p in enumerate(prompts[1:])]
         results = sched.run()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
@@ -190,7 +192,7 @@ def run_workload(name: str, layers: int | None, dtype: str) -> dict:
                        "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                        "requests": len(prompts), "prompt_tokens": sum(len(p) for p in prompts),
                        "new_tokens_each": new_tokens, "token_budget": 2048, "prefix_cache": prefix_cache,
-                       "pages": pages, "page_size": 16},
+                       "pages": pages, "page_size": 16, "temperature": temperature},
             "scheduler": {"steps": stats.steps, "tokens_forwarded": stats.tokens_forwarded, "max_running": stats.max_running,
                           "preemptions": stats.preemptions, "peak_pages": stats.peak_blocks,
                           "forwarded_tokens_per_s": round(stats.tokens_forwarded / elapsed, 1)}}
@@ -240,6 +242,8 @@ def main() -> int:
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
+    parser.add_argument("--temperature", type=float, default=0.0,
+                        help="with --workload: draw with this temperature and top_p 0.95 instead of greedy picks")
     parser.add_argument("--prompt-len", type=int, default=None,
                         help="tokens of every prompt before decoding (default 2,048, the record's; the context the "
                              "record names is then twice that, else the prompt plus the decoded tokens)")
@@ -256,7 +260,7 @@ def main() -> int:
         print(json.dumps(measure_peaks()), flush=True)
         return 0
     if args.workload:
-        print(json.dumps(run_workload(args.workload, args.layers, args.dtype)), flush=True)
+        print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature)), flush=True)
         return 0
     sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
     full_layers = sizes["num_hidden_layers"]
