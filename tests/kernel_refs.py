@@ -110,7 +110,7 @@ class PlainOps:
     def can_fuse_decode(self, rows, dtype, hidden=0):
         return 0 < rows <= self.fuse_rows
 
-    def can_rope_store(self, rows, dtype):
+    def can_rope_store(self, rows, dtype, weight_elements=0):
         return self.fuse_rows < rows <= 64
 
     def fold_norm(self, hidden):

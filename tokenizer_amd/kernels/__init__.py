@@ -471,10 +471,15 @@ class Ops:
         self._check(status, "fused_norm_qkv_rope")
         return q
 
-    def can_rope_store(self, rows: int, dtype: torch.dtype) -> bool:
-        """Whether `fused_norm_qkv_rope` takes this many normalised bfloat16 rows (17 to 64 go through the
-        weight-streaming kernel, which then needs no rotation kernel after it)."""
-        return self.use_fused_decode and dtype == torch.bfloat16 and self.FUSED_ROWS < rows <= self.SKINNY_ROWS
+    ROPE_STORE_WEIGHT = 2 ** 22   # joined q/k/v matrices up to this many elements take the route below at 17-64 rows
+
+    def can_rope_store(self, rows: int, dtype: torch.dtype, weight_elements: int = 0) -> bool:
+        """Whether `fused_norm_qkv_rope` should take this many normalised bfloat16 rows: 17 to 64 go through the
+        weight-streaming kernel, which then needs no rotation kernel after it.  That pays while the matrix is
+        small (measured: 0.5B and 1.5B sizes); a big one is better off with the library's product and the
+        rotation kernel."""
+        return (self.use_fused_decode and dtype == torch.bfloat16 and self.FUSED_ROWS < rows <= self.SKINNY_ROWS
+                and weight_elements <= self.ROPE_STORE_WEIGHT)
 
     def fused_norm_gated(self, residual, norm_weight, eps, weight) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with x = rmsnorm(residual), weight = [Wg; Wu]; bfloat16 [M, I].  With

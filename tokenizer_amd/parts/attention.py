@@ -87,7 +87,7 @@ class GQAttention(Mixer):
     def forward(self, x, ctx, cache):
         ops = self.runtime.ops
         can = getattr(ops, "can_rope_store", None)
-        if (can and can(x.shape[0], self.runtime.dtype) and type(self.position) in (NoPosition, RotaryHalfSplit)
+        if (can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and type(self.position) in (NoPosition, RotaryHalfSplit)
                 and self.d % 32 == 0 and cache.group is not None):
             # A few dozen rows: bias, rotation and the cache write ride in the projection's epilogue.
             qkv = ops.fused_norm_qkv_rope(x, None, 0.0, self.w_qkv, self.b_qkv, ctx.positions, self.position.table(),
