@@ -423,6 +423,31 @@ def test_warm_requests_draw_on_the_device_as_they_would_alone(model_folders):
     sched.assert_idle()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_draws_of_a_replayed_step_equal_eager_draws(model_folders, dtype):
+    # A batch in which every request draws with a temperature: its decode steps replay a captured graph, and the
+    # sampler's launches over that graph's logits replay one as well (with and without the nucleus rounds).  The
+    # tokens equal those of an engine that captures nothing, step after step.
+    from tokenizer_amd.engine import GenerateParams, Scheduler, SchedulerConfig
+    name = "B"
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [random_ids(vocab, n, 90 + n) for n in (6, 6, 6)]
+    for cuts in ((0.9, 0.5, 0.97), (1.0, 1.0, 1.0)):
+        params = [GenerateParams(max_tokens=14, temperature=t, top_p=p, seed=s)
+                  for t, p, s in zip((1.2, 0.8, 2.0), cuts, (3, 4, 5))]
+        tokens = {}
+        for use_graphs in (True, False):
+            eng = engine_for(model_folders[name], dtype, num_pages=32, max_requests=4, use_graphs=use_graphs)
+            sched = Scheduler(eng, SchedulerConfig(num_blocks=32, max_batch_size=4))
+            rids = [sched.add_request(p, q) for p, q in zip(prompts, params)]
+            results = sched.run()
+            tokens[use_graphs] = [results[rid].tokens for rid in rids]
+            if use_graphs:
+                assert any(graph.draws for graph in eng.graphs.values())
+        assert tokens[True] == tokens[False]
+        assert all(len(t) == 14 for t in tokens[True])
+
+
 REAL_SIZES = {
     # Layer sizes of the three model sizes the benchmarks name, cut to two layers and a small vocabulary.
     "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864),
@@ -460,3 +485,40 @@ def test_layers_of_real_sizes(tmp_path, size):
     logits = eng.step([StepEntry(rid, ids[-1:], [0]) for rid, ids in enumerate(prompts)]).float().cpu()
     for rid, ids in enumerate(prompts):
         close(logits[rid:rid + 1], plain.all_logits(cfg, tensors, ids)[-1:], "bfloat16")
+
+
+ODD_SIZES = {
+    # Sizes away from every tile: an inner width that is no multiple of eight, odd vocabularies, head sizes from
+    # 16 to 256, one to eighteen query heads per kv head, a model wider than the norm-folding kernels take.
+    "inner100": dict(num_hidden_layers=1, hidden_size=112, num_attention_heads=7, num_key_value_heads=7,
+                     intermediate_size=100, vocab_size=1001),
+    "inner300_mqa": dict(num_hidden_layers=2, hidden_size=144, num_attention_heads=3, num_key_value_heads=1,
+                         intermediate_size=300, vocab_size=517, tie_word_embeddings=False, rms_norm_eps=1e-5),
+    "group18": dict(num_hidden_layers=1, hidden_size=288, num_attention_heads=18, num_key_value_heads=1,
+                    intermediate_size=204, vocab_size=777),
+    "head256": dict(num_hidden_layers=1, hidden_size=256, num_attention_heads=1, num_key_value_heads=1,
+                    intermediate_size=36, vocab_size=99),
+    "wide": dict(num_hidden_layers=1, hidden_size=2304, num_attention_heads=18, num_key_value_heads=6,
+                 intermediate_size=1004, vocab_size=500),
+    "window_inner44": dict(num_hidden_layers=3, hidden_size=320, num_attention_heads=2, num_key_value_heads=2,
+                           intermediate_size=44, vocab_size=129, use_sliding_window=True, sliding_window=33,
+                           max_window_layers=1),
+}
+
+
+@pytest.mark.parametrize("size", list(ODD_SIZES))
+def test_sizes_away_from_every_tile(tmp_path, size):
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    raw = dict(TINY["A"][0], max_position_embeddings=512, **ODD_SIZES[size])
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 13, str(tmp_path / size))
+    cfg, tensors = plain.load_folder(folder)
+    reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 30 + i) for i, n in enumerate([70, 33, 100, 9])}
+    want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (tt.mixed(reqs, 6), tt.decode_tail(reqs, 32)):
+            eng = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=4)
+            eng.pools.poison()
+            got = tt.run_in_process(eng, steps)
+            for rid in reqs:
+                close(got[rid], want[rid], dtype)

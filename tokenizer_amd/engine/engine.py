@@ -100,6 +100,34 @@ class StepGraph:
             ops.capturing = before
         self.uploaded = None
         self.last_used = 0
+        self.draws = None                           # captured graphs of the sampler over these logits, made on demand
+
+    def draw(self, engine: "Engine", temperature: list[float], top_p: list[float], uniform: list[float],
+             any_cut: bool) -> list[int]:
+        """Temperature / nucleus draws for every row of this graph's logits: the sampler's twenty small launches
+        are captured once (per kind: with or without the rounds of the nucleus cut) and replayed."""
+        rows = self.logits.shape[0]
+        if self.draws is None:
+            self.draws = {}
+            self.draw_host = torch.empty((3, rows), dtype=torch.float32).pin_memory()
+            self.draw_params = torch.empty((3, rows), dtype=torch.float32, device=self.logits.device)
+            self.draw_ids = torch.empty(rows, dtype=torch.int32, device=self.logits.device)
+        self.draw_host.copy_(torch.tensor([temperature, top_p, uniform], dtype=torch.float32))
+        self.draw_params.copy_(self.draw_host, non_blocking=True)
+        ops = engine.model.runtime.ops
+        launch = lambda: ops.sample(self.logits, self.draw_params[0], self.draw_params[1], self.draw_params[2],
+                                    out=self.draw_ids, any_cut=any_cut)
+        captured = self.draws.get(any_cut)
+        if captured is None:
+            launch()                                      # once eagerly: the draw of this call, and a warm-up
+            torch.cuda.synchronize(self.logits.device)
+            captured = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(captured, pool=engine.graph_pool):
+                launch()
+            self.draws[any_cut] = captured
+        else:
+            captured.replay()
+        return [int(v) for v in self.draw_ids.cpu().tolist()]      # (also waits until the pinned buffer is free again)
 
     def run(self, engine: "Engine", entries: list[StepEntry], tokens_on_device: torch.Tensor | None = None) -> torch.Tensor:
         """Pack the batch's description into the fixed buffers again and replay.  `tokens_on_device`: the token
@@ -187,13 +215,17 @@ class Engine:
     def sample(self, logits: torch.Tensor, rows: list[int], temperature: list[float], top_p: list[float],
                uniform: list[float]) -> list[int]:
         """Temperature / nucleus draws for the given rows of a step's logits, on the device; one uniform
-        number per row (from the request's own generator)."""
+        number per row (from the request's own generator).  Draws for all rows of a replayed step's logits
+        replay a captured graph of the sampler's launches as well."""
         device = logits.device
+        any_cut = any(p < 1.0 for p in top_p)
+        graph = self._graph_result
+        if graph is not None and logits is graph.logits and rows == list(range(logits.shape[0])):
+            return graph.draw(self, temperature, top_p, uniform, any_cut)
         picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=device)]
         # One copy to the device for the three vectors.
         packed = torch.tensor([temperature, top_p, uniform], dtype=torch.float32).to(device, non_blocking=True)
-        ids = self.model.runtime.ops.sample(picked.contiguous(), packed[0], packed[1], packed[2],
-                                            any_cut=any(p < 1.0 for p in top_p))
+        ids = self.model.runtime.ops.sample(picked.contiguous(), packed[0], packed[1], packed[2], any_cut=any_cut)
         return [int(v) for v in ids.cpu().tolist()]
 
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):

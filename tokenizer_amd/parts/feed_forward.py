@@ -23,8 +23,17 @@ class GatedDense(FeedForward):
         if spec.activation != "silu":
             raise ValueError(f"gated_dense knows the silu activation, not {spec.activation!r}")
         self.spec, self.runtime = spec, runtime
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        gate, up, down = tensors["gate_proj.weight"], tensors["up_proj.weight"], tensors["down_proj.weight"]
+        # The bfloat16 products read eight elements of K at a time.  An inner width that is no multiple of
+        # eight is filled up with zero rows of gate and up and zero columns of down: act(0) * 0 = 0 meets a
+        # zero weight, so every sum keeps its terms and gains only zeros.
+        fill = (-spec.intermediate_size) % 8 if runtime.dtype == torch.bfloat16 else 0
+        if fill:
+            rows = gate.new_zeros((fill, gate.shape[1]))
+            gate, up = torch.cat([gate, rows], dim=0), torch.cat([up, rows], dim=0)
+            down = torch.cat([down, down.new_zeros((down.shape[0], fill))], dim=1).contiguous()
+        self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+        self.w_down = down
 
     @staticmethod
     def tensor_specs(spec: FeedForwardSpec) -> dict[str, TensorSpec]:
