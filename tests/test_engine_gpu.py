@@ -522,3 +522,25 @@ def test_sizes_away_from_every_tile(tmp_path, size):
             got = tt.run_in_process(eng, steps)
             for rid in reqs:
                 close(got[rid], want[rid], dtype)
+
+
+def test_the_whole_model_at_half_a_billion_parameters(tmp_path):
+    # All 24 layers and the vocabulary of 151,936 at Qwen2.5-0.5B sizes, random weights: prompts in portions beside
+    # decoded tokens and with their last tokens one by one, in 32-bit and in bfloat16, against the plain implementation.
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    raw = dict(TINY["A"][0], num_hidden_layers=24, vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6,
+               tie_word_embeddings=True, max_position_embeddings=32768, sliding_window=32768, max_window_layers=24,
+               **REAL_SIZES["0.5b"])
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 0, str(tmp_path / "half_b"))
+    cfg, tensors = plain.load_folder(folder)
+    reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 50 + i) for i, n in enumerate([150, 70, 33])}
+    want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (tt.mixed(reqs, 3), tt.decode_tail(reqs, 8)):
+            eng = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=4)
+            eng.pools.poison()
+            got = tt.run_in_process(eng, steps)
+            for rid in reqs:
+                close(got[rid], want[rid], dtype)
+            del eng
