@@ -1,13 +1,17 @@
 // C[M,N] = A[M,K] * W[N,K]^T (+ bias) in bfloat16 with float accumulation through the vendor's library
-// (hipBLASLt), called directly: the description of a product and the algorithm the library's heuristic picks
-// for it are made once per shape and kept, so that a call costs the host a few microseconds.  The reference's
-// engine uses a library for its matrix products as well.  No device code here.
+// (hipBLASLt), called directly: the description of a product and its algorithm are made once per shape and
+// kept, so that a call costs the host a few microseconds.  The algorithm is the heuristic's first choice at
+// first.  A big product whose shape is worth it (the caller says so: the step is about to be recorded into a
+// graph; or the shape has come up many times) gets the fastest of the heuristic's candidates instead, each
+// run a few times on the operands of that call.  The reference's engine uses a library for its matrix
+// products as well.  No device code here.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 
 #include <cstdint>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 namespace {
 
@@ -27,14 +31,41 @@ struct ShapeHash {
 struct Plan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t w = nullptr, x = nullptr, c = nullptr;
-  hipblasLtMatmulAlgo_t algo;
-  size_t workspace = 0;
-  bool usable = false;
+  std::vector<hipblasLtMatmulHeuristicResult_t> candidates;   // those that fit the workspace, best guess first
+  size_t chosen = 0;
+  bool usable = false, tuned = false;
+  int calls = 0;
 };
 
 std::mutex guard;
 std::unordered_map<int, hipblasLtHandle_t> handles;       // one per device
 std::unordered_map<Shape, Plan, ShapeHash> plans;
+bool tuning = true;
+constexpr double TUNE_FROM_WORK = 1073741824.0;           // multiply-adds from which the candidates are timed
+constexpr int TUNE_AFTER_CALLS = 64;                      // ... unasked, once a shape has come up this often
+
+// The operands of the call that makes a plan: what the candidates are timed on.
+struct Operands {
+  const void* a; const void* w; const void* bias; void* c;
+  void* workspace; size_t workspace_bytes; hipStream_t stream;
+};
+
+// Milliseconds of `runs` products with this algorithm after one that warms it up; negative if it fails.
+float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& o,
+                hipEvent_t start, hipEvent_t stop, int runs) {
+  const float one = 1.f, zero = 0.f;
+  for (int i = 0; i <= runs; ++i) {
+    if (i == 1 && hipEventRecord(start, o.stream) != hipSuccess) return -1.f;
+    if (hipblasLtMatmul(handle, p.desc, &one, o.w, p.w, o.a, p.x, &zero, o.c, p.c, o.c, p.c, &algo, o.workspace,
+                        o.workspace_bytes, o.stream) != HIPBLAS_STATUS_SUCCESS)
+      return -1.f;
+  }
+  float ms = -1.f;
+  if (hipEventRecord(stop, o.stream) != hipSuccess || hipEventSynchronize(stop) != hipSuccess ||
+      hipEventElapsedTime(&ms, start, stop) != hipSuccess)
+    return -1.f;
+  return ms;
+}
 
 // Row-major C = A W^T is, in the library's column-major terms, C^T [N x M] = op(W) [N x K] * A^T [K x M]:
 // W as stored is a K x N column-major matrix (transposed by the operation), A as stored a K x M one.
@@ -60,30 +91,49 @@ Plan make_plan(hipblasLtHandle_t handle, const Shape& s, size_t workspace_bytes)
   hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
                                         sizeof(workspace_bytes));
   // The heuristic's first choice may want more workspace than it was told there is: the first that fits is taken.
-  constexpr int CANDIDATES = 8;
+  constexpr int CANDIDATES = 24;
   hipblasLtMatmulHeuristicResult_t found[CANDIDATES];
   int count = 0;
   const hipblasStatus_t status =
       hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.x, p.c, p.c, pref, CANDIDATES, found, &count);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (status != HIPBLAS_STATUS_SUCCESS) return p;
-  for (int i = 0; i < count && !p.usable; ++i) {
-    if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > workspace_bytes) continue;
-    p.algo = found[i].algo;
-    p.workspace = found[i].workspaceSize;
-    p.usable = true;
-  }
+  for (int i = 0; i < count; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes)
+      p.candidates.push_back(found[i]);
+  p.usable = !p.candidates.empty();
+  // Small products keep the first choice: timed on operands that sit in the caches they would be misjudged.
+  p.tuned = !tuning || p.candidates.size() < 2 || (double)s.m * s.n * s.k < TUNE_FROM_WORK;
   return p;
+}
+
+// Time every candidate on these operands (the result they leave is the product all the same) and keep the
+// fastest.  Not while the stream records a graph: the plan then stays as it is until a later call.
+void tune_plan(hipblasLtHandle_t handle, Plan& p, const Operands& o) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(o.stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return;
+  p.tuned = true;
+  hipEvent_t start = nullptr, stop = nullptr;
+  if (hipEventCreate(&start) == hipSuccess && hipEventCreate(&stop) == hipSuccess) {
+    float best_ms = -1.f;
+    for (size_t i = 0; i < p.candidates.size(); ++i) {
+      const float ms = time_algo(handle, p, p.candidates[i].algo, o, start, stop, 3);
+      if (ms >= 0.f && (best_ms < 0.f || ms < best_ms)) { best_ms = ms; p.chosen = i; }
+    }
+  }
+  if (start) hipEventDestroy(start);
+  if (stop) hipEventDestroy(stop);
 }
 
 }  // namespace
 
 // A, W, C bfloat16 (rows of A `lda` apart, of C `ldc`), bias float32 [N] or null; `workspace`: device memory
-// the library may use (the same for every call; products on one stream follow one another).
+// the library may use (the same for every call; products on one stream follow one another); `tune`: this
+// shape will come again and again (its step is about to be recorded), so the choice of algorithm is worth timing.
 // Returns 0; -3 if the library offers no algorithm for the shape (the caller uses a kernel of its own);
 // -1 for arguments that make no sense; 1000 + the library's status for its errors.
 extern "C" int ta_library_gemm_bf16(const void* A, const void* W, const void* bias, void* C, int M, int N, int K,
-                                    int lda, int ldc, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                                    int lda, int ldc, void* workspace, size_t workspace_bytes, int tune, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || lda < K || ldc < N || !A || !W || !C) return -1;
   int device = 0;
@@ -100,12 +150,22 @@ extern "C" int ta_library_gemm_bf16(const void* A, const void* W, const void* bi
   auto plan_at = plans.find(shape);
   if (plan_at == plans.end()) plan_at = plans.emplace(shape, make_plan(handle_at->second, shape, workspace_bytes)).first;
   Plan& plan = plan_at->second;
-  if (!plan.usable || plan.workspace > workspace_bytes) return -3;
+  if (!plan.usable) return -3;
   if (bias)
     hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+  if (!plan.tuned && (tune || ++plan.calls >= TUNE_AFTER_CALLS))
+    tune_plan(handle_at->second, plan, Operands{A, W, bias, C, workspace, workspace_bytes, stream});
+  const hipblasLtMatmulHeuristicResult_t& choice = plan.candidates[plan.chosen];
   const float one = 1.f, zero = 0.f;
   const hipblasStatus_t status =
       hipblasLtMatmul(handle_at->second, plan.desc, &one, W, plan.w, A, plan.x, &zero, C, plan.c, C, plan.c,
-                      &plan.algo, workspace, workspace_bytes, stream);
+                      &choice.algo, workspace, workspace_bytes, stream);
   return status == HIPBLAS_STATUS_SUCCESS ? 0 : 1000 + (int)status;
+}
+
+// Whether plans made from now on time the heuristic's candidates (the default) or take its first choice.
+extern "C" int ta_library_gemm_tuning(int on) {
+  std::lock_guard<std::mutex> lock(guard);
+  tuning = on != 0;
+  return 0;
 }

@@ -60,7 +60,7 @@ class Ops:
                      "ta_argmax", "ta_sample", "ta_sample_workspace_words", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
-            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
         self._workspaces: dict[int, torch.Tensor] = {}
 
     @staticmethod
@@ -327,9 +327,12 @@ class Ops:
                 # costs the host some 15 us against 4 us for a kernel of this package: outside graph capture,
                 # products of more than 64 rows that are over on the device in about that time stay with the
                 # tiled kernel (steps of small models with few tokens are bound by the host's launches).
+                # In the run that warms a step up before it is recorded the library is told that the shape
+                # will come again: it then times its candidates for a big product and keeps the fastest.
                 space = self._workspace(x.device)
                 status = self.lib.ta_library_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
-                                                       _ptr(space), space.numel(), self._stream())
+                                                       _ptr(space), space.numel(), int(self.capturing),
+                                                       self._stream())
                 if status != -3:                  # -3: no algorithm for this shape, the kernels below take it
                     self._check(status, "linear (vendor library)")
                     return out
