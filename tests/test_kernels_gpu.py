@@ -167,6 +167,28 @@ def make_batch(lengths, q_lens):
                                  max_position=max(lengths) - 1)
 
 
+def dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale):
+    """Attention of each request's last q_len tokens over its keys as one masked matrix product per request
+    (float32): what the per-token reference computes, fast enough for thousands of tokens."""
+    page_size, group = k_pages.shape[2], n_q // n_kv
+    out, row = [], 0
+    for e, (length, q_len) in enumerate(zip(lengths, q_lens)):
+        pages = table[e, :-(-length // page_size)].long()
+        k = k_pages[pages].float().permute(1, 0, 2, 3).reshape(n_kv, -1, d)[:, :length]          # [n_kv, L, d]
+        v = v_pages[pages].float().permute(1, 0, 3, 2).reshape(n_kv, -1, d)[:, :length]
+        q = qkv[row:row + q_len, :n_q * d].float().reshape(q_len, n_kv, group, d).permute(1, 2, 0, 3)   # [n_kv, g, T, d]
+        scores = torch.einsum("kgtd,kld->kgtl", q, k) * scale
+        pos = torch.arange(length - q_len, length, device=qkv.device)[:, None]
+        key = torch.arange(length, device=qkv.device)[None, :]
+        seen = key <= pos
+        if window is not None:
+            seen &= key >= pos - window
+        probs = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1)
+        out.append(torch.einsum("kgtl,kld->tkgd", probs, v).reshape(q_len, n_q * d))
+        row += q_len
+    return torch.cat(out)
+
+
 # (dtype, fast): the generic kernel in both dtypes, the matrix-core kernels in bfloat16.
 ATTENTION_MODES = [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)]
 
@@ -227,6 +249,30 @@ def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, windo
                         max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
     ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
     torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
+
+
+@pytest.mark.parametrize("geometry,lengths,q_lens", [((14, 2, 64, 16), [4500, 333], [4400, 50]),
+                                                     ((28, 2, 64, 16), [2300, 40], [2200, 33])])
+@pytest.mark.parametrize("window", [None, 1000])
+def test_prefill_attention_with_all_heads_of_a_group_in_one_wave(ops, ref, geometry, lengths, q_lens, window):
+    # Head size 64, seven (or twice seven) query heads per kv head and so many tiles that the launcher gives a
+    # wave all seven heads: portions that start and end inside pages and tiles, with and without a window.
+    n_q, n_kv, d, page_size = geometry
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=23)
+    batch = make_batch(lengths, q_lens)
+    assert batch.q_tiles.shape[0] * n_kv * (n_q // n_kv // 7) >= 512
+    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, 0.125,
+                        max_position=max(lengths) - 1, batch=batch)
+    out_b = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, 0.125)
+    torch.testing.assert_close(out_a.float(), out_b, **attention_tol(torch.bfloat16, True))
+    # The plain per-token reference on a few rows pins the dense one used above.
+    rows = torch.tensor([0, 17, q_lens[0] - 1, q_lens[0], qkv.shape[0] - 1]).cuda()
+    out_c = torch.empty((len(rows), n_q * d), dtype=torch.bfloat16).cuda()
+    ref.paged_attention(qkv[rows], out_c, k_pages, v_pages, positions[rows], entry_of_token[rows], table, n_q, n_kv, d,
+                        window, 0.125)
+    torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
 
 
 @pytest.mark.parametrize("window", [None, 1000])
