@@ -119,7 +119,7 @@ def run_decode(model, batch: int, steps: int, warmup: int):
     return elapsed, kv_mean
 
 
-def run_prefill(model, repeats: int = 3):
+def run_prefill(model, repeats: int = 7):
     import torch
     from tokenizer_amd.engine import Engine, StepEntry
     engine = Engine(model, num_pages=PROMPT_LEN // 16 + 8, page_size=16, max_requests=1)

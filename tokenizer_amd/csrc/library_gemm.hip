@@ -41,7 +41,10 @@ std::mutex guard;
 std::unordered_map<int, hipblasLtHandle_t> handles;       // one per device
 std::unordered_map<Shape, Plan, ShapeHash> plans;
 bool tuning = true;
-constexpr double TUNE_FROM_WORK = 1073741824.0;           // multiply-adds from which the candidates are timed
+// Multiply-adds from which the candidates are timed.  The timing sees launches from the host, one after the
+// other: a product that is over on the device before the host has launched the next one (some 15 us) would be
+// judged by the host's pace and not by its own.
+constexpr double TUNE_FROM_WORK = 4294967296.0;
 constexpr int TUNE_AFTER_CALLS = 64;                      // ... unasked, once a shape has come up this often
 
 // The operands of the call that makes a plan: what the candidates are timed on.
@@ -117,7 +120,7 @@ void tune_plan(hipblasLtHandle_t handle, Plan& p, const Operands& o) {
   if (hipEventCreate(&start) == hipSuccess && hipEventCreate(&stop) == hipSuccess) {
     float best_ms = -1.f;
     for (size_t i = 0; i < p.candidates.size(); ++i) {
-      const float ms = time_algo(handle, p, p.candidates[i].algo, o, start, stop, 3);
+      const float ms = time_algo(handle, p, p.candidates[i].algo, o, start, stop, 5);
       if (ms >= 0.f && (best_ms < 0.f || ms < best_ms)) { best_ms = ms; p.chosen = i; }
     }
   }
