@@ -550,6 +550,37 @@ def test_fused_norm_gated_and_linear_add(ops, ref, shape):
     torch.testing.assert_close(res_a, res_b, **linear_tol(torch.float32, wide[:, :inner], down))
 
 
+@pytest.mark.parametrize("shape", [(40, 896, 4864), (64, 1536, 8960), (17, 2048, 11008), (33, 100, 2048)])
+def test_product_left_in_parts_and_added_by_the_norm(ops, ref, shape):
+    # A product of 17 to 64 rows whose K is cut over workgroups may come back in parts; the norm that takes it as
+    # its delta adds the parts, the bias and the residual and normalises in one kernel.  Both that and the parts
+    # added on their own agree with the plain product and the plain norm.
+    from tokenizer_amd.kernels import PendingSum
+    m, n, k = shape
+    x, w = rand((m, k), torch.bfloat16, 1), rand((n, k), torch.bfloat16, 2, 0.05)
+    bias, gain = rand((n,), torch.float32, 3), 1 + rand((n,), torch.float32, 4, 0.1)
+    residual = rand((m, n), torch.float32, 5, 2.0)
+    got = ops.linear(x, w, bias, pending=True)
+    assert isinstance(got, PendingSum) and got.shape == (m, n) and got.partial.shape[0] > 1
+    plain_product = ref.linear(x, w, bias, out_dtype=torch.float32)
+    torch.testing.assert_close(got.resolve().float(), plain_product, rtol=2e-2, atol=2e-2)
+    # (the product that adds its parts itself may cut K differently: equal up to the rounding of the sums)
+    torch.testing.assert_close(got.resolve().float(), ops.linear(x, w, bias).float(), **tol(torch.bfloat16))
+    assert torch.equal(got.resolve(), got.resolve())
+    res_a, res_b = residual.clone(), residual.clone()
+    out_a = ops.add_rmsnorm(res_a, got, gain, 1e-6, torch.empty((m, n), dtype=torch.bfloat16).cuda())
+    out_b = ref.add_rmsnorm(res_b, plain_product, gain, 1e-6, torch.empty((m, n), dtype=torch.float32).cuda())
+    torch.testing.assert_close(res_a, res_b, rtol=1e-4, atol=1e-3)
+    torch.testing.assert_close(out_a.float(), out_b, rtol=2e-2, atol=2e-2)
+    # A row subset (the final norm) has the parts added first.
+    rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
+    res_c = residual.clone()
+    out_c = ops.add_rmsnorm(res_c, got, gain, 1e-6, torch.empty((2, n), dtype=torch.bfloat16).cuda(), rows,
+                            store_residual=False)
+    assert torch.equal(res_c, residual)
+    torch.testing.assert_close(out_c.float(), out_b[rows.long()], rtol=2e-2, atol=2e-2)
+
+
 def test_linear_float32_is_true_float32(ops):
     # Inputs that need 13 mantissa bits: a reduced-precision matrix mode (10 or 7 bits) would be off by
     # about 1e-2 here, float32 accumulation by less than 3e-4.

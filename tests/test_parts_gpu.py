@@ -177,6 +177,7 @@ def test_wide_models_take_the_norm_out_of_the_fused_decode_products(hidden):
 def test_block_alone(dtype):
     # One pre-norm block with its own sizes: norm, attention, add, norm, feed-forward, add (the last add is
     # left to the next norm, so the block hands back the stream and what is still to be added).
+    from tokenizer_amd.parts import as_tensor
     from tokenizer_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, FeedForwardSpec, LayerCache, MixerSpec,
                                      NormSpec, PositionSpec)
     n_q, n_kv, d, hidden, inner = 3, 1, 32, 96, 136
@@ -207,7 +208,7 @@ def test_block_alone(dtype):
         x = rand((sum(lengths), hidden), 45)
         residual = x.cuda().clone()
         delta = block.forward(residual, None, ctx, LayerCache(group=0, k_pages=k_pages, v_pages=v_pages))
-        got = residual.cpu() + (0 if delta is None else delta.float().cpu())
+        got = residual.cpu() + (0 if delta is None else as_tensor(delta).float().cpu())
         cos, sin = plain.rope_tables(10000.0, d, 64)
         at = 0
         for n in lengths:

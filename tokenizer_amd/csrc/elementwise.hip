@@ -95,6 +95,51 @@ add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta
   }
 }
 
+// The same with the delta still in parts: a product whose K was cut over workgroups left `splits` slabs of
+// float sums [M, hidden]; they are added in their order, the bias joins, the sum goes into the residual stream
+// (stored back) and the row is normalised.  One kernel instead of the addition and the norm after it.
+template <typename T>
+__global__ void __launch_bounds__(256)
+splitk_add_rmsnorm_kernel(float* __restrict__ residual, const float* __restrict__ partial, int splits,
+                          const float* __restrict__ bias, const float* __restrict__ weight, T* __restrict__ out,
+                          int n_rows, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  float* res = residual + (size_t)i * hidden;
+  float4 x[4];
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int h = (c * 256 + threadIdx.x) * 4;
+    x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (h < hidden) {
+      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int s = 0; s < splits; ++s) {
+        const float4 v = ld4(partial + ((size_t)s * n_rows + i) * hidden + h);
+        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+      }
+      if (bias) {
+        const float4 b = ld4(bias + h);
+        sum.x += b.x; sum.y += b.y; sum.z += b.z; sum.w += b.w;
+      }
+      x[c] = ld4(res + h);
+      x[c].x += sum.x; x[c].y += sum.y; x[c].z += sum.z; x[c].w += sum.w;
+      st4(res + h, x[c]);
+    }
+    sq += x[c].x * x[c].x + x[c].y * x[c].y + x[c].z * x[c].z + x[c].w * x[c].w;
+  }
+  const float total = block_sum(sq, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int h = (c * 256 + threadIdx.x) * 4;
+    if (h >= hidden) continue;
+    const float4 w = ld4(weight + h);
+    st4(dst + h, make_float4(x[c].x * inv * w.x, x[c].y * inv * w.y, x[c].z * inv * w.z, x[c].w * inv * w.w));
+  }
+}
+
 // out[t, j] = silu(in[t, j]) * in[t, inner + j], silu(z) = z * sigmoid(z), in float.
 template <typename T>
 __global__ void silu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, int inner, size_t total) {
@@ -157,6 +202,24 @@ extern "C" int ta_add_rmsnorm(void* residual, const void* delta, const void* wei
   else
     add_rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((float*)residual, (const bf16_t*)delta, (const float*)weight,
                                                            (bf16_t*)out, (const int*)rows, hidden, eps, store_residual);
+  return LAUNCH_STATUS();
+}
+
+// residual [n_rows, hidden] += the slabs of `partial` ([splits, n_rows, hidden] floats, added in order) + bias;
+// out = rmsnorm(residual) * weight.  hidden a multiple of 4 and at most 4096.
+extern "C" int ta_splitk_add_rmsnorm(void* residual, const void* partial, int splits, const void* bias,
+                                     const void* weight, void* out, int n_rows, int hidden, float eps, int dtype,
+                                     hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (hidden % 4 || hidden > 4096 || splits < 1 || !partial) return -1;
+  if (dtype == DT_F32)
+    splitk_add_rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)partial, splits,
+                                                                 (const float*)bias, (const float*)weight, (float*)out,
+                                                                 n_rows, hidden, eps);
+  else
+    splitk_add_rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)partial, splits,
+                                                                  (const float*)bias, (const float*)weight, (bf16_t*)out,
+                                                                  n_rows, hidden, eps);
   return LAUNCH_STATUS();
 }
 

@@ -144,7 +144,7 @@ static int launch(const void* A, const void* W, const void* bias, void* C, int M
     gemm_bf16_kernel<BM, BN, BK, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, (const float*)bias,
                                                                (bf16_t*)C, M, N, K, lda, ldc, k_chunk, slabs);
   int status = LAUNCH_STATUS();
-  if (status == 0 && splits > 1) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
+  if (status == 0 && splits > 1 && C) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
   return status;
 }
 
@@ -164,9 +164,19 @@ extern "C" int ta_gemm_bf16(const void* A, const void* W, const void* bias, void
 
 // The same product with K cut into `splits` parts (at most; parts are multiples of 64) over 64 x 64 tiles, the
 // parts' float sums added afterwards in a fixed order.  partial: room for splits * M * N floats; N % 4 == 0.
+// With C null (and more than one part after the rounding of the parts' length) the sums are left in `partial`.
 extern "C" int ta_gemm_bf16_splitk(const void* A, const void* W, const void* bias, void* C, void* partial, int M,
                                    int N, int K, int lda, int ldc, int out_dtype, int splits, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if ((K & 7) || (lda & 7) || (N & 3) || splits < 1 || (splits > 1 && !partial)) return -1;
+  if (!C && parts_of_k(K, splits, 64) < 2) return -1;
   return launch<64, 64, 64>(A, W, bias, C, M, N, K, lda, ldc, out_dtype, stream, splits, partial);
+}
+
+// The addition alone: C[M, N] (row stride ldc) = the `splits` slabs of `partial` in their order + bias.
+extern "C" int ta_splitk_reduce(const void* partial, const void* bias, void* C, int M, int N, int ldc, int splits,
+                                int out_dtype, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if ((N & 3) || splits < 1 || !partial || !C) return -1;
+  return launch_splitk_reduce((const float*)partial, bias, C, M, N, ldc, splits, out_dtype, stream);
 }

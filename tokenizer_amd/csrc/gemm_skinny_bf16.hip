@@ -217,7 +217,7 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
     skinny_gemm_kernel<MB, NW, GATED, bf16_t><<<grid, NW * WAVE, 0, stream>>>(
         (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)C, ldc, M, N, K, k_chunk, slabs);
   int status = LAUNCH_STATUS();
-  if (status == 0 && splits > 1) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
+  if (status == 0 && splits > 1 && C) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
   return status;
 }
 
@@ -253,12 +253,14 @@ extern "C" int ta_gemm_skinny_bf16(const void* A, int lda, const void* W, const 
 
 // The same product (not gated) with K cut into `splits` parts (at most; parts are multiples of 32) over the
 // workgroups, the parts' float sums added afterwards in a fixed order.  partial: room for splits * M * N floats;
-// N % 4 == 0; M <= 64.
+// N % 4 == 0; M <= 64.  With C null (and more than one part after the rounding of the parts' length) the sums are
+// left in `partial` for a later kernel to add.
 extern "C" int ta_gemm_skinny_bf16_splitk(const void* A, int lda, const void* W, const void* bias, void* C, int ldc,
                                           void* partial, int M, int N, int K, int out_dtype, int splits,
                                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 7) || (lda & 7) || (N & 3) || splits < 1 || (splits > 1 && !partial)) return -1;
+  if (!C && parts_of_k(K, splits, 32) < 2) return -1;
 #define GO(MBV) launch_skinny<MBV, 8, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, splits, partial)
   switch ((M + 15) / 16) {
     case 1: return GO(1);

@@ -25,6 +25,14 @@ __global__ void splitk_reduce(const float* __restrict__ partial, const float* __
   store_out(dst, sum.x); store_out(dst + 1, sum.y); store_out(dst + 2, sum.z); store_out(dst + 3, sum.w);
 }
 
+// Into how many parts K really falls when `splits` are asked for and a part is a multiple of `step`: no part
+// without a step of its own.
+static inline int parts_of_k(int K, int splits, int step) {
+  if (splits <= 1) return 1;
+  const int chunk = ((K + splits - 1) / splits + step - 1) / step * step;
+  return (K + chunk - 1) / chunk;
+}
+
 // Launches the reduction; returns the launch status.
 static inline int launch_splitk_reduce(const float* slabs, const void* bias, void* C, int M, int N, int ldc, int splits,
                                        int out_dtype, hipStream_t stream) {

@@ -49,6 +49,31 @@ def _dev(*tensors: torch.Tensor | None) -> None:
             _need(tensor.is_contiguous(), "kernel operands must be contiguous")
 
 
+def _parts_of_k(k: int, splits: int, step: int) -> int:
+    """Into how many parts K really falls when `splits` are asked for and a part is a multiple of `step`."""
+    if splits <= 1:
+        return 1
+    chunk = -(-(-(-k // splits)) // step) * step
+    return -(-k // chunk)
+
+
+class PendingSum:
+    """A product whose K was cut over workgroups, before its parts are added: float32 slabs [parts, M, N] and
+    the bias that joins their sum.  `Ops.add_rmsnorm` takes it as the delta and adds the parts, the bias and the
+    residual and normalises in one kernel; `resolve()` adds the parts on their own and gives the product."""
+
+    def __init__(self, ops: "Ops", partial: torch.Tensor, bias: torch.Tensor | None, dtype: torch.dtype):
+        self.ops, self.partial, self.bias, self.dtype = ops, partial, bias, dtype
+        self.shape = tuple(partial.shape[1:])
+
+    def resolve(self) -> torch.Tensor:
+        parts, m, n = self.partial.shape
+        out = torch.empty((m, n), dtype=self.dtype, device=self.partial.device)
+        self.ops._check(self.ops.lib.ta_splitk_reduce(_ptr(self.partial), _ptr(self.bias), _ptr(out), m, n, n, parts,
+                                                      _code(self.dtype), self.ops._stream()), "splitk_reduce")
+        return out
+
+
 class Ops:
     """The kernel library.  One instance per process; see `get_ops()`."""
 
@@ -56,7 +81,7 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated", "ta_splitk_reduce", "ta_splitk_add_rmsnorm",
                      "ta_argmax", "ta_sample", "ta_sample_workspace_words", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
@@ -102,9 +127,25 @@ class Ops:
                     store_residual: bool = True) -> torch.Tensor:
         """x = residual[r] (+ delta[r]); optionally residual[r] = x; out[i] = rmsnorm(x) * weight.
 
-        residual float32 [T, H]; delta [T, H] in out's dtype or None; weight float32 [H];
+        residual float32 [T, H]; delta [T, H] in out's dtype, None, or a `PendingSum` (the parts of a product
+        still to be added: they are added here, in the same kernel); weight float32 [H];
         rows int32 [R] picks the rows (None: all, R = T); out [R, H].
         """
+        if isinstance(delta, PendingSum):
+            n_tokens, hidden = residual.shape
+            if (rows is not None or not store_residual or hidden % 4 or hidden > 4096
+                    or delta.shape != (n_tokens, hidden)):
+                delta = delta.resolve()
+            else:
+                _dev(residual, weight, out)
+                _need(residual.dtype == torch.float32, "the residual stream is float32")
+                _need(weight.dtype == torch.float32 and weight.numel() == hidden, "norm weight must be float32 [H]")
+                _need(tuple(out.shape) == (n_tokens, hidden) and out.dtype == delta.dtype, "norm output has the wrong shape")
+                self._check(self.lib.ta_splitk_add_rmsnorm(
+                    _ptr(residual), _ptr(delta.partial), delta.partial.shape[0], _ptr(delta.bias), _ptr(weight),
+                    _ptr(out), n_tokens, hidden, ctypes.c_float(eps), _code(out.dtype), self._stream()),
+                    "splitk_add_rmsnorm")
+                return out
         _dev(residual, delta, weight, out, rows)
         n_tokens, hidden = residual.shape
         n_rows = n_tokens if rows is None else rows.numel()
@@ -264,12 +305,17 @@ class Ops:
         return out
 
     # --------------------------------------------------------------------- linear
+    takes_pending = True      # `linear(pending=True)` and `add_rmsnorm` with a `PendingSum` exist here
+
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+               out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+               pending: bool = False) -> "torch.Tensor | PendingSum":
         """out = x @ weight.T (+ bias).  x [M, K] (rows may be strided); weight [N, K]; bias float32 [N].
 
         float32 operands run on plain multiply-adds; bfloat16 operands on the matrix cores with
-        float accumulation and a bfloat16 or float32 result.
+        float accumulation and a bfloat16 or float32 result.  `pending=True` allows the result to come back
+        as a `PendingSum` when K is cut over workgroups: whoever takes it next (the norm that follows) adds the
+        parts in its own kernel and the addition's launch is saved.
         """
         _need(x.is_cuda and weight.is_cuda, "kernel operands must live on the GPU")
         _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "linear shapes do not fit")
@@ -280,9 +326,11 @@ class Ops:
         lda = x.stride(0) if m > 1 else k
         if out_dtype is None:
             out_dtype = x.dtype if out is None else out.dtype
-        if out is None:
+        pending = pending and out is None and x.dtype == torch.bfloat16
+        if out is None and not pending:
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-        _need(tuple(out.shape) == (m, n) and out.is_contiguous() and out.dtype == out_dtype, "linear output shape")
+        if out is not None:
+            _need(tuple(out.shape) == (m, n) and out.is_contiguous() and out.dtype == out_dtype, "linear output shape")
         if bias is not None:
             _need(bias.is_cuda and bias.dtype == torch.float32 and bias.numel() == n, "bias must be float32 [N]")
         if x.dtype == torch.float32:
@@ -293,24 +341,34 @@ class Ops:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-            streaming_splits = self._streaming_splits(m, n, k)
+            streaming_splits = self._streaming_splits(m, n, k, pending)
             if streaming_splits > 1 and self.split_k_kind == "streaming":
                 # 17 to 64 rows, a long K and few output columns (the down projection of a decode batch): the
                 # weight-streaming kernel with K cut over workgroups, so that every compute unit streams a share
                 # of the weights; the parts are added in a fixed order by a second small kernel.
-                partial = torch.empty((streaming_splits, m, n), dtype=torch.float32, device=x.device)
+                parts = _parts_of_k(k, streaming_splits, 32)
+                leave = pending and parts > 1
+                if out is None and not leave:
+                    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+                partial = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
                 self._check(self.lib.ta_gemm_skinny_bf16_splitk(
-                    _ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, _ptr(partial), m, n, k, _code(out_dtype),
-                    streaming_splits, self._stream()), "linear")
-                return out
+                    _ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(None if leave else out), n, _ptr(partial), m, n, k,
+                    _code(out_dtype), streaming_splits, self._stream()), "linear")
+                return PendingSum(self, partial, bias, out_dtype) if leave else out
             splits = self._k_splits(m, n, k)
             if splits > 1:
                 # The same with the tiled kernel.
-                partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
-                self._check(self.lib.ta_gemm_bf16_splitk(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(partial),
-                                                         m, n, k, lda, n, _code(out_dtype), splits, self._stream()),
-                            "linear")
-                return out
+                parts = _parts_of_k(k, splits, 64)
+                leave = pending and parts > 1
+                if out is None and not leave:
+                    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+                partial = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+                self._check(self.lib.ta_gemm_bf16_splitk(
+                    _ptr(x), _ptr(weight), _ptr(bias), _ptr(None if leave else out), _ptr(partial), m, n, k, lda, n,
+                    _code(out_dtype), splits, self._stream()), "linear")
+                return PendingSum(self, partial, bias, out_dtype) if leave else out
+            if out is None:
+                out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             if m > self.SKINNY_ROWS:
                 to_library = self.capturing or m * n * k >= self.EAGER_LIBRARY_WORK
             else:
@@ -359,20 +417,23 @@ class Ops:
 
     split_k_kind = "streaming"     # which kernel cuts K for 17 to 64 rows ("tiled": only the tiled one)
 
-    def _streaming_splits(self, m: int, n: int, k: int) -> int:
+    def _streaming_splits(self, m: int, n: int, k: int, pending: bool = False) -> int:
         """Into how many parts the weight-streaming kernel cuts K for 17 to 64 rows and a K of 2,048 up to where
         the tiled kernel takes over: so many that its tiles of sixteen output columns times the parts give every
         compute unit a workgroup, each part at least 512 long.  (Measured with cold weights for the down
         projections of the 0.5B to 7B models: one of the two beats the library at every row count from 17 to 64,
         the streaming kernel while a part is a few steps per wave, the tiled one, which reads the rows a quarter
-        as often, for longer K.)"""
+        as often, for longer K.)  When the parts may be left for the next norm to add (`pending`), the addition
+        costs no launch, and a K from 512 on is cut as well, into parts of at least 224 (the output projection of
+        a decode batch: every workgroup reads all the rows, and a quarter of K is a quarter of them)."""
+        shortest, part = (512, 224) if pending else (2048, 512)
         if (not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or n % 4
-                or not (2048 <= k < self.SPLIT_K_FROM)):
+                or not (shortest <= k < self.SPLIT_K_FROM)):
             return 1
         tiles = -(-n // 16)
         if tiles >= 128:
             return 1
-        return max(1, min(-(-256 // tiles), k // 512))
+        return max(1, min(-(-256 // tiles), k // part))
 
     SPLIT_K_FROM = 8192        # the shortest K that the tiled kernel cuts (shorter ones are the weight-streaming kernel's)
 

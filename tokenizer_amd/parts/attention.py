@@ -69,7 +69,9 @@ class GQAttention(Mixer):
                  and self.d % 32 == 0 and cache.group is not None
                  and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
-            return super().forward_normed(residual, delta, norm, ctx, cache)
+            # The output is handed on as a delta: an output product whose K is cut over workgroups may stay in
+            # parts, and the norm that takes it next adds them in its own kernel.
+            return self._run(norm.apply(residual, delta), ctx, cache, pending=getattr(ops, "takes_pending", False))
         if getattr(ops, "fold_norm", lambda hidden: True)(residual.shape[1]):
             rows, norm_weight = residual, norm.weight
         else:                       # a wide model: the norm's own kernel once, not again in every workgroup
@@ -85,6 +87,9 @@ class GQAttention(Mixer):
         return None
 
     def forward(self, x, ctx, cache):
+        return self._run(x, ctx, cache, pending=False)
+
+    def _run(self, x, ctx, cache, pending: bool):
         ops = self.runtime.ops
         can = getattr(ops, "can_rope_store", None)
         if (can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and type(self.position) in (NoPosition, RotaryHalfSplit)
@@ -100,4 +105,4 @@ class GQAttention(Mixer):
         ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
                             ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
                             self.scale, max_position=ctx.max_position, batch=ctx)
-        return ops.linear(mixed, self.w_o, self.b_o)
+        return ops.linear(mixed, self.w_o, self.b_o, pending=True) if pending else ops.linear(mixed, self.w_o, self.b_o)

@@ -8,14 +8,17 @@ Interfaces
 Norm            tensor_specs(spec) -> {local name: TensorSpec}
                 apply(residual, delta, rows=None) -> normalised rows in the compute dtype.
                 `residual` is the float32 stream [T, H]; `delta` (or None) is added to it first and,
-                unless `rows` picks a subset, the sum is stored back.
+                unless `rows` picks a subset, the sum is stored back.  `delta` may also be a product still
+                in parts (`kernels.PendingSum`, which the kernel library's `add_rmsnorm` takes as it is): a
+                norm with kernels of its own calls `as_tensor(delta)` first.
 PositionEncoding
                 encode_and_store(qkv, geometry, ctx, cache, bias): adds the projection bias, encodes
                 the query and key heads in place and writes keys and values of this step into `cache`.
 Mixer           tensor_specs(spec), cache_need(spec) -> CacheNeed
                 forward(x [T, H], ctx: StepContext, cache: LayerCache) -> [T, H] in the compute dtype.
                 Optional: forward_normed(residual, delta, norm, ctx, cache) to fold the norm before it and the
-                residual add after it into its own kernels (returns None when it added its output itself).
+                residual add after it into its own kernels (returns None when it added its output itself; what
+                it returns is only ever handed to a norm as its delta, so it may be a product still in parts).
 FeedForward     tensor_specs(spec); forward(x [T, H], ctx) -> [T, H]; optional forward_normed likewise.
 Block           arranges two norms, a mixer and a feed-forward around the residual stream:
                 forward(residual, delta, ctx, cache) -> delta still to be added.
@@ -121,6 +124,12 @@ class Block:
 
     def forward(self, residual: torch.Tensor, delta: torch.Tensor | None, ctx, cache) -> torch.Tensor:
         raise NotImplementedError
+
+
+def as_tensor(delta):
+    """The delta as a tensor: a product still in parts has them added now."""
+    resolve = getattr(delta, "resolve", None)
+    return resolve() if resolve is not None and not isinstance(delta, torch.Tensor) else delta
 
 
 def can_fuse_decode(ops, residual, dtype) -> bool:

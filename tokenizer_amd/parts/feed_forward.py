@@ -48,7 +48,9 @@ class GatedDense(FeedForward):
         fused = (delta is None and type(norm) is RMSNorm
                  and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
-            return super().forward_normed(residual, delta, norm, ctx)
+            # The output is handed on as a delta: a down product whose K is cut over workgroups may stay in
+            # parts, and the norm that takes it next adds them in its own kernel.
+            return self._run(norm.apply(residual, delta), pending=getattr(ops, "takes_pending", False))
         if getattr(ops, "fold_norm", lambda hidden: True)(residual.shape[1]):
             act = ops.fused_norm_gated(residual, norm.weight, norm.eps, self.w_gate_up)
         else:                       # a wide model: the norm's own kernel once, not again in every workgroup
@@ -57,5 +59,9 @@ class GatedDense(FeedForward):
         return None
 
     def forward(self, x, ctx):
+        return self._run(x, pending=False)
+
+    def _run(self, x, pending: bool):
         ops = self.runtime.ops
-        return ops.linear(ops.linear_silu_gate(x, self.w_gate_up), self.w_down)
+        act = ops.linear_silu_gate(x, self.w_gate_up)
+        return ops.linear(act, self.w_down, pending=True) if pending else ops.linear(act, self.w_down)
