@@ -426,7 +426,7 @@ class Ops:
         as often, for longer K.)  When the parts may be left for the next norm to add (`pending`), the addition
         costs no launch, and a K from 512 on is cut as well, into parts of at least 224 (the output projection of
         a decode batch: every workgroup reads all the rows, and a quarter of K is a quarter of them)."""
-        shortest, part = (512, 224) if pending else (2048, 512)
+        shortest, part = (self.PENDING_SHORTEST_K, 224) if pending else (2048, 512)
         if (not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or n % 4
                 or not (shortest <= k < self.SPLIT_K_FROM)):
             return 1
@@ -435,6 +435,7 @@ class Ops:
             return 1
         return max(1, min(-(-256 // tiles), k // part))
 
+    PENDING_SHORTEST_K = 512   # the shortest K that is cut when the parts may be left for the next norm
     SPLIT_K_FROM = 8192        # the shortest K that the tiled kernel cuts (shorter ones are the weight-streaming kernel's)
 
     EAGER_LIBRARY_WORK = 2 ** 30   # multiply-adds from which a product launched eagerly goes to the library
