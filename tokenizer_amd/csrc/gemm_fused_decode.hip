@@ -1,7 +1,10 @@
 // Fused products for decode batches of up to 16 rows.  Each keeps the layout of the weight-streaming kernel
 // (C^T = W A^T on 16x16x32 MFMAs, the waves of a workgroup split K and add up through LDS) and folds the
 // neighbouring small kernels into its prologue or epilogue:
-//   NORM prologue   the rows are read from the float residual stream and RMS-normalised on the fly
+//   NORM prologue   the rows are read from the float residual stream and RMS-normalised on the fly into LDS
+//                   (or, normalised already, copied there once: what a workgroup pulls in over the fabric from
+//                   the caches counts like what it pulls from memory, and rows asked for again in every batch
+//                   of weights would be half as many bytes again as the weights)
 //   ROPE_STORE      q/k/v projection: bias, half-split rotation, keys and values written into their pages
 //   GATED           silu(gate) * up
 //   RESIDUAL        the product is added into the float residual stream in place
@@ -50,7 +53,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   constexpr int HELD = ONE ? PASSES : 1;                     // batches of weights held at once
   static_assert(EPI != EPI_ROPE_STORE || PASSES == 1, "the rotation pairs rows within one block");
   __shared__ float red[NW][SETS * 4][WAVE];
-  extern __shared__ __attribute__((aligned(16))) uint16_t a_s[];   // NORM: 16 normalised rows of K + 8 bfloat16
+  extern __shared__ __attribute__((aligned(16))) uint16_t a_s[];   // NORM: the m normalised rows of K + 8 bfloat16
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int M = p.m, K = p.k, R = p.rows;
@@ -158,7 +161,16 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
     }
   }
 
-  if (NORM) {
+  if (NORM && !p.residual_in) {
+    // Rows that are normalised already: copied into LDS once.
+    for (int m = wave; m < M; m += NW) {
+      const bf16_t* x = p.a + (size_t)m * p.lda;
+      uint16_t* dst = a_s + (size_t)m * lds_stride;
+      for (int k = lane * 8; k < K; k += WAVE * 8)
+        *reinterpret_cast<uint4*>(dst + k) = *reinterpret_cast<const uint4*>(x + k);
+    }
+    __syncthreads();
+  } else if (NORM) {
     // Each row once: 1 / sqrt(mean(x^2) + eps), then x * that * weight rounded to bfloat16 into LDS.
     for (int m = wave; m < M; m += NW) {
       const float* x = p.residual_in + (size_t)m * K;
@@ -330,7 +342,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
 
 template <int NW, int EPI, bool NORM, int UN, bool ONE, int PASSES>
 static int launch_kernel(const FusedArgs& args, int tiles, hipStream_t stream) {
-  size_t lds = NORM ? (size_t)16 * (args.k + 8) * sizeof(uint16_t) : 0;
+  size_t lds = NORM ? (size_t)args.m * (args.k + 8) * sizeof(uint16_t) : 0;
   if (lds > 48 * 1024) {
     // More dynamic LDS than the default limit: ask for it (the device has 160 KB per compute unit).
     if (lds > 140 * 1024) return -1;
@@ -416,6 +428,10 @@ static int rows_per_workgroup(int n_rows, int rows_override) {
   return rows < 4 ? 4 : rows;
 }
 
+// Rows that are normalised already go through LDS (the NORM instances, which then copy instead of normalising)
+// while two workgroups' copies fit a compute unit beside their other LDS.
+static bool stage_rows(int m, int k) { return (size_t)m * (k + 8) * sizeof(uint16_t) <= 60 * 1024; }
+
 static int fused_qkv_rope(const FusedArgs& base, bool norm, const void* w, const void* bias, void* q_out,
                           const void* positions, const void* cos_sin, const void* slots, void* k_pages, void* v_pages,
                           int m, int k, int n_q, int n_kv, int d, int page_size, int rows, int waves, hipStream_t stream) {
@@ -428,7 +444,7 @@ static int fused_qkv_rope(const FusedArgs& base, bool norm, const void* w, const
   a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.n_q = n_q; a.n_kv = n_kv; a.d = d; a.page_size = page_size;
   a.rows = rows_per_tile(n_q, n_kv, d, m, k, norm, rows);
   const int tiles = (n_q + n_kv) * (d / 2 / a.rows) + n_kv * d / a.rows;
-  if (norm) return launch_rows<EPI_ROPE_STORE, true>(a, tiles, waves, stream);
+  if (norm || stage_rows(m, k)) return launch_rows<EPI_ROPE_STORE, true>(a, tiles, waves, stream);
   return launch_rows<EPI_ROPE_STORE, false>(a, tiles, waves, stream);
 }
 
@@ -479,6 +495,7 @@ extern "C" int ta_fused_gated(const void* x, int lda, const void* w, void* out, 
   a.a = (const bf16_t*)x; a.lda = lda;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
   a.rows = rows_per_workgroup(n / 2, rows);
+  if (stage_rows(m, k)) return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
   return launch_rows<EPI_GATED, false>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
 }
 
