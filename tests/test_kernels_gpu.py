@@ -581,6 +581,32 @@ def test_product_left_in_parts_and_added_by_the_norm(ops, ref, shape):
     torch.testing.assert_close(out_c.float(), out_b[rows.long()], rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("shape", [(33, 48, 264), (64, 100, 896), (50, 900, 40), (64, 1000, 2048)])
+def test_weight_streaming_product_with_two_column_blocks(ops, ref, shape, monkeypatch):
+    # More than 32 rows may take two blocks of sixteen output columns per workgroup (the rows are then read half as
+    # often): with one block and with two, plain, gated and with K cut over workgroups, at widths that end inside
+    # a block and inside a pair of blocks.
+    m, n, k = shape
+    x, w = rand((m, k), torch.bfloat16, 31), rand((n, k), torch.bfloat16, 32, 0.05)
+    bias = rand((n,), torch.float32, 33)
+    monkeypatch.setattr(ops, "use_library_gemm", False)
+    want = ref.linear(x, w, bias, out_dtype=torch.float32)
+    gated_want = ref.linear_silu_gate(x.float(), w.float(), None)
+    results = []
+    for blocks in (1, 2):
+        monkeypatch.setattr(ops, "skinny_column_blocks", blocks)
+        got = ops.linear(x, w, bias)
+        torch.testing.assert_close(got.float(), want, **tol(torch.bfloat16))
+        gated = ops.linear_silu_gate(x, w)
+        torch.testing.assert_close(gated.float(), gated_want, rtol=2e-2, atol=2e-3)
+        parts = ops.linear(x, w, bias, pending=True)
+        if not isinstance(parts, torch.Tensor):
+            parts = parts.resolve()
+        torch.testing.assert_close(parts.float(), want, **tol(torch.bfloat16))
+        results.append((got, gated))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+
+
 def test_linear_float32_is_true_float32(ops):
     # Inputs that need 13 mantissa bits: a reduced-precision matrix mode (10 or 7 bits) would be off by
     # about 1e-2 here, float32 accumulation by less than 3e-4.

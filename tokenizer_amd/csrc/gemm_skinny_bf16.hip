@@ -44,14 +44,19 @@ struct RopeStore {
   int n_q, n_kv, d, page_size;
 };
 
-template <int MB, int NW, bool GATED, typename OutT, bool ROPE = false>
+// NB: blocks of sixteen output columns per workgroup.  Every workgroup reads all the rows of A for its part of K;
+// with two blocks the rows are read half as often, which is what a product of many rows is bound by once the
+// rows outweigh a tile's weights (what comes over the fabric from the caches counts like what comes from memory).
+template <int MB, int NW, bool GATED, typename OutT, bool ROPE = false, int NB = 1>
 __global__ void __launch_bounds__(NW * WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
                    const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K_all,
                    int k_chunk, float* __restrict__ partial, const RopeStore rope = RopeStore()) {
   static_assert(!ROPE || GATED, "the rotation uses the two sets of weight rows");
-  constexpr int SETS = GATED ? 2 : 1;
-  __shared__ float red[NW][SETS * MB * 4][WAVE];
+  static_assert(!ROPE || NB == 1, "the rotation pairs rows within one block");
+  constexpr int HALVES = GATED ? 2 : 1;                     // gate and up rows (or the two halves of a head)
+  constexpr int SETS = HALVES * NB;                         // set h * NB + b: half h, column block b
+  __shared__ float red[NW][HALVES * MB * 4][WAVE];
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int n_out = ROPE ? N : GATED ? N / 2 : N;
@@ -59,14 +64,19 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int rope_half = ROPE ? rope.d / 2 : 0;
   const int rope_head = ROPE ? blockIdx.x / (rope_half / 16) : 0;
   const int rope_first = ROPE ? (blockIdx.x % (rope_half / 16)) * 16 : 0;      // first element of the tile in its head
-  const int n0 = ROPE ? rope_head * rope.d + rope_first : blockIdx.x * 16;
-  // Rows past the end are clamped, not masked: they only feed outputs that are never stored.
-  const int wrow = min(n0 + col, n_out - 1);
+  const int n_first = ROPE ? rope_head * rope.d + rope_first : blockIdx.x * 16 * NB;
   const int k_lo = blockIdx.y * k_chunk;
   const int K = min(K_all, k_lo + k_chunk) - k_lo;                // this workgroup's part of K
-  const bf16_t* w0 = W + (size_t)wrow * K_all + k_lo + 8 * g;
-  // The second set: the `up` rows when GATED, the rows half a head further on with ROPE.
-  const bf16_t* w1 = W + (size_t)(wrow + (ROPE ? rope_half : n_out)) * K_all + k_lo + 8 * g;
+  // Rows past the end are clamped, not masked: they only feed outputs that are never stored.
+  // The second half: the `up` rows when GATED, the rows half a head further on with ROPE.
+  const bf16_t* wp[SETS];
+#pragma unroll
+  for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int wrow = min(n_first + 16 * b + col, n_out - 1) + h * (ROPE ? rope_half : n_out);
+      wp[h * NB + b] = W + (size_t)wrow * K_all + k_lo + 8 * g;
+    }
   // Lanes of activation rows past M load nothing and hold zeros: a load costs the memory pipeline by its
   // active lanes, and with few rows most of a block's lanes are such.
   const bf16_t* a_row[MB];
@@ -95,8 +105,8 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       const int step = ks + u * NW;
       const bool valid = step < full_steps;
       const int k = min(step, full_steps - 1) * 32;
-      wf[u][0] = load8(w0 + k, valid);
-      if (GATED) wf[u][SETS - 1] = load8(w1 + k, valid);
+#pragma unroll
+      for (int s = 0; s < SETS; ++s) wf[u][s] = load8(wp[s] + k, valid);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) af[u][mb] = load8(a_row[mb] + k, valid && a_ok[mb]);
     }
@@ -113,22 +123,27 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     // instruction sits behind a condition on the wave (it would run whatever a lane mask says).
     const int k = full_steps * 32;
     const bool k_ok = wave == full_steps % NW && k + 8 * g < K;
-    const bf16x8 wf0 = load8(w0 + k, k_ok);
-    bf16x8 wf1;
-    if (GATED) wf1 = load8(w1 + k, k_ok);
+    bf16x8 wt[SETS];
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) wt[s] = load8(wp[s] + k, k_ok);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const bf16x8 af = load8(a_row[mb] + k, k_ok && a_ok[mb]);
-      acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, af, acc[0][mb], 0, 0, 0);
-      if (GATED) acc[SETS - 1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, af, acc[SETS - 1][mb], 0, 0, 0);
+#pragma unroll
+      for (int s = 0; s < SETS; ++s) acc[s][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt[s], af, acc[s][mb], 0, 0, 0);
     }
   }
+  // One column block at a time through LDS (both halves of it), so that more blocks need no more LDS.
 #pragma unroll
-  for (int s = 0; s < SETS; ++s)
+  for (int b = 0; b < NB; ++b) {
+  const int n0 = n_first + 16 * b;
+  if (b > 0) __syncthreads();                                   // the block before has been read
+#pragma unroll
+  for (int h = 0; h < HALVES; ++h)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave][(s * MB + mb) * 4 + r][lane] = acc[s][mb][r];
+      for (int r = 0; r < 4; ++r) red[wave][(h * MB + mb) * 4 + r][lane] = acc[h * NB + b][mb][r];
   __syncthreads();
   // Lane (col, g) of block mb holds C^T rows n0 + 4g + r (r = 0..3), column m = mb*16 + col.
   for (int item = threadIdx.x; item < MB * WAVE; item += NW * WAVE) {
@@ -200,21 +215,29 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         if (n + r < n_out) store1(dst + r, v[r]);
     }
   }
+  }
 }
 
-template <int MB, int NW, bool GATED>
+// Column blocks per workgroup, by the launcher's choice (`asked` 0) or the caller's (1 or 2): two once there are
+// more than 32 rows and the workgroups still fill the device.
+static int column_blocks(int asked, int M, int n_out, int splits) {
+  if (asked == 1 || asked == 2) return asked;
+  return (M > 32 && (long)((n_out + 31) / 32) * splits >= 128) ? 2 : 1;
+}
+
+template <int MB, int NW, bool GATED, int NB = 1>
 static int launch_skinny(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
                          int K, int out_dtype, hipStream_t stream, int splits = 1, void* partial = nullptr) {
   const int n_out = GATED ? N / 2 : N;
   const int k_chunk = splits > 1 ? ((K + splits - 1) / splits + 31) / 32 * 32 : K;
   if (splits > 1) splits = (K + k_chunk - 1) / k_chunk;          // no part without a step of its own
-  const dim3 grid((n_out + 15) / 16, splits);
+  const dim3 grid((n_out + 16 * NB - 1) / (16 * NB), splits);
   float* slabs = splits > 1 ? (float*)partial : nullptr;
   if (out_dtype == DT_F32)
-    skinny_gemm_kernel<MB, NW, GATED, float><<<grid, NW * WAVE, 0, stream>>>(
+    skinny_gemm_kernel<MB, NW, GATED, float, false, NB><<<grid, NW * WAVE, 0, stream>>>(
         (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (float*)C, ldc, M, N, K, k_chunk, slabs);
   else
-    skinny_gemm_kernel<MB, NW, GATED, bf16_t><<<grid, NW * WAVE, 0, stream>>>(
+    skinny_gemm_kernel<MB, NW, GATED, bf16_t, false, NB><<<grid, NW * WAVE, 0, stream>>>(
         (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)C, ldc, M, N, K, k_chunk, slabs);
   int status = LAUNCH_STATUS();
   if (status == 0 && splits > 1 && C) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
@@ -223,7 +246,11 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
 
 template <int MB, bool GATED>
 static int pick_waves(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
-                      int K, int out_dtype, hipStream_t stream) {
+                      int K, int out_dtype, hipStream_t stream, int col_blocks = 0) {
+  if constexpr (MB >= 3) {
+    if (column_blocks(col_blocks, M, GATED ? N / 2 : N, 1) == 2)
+      return launch_skinny<MB, 8, GATED, 2>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+  }
   // Few output tiles and a long K: more waves per tile, so that enough loads are in flight.
   const int tiles = ((GATED ? N / 2 : N) + 15) / 16;
   const int k_steps = (K + 31) / 32;
@@ -235,13 +262,14 @@ static int pick_waves(const void* A, int lda, const void* W, const void* bias, v
 }
 
 // M <= 64; K, lda multiples of 8; pointers 16-byte aligned; with `gated` N is even and C is [M, N/2].
+// col_blocks: blocks of sixteen output columns per workgroup, 0 = the launcher's choice (see column_blocks).
 extern "C" int ta_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* bias, void* C, int ldc,
-                                   int M, int N, int K, int out_dtype, int gated, hipStream_t stream) {
+                                   int M, int N, int K, int out_dtype, int gated, int col_blocks, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 7) || (lda & 7) || (gated && (N & 1))) return -1;
   const int mb = (M + 15) / 16;
-#define GO(MBV) (gated ? pick_waves<MBV, true>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream) \
-                       : pick_waves<MBV, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream))
+#define GO(MBV) (gated ? pick_waves<MBV, true>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, col_blocks) \
+                       : pick_waves<MBV, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, col_blocks))
   switch (mb) {
     case 1: return GO(1);
     case 2: return GO(2);
@@ -257,16 +285,17 @@ extern "C" int ta_gemm_skinny_bf16(const void* A, int lda, const void* W, const 
 // left in `partial` for a later kernel to add.
 extern "C" int ta_gemm_skinny_bf16_splitk(const void* A, int lda, const void* W, const void* bias, void* C, int ldc,
                                           void* partial, int M, int N, int K, int out_dtype, int splits,
-                                          hipStream_t stream) {
+                                          int col_blocks, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 7) || (lda & 7) || (N & 3) || splits < 1 || (splits > 1 && !partial)) return -1;
   if (!C && parts_of_k(K, splits, 32) < 2) return -1;
-#define GO(MBV) launch_skinny<MBV, 8, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, splits, partial)
+#define GO(MBV, NBV) launch_skinny<MBV, 8, false, NBV>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, splits, partial)
+  const bool two = column_blocks(col_blocks, M, N, parts_of_k(K, splits, 32)) == 2;
   switch ((M + 15) / 16) {
-    case 1: return GO(1);
-    case 2: return GO(2);
-    case 3: return GO(3);
-    default: return GO(4);
+    case 1: return GO(1, 1);
+    case 2: return GO(2, 1);
+    case 3: return two ? GO(3, 2) : GO(3, 1);
+    default: return two ? GO(4, 2) : GO(4, 1);
   }
 #undef GO
 }

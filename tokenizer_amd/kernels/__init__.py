@@ -353,7 +353,7 @@ class Ops:
                 partial = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
                 self._check(self.lib.ta_gemm_skinny_bf16_splitk(
                     _ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(None if leave else out), n, _ptr(partial), m, n, k,
-                    _code(out_dtype), streaming_splits, self._stream()), "linear")
+                    _code(out_dtype), streaming_splits, self.skinny_column_blocks, self._stream()), "linear")
                 return PendingSum(self, partial, bias, out_dtype) if leave else out
             splits = self._k_splits(m, n, k)
             if splits > 1:
@@ -396,7 +396,7 @@ class Ops:
                     return out
             if m <= self.FUSED_ROWS or (m <= self.SKINNY_ROWS and n < self.WIDE_OUTPUT):
                 status = self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(out), n, m, n, k,
-                                                      _code(out_dtype), 0, self._stream())
+                                                      _code(out_dtype), 0, self.skinny_column_blocks, self._stream())
             else:
                 status = self.lib.ta_gemm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), m, n, k, lda, n,
                                                _code(out_dtype), self._stream())
@@ -404,6 +404,7 @@ class Ops:
         return out
 
     use_split_k = True
+    skinny_column_blocks = 0   # blocks of sixteen output columns per workgroup of the weight-streaming kernel: 0 = its choice
 
     def _k_splits(self, m: int, n: int, k: int) -> int:
         """Into how many parts the tiled kernel cuts K: more than one for 17 to 64 rows with a K so long, and so
@@ -433,6 +434,8 @@ class Ops:
         tiles = -(-n // 16)
         if tiles >= 128:
             return 1
+        if m > 32:
+            tiles = -(-n // 32)        # more than 32 rows: a workgroup takes two blocks of sixteen columns
         return max(1, min(-(-256 // tiles), k // part))
 
     PENDING_SHORTEST_K = 512   # the shortest K that is cut when the parts may be left for the next norm
@@ -466,7 +469,8 @@ class Ops:
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
             self._check(self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), None, _ptr(out), inner, m, 2 * inner,
-                                                     k, _BF16, 1, self._stream()), "linear_silu_gate")
+                                                     k, _BF16, 1, self.skinny_column_blocks, self._stream()),
+                        "linear_silu_gate")
             return out
         return self.silu_gate(self.linear(x, weight), out)
 
