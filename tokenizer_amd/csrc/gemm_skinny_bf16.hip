@@ -251,6 +251,12 @@ static int pick_waves(const void* A, int lda, const void* W, const void* bias, v
     if (column_blocks(col_blocks, M, GATED ? N / 2 : N, 1) == 2)
       return launch_skinny<MB, 8, GATED, 2>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
   }
+  if constexpr (MB == 1 && !GATED) {
+    // Up to sixteen rows against tens of thousands of output columns (the vocabulary projection of a decode
+    // step): four column blocks per workgroup, or a quarter of the workgroups would each read all the rows again.
+    if ((col_blocks == 0 || col_blocks == 4) && (N + 15) / 16 >= 4096 && K <= 8192)
+      return launch_skinny<1, 4, false, 4>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+  }
   // Few output tiles and a long K: more waves per tile, so that enough loads are in flight.
   const int tiles = ((GATED ? N / 2 : N) + 15) / 16;
   const int k_steps = (K + 31) / 32;
