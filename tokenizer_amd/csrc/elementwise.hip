@@ -113,10 +113,18 @@ splitk_add_rmsnorm_kernel(float* __restrict__ residual, const float* __restrict_
     const int h = (c * 256 + threadIdx.x) * 4;
     x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (h < hidden) {
+      // Eight slabs are asked for at a time (a product cut into twenty parts is twenty trips otherwise); they are
+      // added in their order all the same.
       float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-      for (int s = 0; s < splits; ++s) {
-        const float4 v = ld4(partial + ((size_t)s * n_rows + i) * hidden + h);
-        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+      const float* slab = partial + (size_t)i * hidden + h;
+      const size_t slab_stride = (size_t)n_rows * hidden;
+      for (int s0 = 0; s0 < splits; s0 += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          v[j] = s0 + j < splits ? ld4(slab + (size_t)(s0 + j) * slab_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { sum.x += v[j].x; sum.y += v[j].y; sum.z += v[j].z; sum.w += v[j].w; }
       }
       if (bias) {
         const float4 b = ld4(bias + h);
