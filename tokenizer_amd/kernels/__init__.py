@@ -81,8 +81,12 @@ class Ops:
         self.path = path
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
-                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16", "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16", "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope", "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated", "ta_splitk_reduce", "ta_splitk_add_rmsnorm",
-                     "ta_argmax", "ta_sample", "ta_sample_workspace_words", "ta_library_gemm_bf16"):
+                     "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16",
+                     "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16",
+                     "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
+                     "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
+                     "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_sample",
+                     "ta_sample_workspace_words", "ta_library_gemm_bf16"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
@@ -603,7 +607,6 @@ class Ops:
         self._check(self.lib.ta_argmax(_ptr(logits), _ptr(out), _ptr(partial_v), _ptr(partial_i), n_rows, vocab,
                                        chunks, self._stream()), "argmax")
         return out
-
 
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniform: torch.Tensor,
                out: torch.Tensor | None = None, any_cut: bool = True) -> torch.Tensor:
