@@ -429,8 +429,9 @@ static int rows_per_workgroup(int n_rows, int rows_override) {
 }
 
 // Rows that are normalised already go through LDS (the NORM instances, which then copy instead of normalising)
-// while two workgroups' copies fit a compute unit beside their other LDS.
-static bool stage_rows(int m, int k) { return (size_t)m * (k + 8) * sizeof(uint16_t) <= 60 * 1024; }
+// while a workgroup's copy fits a compute unit beside its other LDS (measured at a width of 3,584: 1.06x for 8
+// rows, where two workgroups' copies fit, level for 12, 1.02x for 16).
+static bool stage_rows(int m, int k) { return (size_t)m * (k + 8) * sizeof(uint16_t) <= 120 * 1024; }
 
 static int fused_qkv_rope(const FusedArgs& base, bool norm, const void* w, const void* bias, void* q_out,
                           const void* positions, const void* cos_sin, const void* slots, void* k_pages, void* v_pages,
