@@ -181,14 +181,19 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     for (int db = 0; db < DB; ++db) acc[h][db] = (floatx4){0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int kb = (lo / 64) * 64 + 64 * wave; kb <= hi; kb += 64 * NWV) {
-    if (kb >= lo_all && kb + 63 <= p0)
-      prefill_block<D, HG, true>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                 my_lo, lo, hi, scale_log2, qf, acc, m, l);
-    else
-      prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                  my_lo, lo, hi, scale_log2, qf, acc, m, l);
-  }
+  // A wave's blocks come in three runs: those at the window's edge (some keys masked), those that every token
+  // of the tile sees whole, and those on the diagonal.  Each run is a loop of its own over one variant of the
+  // block: in one loop over both, the accumulators would be copied between the variants' registers every turn.
+  int kb = (lo / 64) * 64 + 64 * wave;
+  for (; kb <= hi && kb < lo_all; kb += 64 * NWV)
+    prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l);
+  for (; kb + 63 <= p0; kb += 64 * NWV)
+    prefill_block<D, HG, true>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                               my_lo, lo, hi, scale_log2, qf, acc, m, l);
+  for (; kb <= hi; kb += 64 * NWV)
+    prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l);
   if (NWV > 1) {
     // Waves 1.. hand their state to wave 0: maximum, sum and the output accumulators of each head.
     if (wave > 0) {
