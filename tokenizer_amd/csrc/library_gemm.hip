@@ -41,10 +41,9 @@ std::mutex guard;
 std::unordered_map<int, hipblasLtHandle_t> handles;       // one per device
 std::unordered_map<Shape, Plan, ShapeHash> plans;
 bool tuning = true;
-// Multiply-adds from which the candidates are timed.  The timing sees launches from the host, one after the
-// other: a product that is over on the device before the host has launched the next one (some 15 us) would be
-// judged by the host's pace and not by its own.
-constexpr double TUNE_FROM_WORK = 4294967296.0;
+// Multiply-adds from which the candidates are timed (a small product keeps the first choice: timed on operands
+// that sit in the caches it would be misjudged).
+constexpr double TUNE_FROM_WORK = 1073741824.0;
 constexpr int TUNE_AFTER_CALLS = 64;                      // ... unasked, once a shape has come up this often
 
 // The operands of the call that makes a plan: what the candidates are timed on.
@@ -53,21 +52,27 @@ struct Operands {
   void* workspace; size_t workspace_bytes; hipStream_t stream;
 };
 
-// Milliseconds of `runs` products with this algorithm after one that warms it up; negative if it fails.
+// Milliseconds of one product with this algorithm, the best of `runs`, each with cold caches: before every run
+// `flush` (more bytes than the caches hold) is overwritten, which also keeps the device busy long enough for the
+// host to have the product queued behind it, so that the two events bracket the product's own time on the device.
+// In a model's step the weights of a product come from memory, not from the caches: candidates timed on operands
+// that stay in the caches rank differently, and wrongly.  Negative if anything fails.
 float time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo, const Operands& o,
-                hipEvent_t start, hipEvent_t stop, int runs) {
+                void* flush, size_t flush_bytes, hipEvent_t start, hipEvent_t stop, int runs) {
   const float one = 1.f, zero = 0.f;
-  for (int i = 0; i <= runs; ++i) {
-    if (i == 1 && hipEventRecord(start, o.stream) != hipSuccess) return -1.f;
-    if (hipblasLtMatmul(handle, p.desc, &one, o.w, p.w, o.a, p.x, &zero, o.c, p.c, o.c, p.c, &algo, o.workspace,
-                        o.workspace_bytes, o.stream) != HIPBLAS_STATUS_SUCCESS)
+  float best = -1.f;
+  for (int i = 0; i < runs; ++i) {
+    float ms = -1.f;
+    if (hipMemsetAsync(flush, i, flush_bytes, o.stream) != hipSuccess ||
+        hipEventRecord(start, o.stream) != hipSuccess ||
+        hipblasLtMatmul(handle, p.desc, &one, o.w, p.w, o.a, p.x, &zero, o.c, p.c, o.c, p.c, &algo, o.workspace,
+                        o.workspace_bytes, o.stream) != HIPBLAS_STATUS_SUCCESS ||
+        hipEventRecord(stop, o.stream) != hipSuccess || hipEventSynchronize(stop) != hipSuccess ||
+        hipEventElapsedTime(&ms, start, stop) != hipSuccess)
       return -1.f;
+    if (best < 0.f || ms < best) best = ms;
   }
-  float ms = -1.f;
-  if (hipEventRecord(stop, o.stream) != hipSuccess || hipEventSynchronize(stop) != hipSuccess ||
-      hipEventElapsedTime(&ms, start, stop) != hipSuccess)
-    return -1.f;
-  return ms;
+  return best;
 }
 
 // Row-major C = A W^T is, in the library's column-major terms, C^T [N x M] = op(W) [N x K] * A^T [K x M]:
@@ -105,10 +110,11 @@ Plan make_plan(hipblasLtHandle_t handle, const Shape& s, size_t workspace_bytes)
     if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes)
       p.candidates.push_back(found[i]);
   p.usable = !p.candidates.empty();
-  // Small products keep the first choice: timed on operands that sit in the caches they would be misjudged.
   p.tuned = !tuning || p.candidates.size() < 2 || (double)s.m * s.n * s.k < TUNE_FROM_WORK;
   return p;
 }
+
+constexpr size_t FLUSH_BYTES = (size_t)384 << 20;        // more than the last-level caches hold together
 
 // Time every candidate on these operands (the result they leave is the product all the same) and keep the
 // fastest.  Not while the stream records a graph: the plan then stays as it is until a later call.
@@ -116,16 +122,21 @@ void tune_plan(hipblasLtHandle_t handle, Plan& p, const Operands& o) {
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(o.stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return;
   p.tuned = true;
+  void* flush = nullptr;
   hipEvent_t start = nullptr, stop = nullptr;
-  if (hipEventCreate(&start) == hipSuccess && hipEventCreate(&stop) == hipSuccess) {
+  if (hipMalloc(&flush, FLUSH_BYTES) == hipSuccess && hipEventCreate(&start) == hipSuccess &&
+      hipEventCreate(&stop) == hipSuccess) {
     float best_ms = -1.f;
     for (size_t i = 0; i < p.candidates.size(); ++i) {
-      const float ms = time_algo(handle, p, p.candidates[i].algo, o, start, stop, 5);
+      const float ms = time_algo(handle, p, p.candidates[i].algo, o, flush, FLUSH_BYTES, start, stop, 3);
       if (ms >= 0.f && (best_ms < 0.f || ms < best_ms)) { best_ms = ms; p.chosen = i; }
     }
+    hipStreamSynchronize(o.stream);
   }
   if (start) hipEventDestroy(start);
   if (stop) hipEventDestroy(stop);
+  if (flush) hipFree(flush);
+  (void)hipGetLastError();                                  // a failed allocation leaves no error behind
 }
 
 }  // namespace
