@@ -3,8 +3,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--dtype bfloat16]
 
 A step is one decode step of the whole batch.  The default run prefills 8 prompts of 2,048
-random ids and decodes from there; it also times a prefill of 2,048 tokens and decoding at
-batch 1 and 64, and prints one JSON line.
+random ids and decodes every request on to 4,096 tokens (8 warm-up steps, 2,040 timed ones); it
+also times a prefill of 2,048 tokens and the same decoding at batch 1 and 64, and prints one
+JSON line.
 
     python bench.py --workload mixed-1.5b | prefix-7b
 
@@ -84,36 +85,47 @@ def make_prompts(batch: int, vocab: int, seed: int):
 
 
 def run_decode(model, batch: int, steps: int, warmup: int):
-    """Prefill `batch` prompts, then time `steps` decode steps (greedy, ids picked on the device)."""
+    """Prefill `batch` prompts, then time `steps` decode steps (greedy, ids picked on the device).  When the
+    timed steps reach into further 512-token ranges of context than the warm-up did, the whole run is done once
+    untimed before: a range's first step records its graph, which is set-up, not a decode step."""
     import torch
     from tokenizer_amd.engine import Engine, StepEntry
 
     page_size = 16
-    engine = Engine(model, num_pages=batch * (CONTEXT_LEN // page_size) + 8, page_size=page_size, max_requests=batch)
+    longest = PROMPT_LEN + warmup + steps
+    pages_each = -(-max(CONTEXT_LEN, longest) // page_size)
+    engine = Engine(model, num_pages=batch * pages_each + 8, page_size=page_size, max_requests=batch)
     prompts = make_prompts(batch, model.vocab_size, seed=1)
-    last = []
-    for rid, prompt in enumerate(prompts):
-        engine.add_request(rid)
-        for at in range(0, len(prompt), 2048):                  # long prompts in portions
-            portion = prompt[at:at + 2048]
-            logits = engine.step([StepEntry(rid, portion, [len(portion) - 1] if at + 2048 >= len(prompt) else [])])
-        last.append(engine.argmax(logits)[0])
-
-    # Greedy decode steps back to back: each step's ids feed the next on the device and reach the host one
-    # step late (`Engine.decode_greedy`), so the host's work on a step hides behind the device's.
     rids = list(range(batch))
-    if warmup:
-        last = engine.decode_greedy(rids, last, warmup)[-1]
-    torch.cuda.synchronize()
-    kv_start = engine.cache.seq_len(0)
-    started = time.perf_counter()
-    picked = engine.decode_greedy(rids, last, steps)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - started
-    assert len(picked) == steps and all(len(ids) == batch for ids in picked)
+
+    def one_pass():
+        last = []
+        for rid, prompt in enumerate(prompts):
+            engine.add_request(rid)
+            for at in range(0, len(prompt), 2048):                  # long prompts in portions
+                portion = prompt[at:at + 2048]
+                logits = engine.step([StepEntry(rid, portion, [len(portion) - 1] if at + 2048 >= len(prompt) else [])])
+            last.append(engine.argmax(logits)[0])
+        # Greedy decode steps back to back: each step's ids feed the next on the device and reach the host one
+        # step late (`Engine.decode_greedy`), so the host's work on a step hides behind the device's.
+        if warmup:
+            last = engine.decode_greedy(rids, last, warmup)[-1]
+        torch.cuda.synchronize()
+        kv_start = engine.cache.seq_len(0)
+        started = time.perf_counter()
+        picked = engine.decode_greedy(rids, last, steps)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        assert len(picked) == steps and all(len(ids) == batch for ids in picked)
+        for rid in rids:
+            engine.end_request(rid)
+        return elapsed, kv_start
+
+    bucket = engine.GRAPH_BUCKET
+    if engine.use_graphs and -(-longest // bucket) > -(-(PROMPT_LEN + warmup + 1) // bucket):
+        one_pass()
+    elapsed, kv_start = one_pass()
     kv_mean = kv_start + (steps - 1) / 2 + 1          # keys each step reads, averaged over the timed steps
-    for rid in range(batch):
-        engine.end_request(rid)
     del engine
     torch.cuda.empty_cache()
     return elapsed, kv_mean
@@ -230,7 +242,9 @@ def measure_peaks() -> dict:
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=128)
+    parser.add_argument("--steps", type=int, default=None,
+                        help="timed decode steps (default: from the prompt's end to the context the record names, "
+                             "2,048 -> 4,096 tokens per request)")
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
@@ -248,10 +262,14 @@ def main() -> int:
                         help="tokens of every prompt before decoding (default 2,048, the record's; the context the "
                              "record names is then twice that, else the prompt plus the decoded tokens)")
     args = parser.parse_args()
+    global PROMPT_LEN, CONTEXT_LEN
     if args.prompt_len:
-        global PROMPT_LEN, CONTEXT_LEN
         PROMPT_LEN = args.prompt_len
+        if args.steps is None:
+            args.steps = 128
         CONTEXT_LEN = -(-(args.prompt_len + args.warmup + max(args.steps, 64) + 1) // 16) * 16
+    if args.steps is None:
+        args.steps = CONTEXT_LEN - PROMPT_LEN - args.warmup
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; runs with --gpus > 1 are not supported")
         return 2
@@ -297,7 +315,8 @@ def main() -> int:
                    "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied_head": cfg.tie_word_embeddings, "global_batch": args.batch, "prompt_len": PROMPT_LEN,
-                   "seq_len": CONTEXT_LEN, "page_size": 16, "parallelism": "single-gpu"},
+                   "seq_len": CONTEXT_LEN, "decoded_to": PROMPT_LEN + args.warmup + args.steps, "page_size": 16,
+                   "parallelism": "single-gpu"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
     }
@@ -308,7 +327,7 @@ def main() -> int:
         record["prefill"] = {"value": round(PROMPT_LEN / seconds, 1), "tokens": PROMPT_LEN, "ms": round(seconds * 1e3, 3),
                              "frac": round(flops / seconds / (PEAK_TFLOPS[args.dtype] * 1e12), 5)}
         points = {}
-        for batch, steps in ((1, args.steps), (64, max(16, args.steps // 4))):
+        for batch, steps in ((1, args.steps), (64, args.steps)):
             log(f"decode at batch {batch}: {steps} timed steps")
             e, _ = run_decode(model, batch, steps, min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(batch * steps / e, 1)
