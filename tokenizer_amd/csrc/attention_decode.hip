@@ -70,23 +70,26 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   for (int db = 0; db < DB; ++db) acc[db] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  for (int kb = first + wave * 32; kb <= last; kb += DEC_WAVES * 32) {
-    // All loads of the block are issued first: keys, and values (whose addresses do not wait for the scores).
+  // A block of 32 keys (two tiles of 16, each inside one page) as the matrix instructions want it.
+  struct KeyBlock {
     bf16x8 kf[2][KS];
     union VFrag { uint2 half[2]; bf16x8 v; } vf[DB];
     bool active[2];
+  };
+  // All loads of a block are issued together: keys, and values (whose addresses do not wait for the scores).
+  auto load_block = [&](KeyBlock& blk, int kb) {
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile) {
       const int k0 = kb + tile * 16;                       // 16 keys of one page
-      active[tile] = (k0 <= last) && (k0 + 15 >= lo);
-      if (active[tile]) {
+      blk.active[tile] = (k0 <= last) && (k0 + 15 >= lo);
+      if (blk.active[tile]) {
         const int page = table[k0 / page_size];
         const size_t base = ((size_t)page * n_kv + kvh) * page_size * D;   // same element count for K and V^T pages
         const bf16_t* kr = k_pages + base + (size_t)((k0 % page_size) + col) * D + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          if (ks * 32 + 8 * g < D) kf[tile][ks] = *reinterpret_cast<const bf16x8*>(kr + ks * 32);
-          else kf[tile][ks] = zero8();
+          if (ks * 32 + 8 * g < D) blk.kf[tile][ks] = *reinterpret_cast<const bf16x8*>(kr + ks * 32);
+          else blk.kf[tile][ks] = zero8();
         }
         const bf16_t* vr = vt_pages + base + (size_t)col * page_size + (k0 % page_size) + 4 * g;
         const int left = last - (k0 + 4 * g);              // keys of this lane that exist: 0..left
@@ -97,26 +100,29 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
             if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
             if (left < 2) v.y = 0; else v.y &= 0xffffu;
           }
-          vf[db].half[tile] = v;
+          blk.vf[db].half[tile] = v;
         }
       } else {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kf[tile][ks] = zero8();
+        for (int ks = 0; ks < KS; ++ks) blk.kf[tile][ks] = zero8();
 #pragma unroll
-        for (int db = 0; db < DB; ++db) vf[db].half[tile] = make_uint2(0, 0);
+        for (int db = 0; db < DB; ++db) blk.vf[db].half[tile] = make_uint2(0, 0);
       }
     }
+  };
+  // One step of the online softmax over a block that has been brought in.
+  auto attend = [&](const KeyBlock& blk, int kb) {
     float s[2][4];
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile) {
       floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
-        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tile][ks], qf[ks], st, 0, 0, 0);
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[tile][ks], qf[ks], st, 0, 0, 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = kb + tile * 16 + 4 * g + r;
-        s[tile][r] = (active[tile] && key >= lo && key <= last) ? st[r] * scale : -INFINITY;
+        s[tile][r] = (blk.active[tile] && key >= lo && key <= last) ? st[r] * scale : -INFINITY;
       }
     }
     float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
@@ -124,7 +130,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(m, mx);
-    if (__all(m_new == -INFINITY)) continue;               // nothing visible yet: the same for every head, a scalar branch
+    if (__all(m_new == -INFINITY)) return;                 // nothing visible yet: the same for every head, a scalar branch
     const float corr = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
     bf16x8 pf;
     float psum = 0.f;
@@ -142,7 +148,27 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     for (int db = 0; db < DB; ++db) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[db][r] *= corr;
-      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db].v, pf, acc[db], 0, 0, 0);
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[db].v, pf, acc[db], 0, 0, 0);
+    }
+  };
+  // Two blocks in turn: while one is worked on, the next one's keys and values are on their way (a wave that
+  // asked for them only when it got there would wait a trip to memory in every block).
+  constexpr int STRIDE = DEC_WAVES * 32;
+  int kb = first + wave * 32;
+  if (kb <= last) {
+    KeyBlock one, two;
+    load_block(one, kb);
+    while (true) {
+      const bool more = kb + STRIDE <= last;
+      if (more) load_block(two, kb + STRIDE);
+      attend(one, kb);
+      kb += STRIDE;
+      if (!more) break;
+      const bool further = kb + STRIDE <= last;
+      if (further) load_block(one, kb + STRIDE);
+      attend(two, kb);
+      kb += STRIDE;
+      if (!further) break;
     }
   }
   // Sum of the lane groups' partial denominators (the maximum is already common to them).
