@@ -67,6 +67,9 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int n_first = ROPE ? rope_head * rope.d + rope_first : blockIdx.x * 16 * NB;
   const int k_lo = blockIdx.y * k_chunk;
   const int K = min(K_all, k_lo + k_chunk) - k_lo;                // this workgroup's part of K
+  // grid.z: the rows in shares of MB blocks of sixteen (one share unless the launcher cut them: a small matrix
+  // whose tiles would not fill the device otherwise; the weights are then read once per share).
+  const int m_base = blockIdx.z * (MB * 16);
   // Rows past the end are clamped, not masked: they only feed outputs that are never stored.
   // The second half: the `up` rows when GATED, the rows half a head further on with ROPE.
   const bf16_t* wp[SETS];
@@ -83,8 +86,8 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   bool a_ok[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    a_ok[mb] = mb * 16 + col < M;
-    a_row[mb] = A + (size_t)min(mb * 16 + col, M - 1) * lda + k_lo + 8 * g;
+    a_ok[mb] = m_base + mb * 16 + col < M;
+    a_row[mb] = A + (size_t)min(m_base + mb * 16 + col, M - 1) * lda + k_lo + 8 * g;
   }
 
   floatx4 acc[SETS][MB];
@@ -148,7 +151,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   // Lane (col, g) of block mb holds C^T rows n0 + 4g + r (r = 0..3), column m = mb*16 + col.
   for (int item = threadIdx.x; item < MB * WAVE; item += NW * WAVE) {
     const int mb = item / WAVE, ln = item % WAVE;
-    const int m = mb * 16 + (ln & 15);
+    const int m = m_base + mb * 16 + (ln & 15);
     const int n = n0 + 4 * (ln >> 4);
     if (m >= M || n >= n_out) continue;
     float v[4], v2[4] = {0.f, 0.f, 0.f, 0.f};
@@ -322,10 +325,15 @@ extern "C" int ta_gemm_skinny_qkv_rope(const void* x, int lda, const void* W, co
   rope.k_pages = (bf16_t*)k_pages; rope.v_pages = (bf16_t*)v_pages;
   rope.n_q = n_q; rope.n_kv = n_kv; rope.d = d; rope.page_size = page_size;
   const int N = (n_q + 2 * n_kv) * d;
-  const dim3 grid((n_q + 2 * n_kv) * (d / 32), 1);
+  const int tiles = (n_q + 2 * n_kv) * (d / 32);
+  const int blocks = (M + 15) / 16;
+  // Few tiles (a small model's joined matrix is a few dozen): every block of sixteen rows gets workgroups of
+  // its own, which read the small matrix again and fill the device.
+  const int per_share = (blocks > 1 && tiles * blocks <= 512) ? 1 : blocks;
+  const dim3 grid(tiles, 1, (blocks + per_share - 1) / per_share);
 #define GO(MBV) skinny_gemm_kernel<MBV, 8, true, bf16_t, true><<<grid, 8 * WAVE, 0, stream>>>( \
     (const bf16_t*)x, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)q_out, n_q * d, M, N, K, K, nullptr, rope)
-  switch ((M + 15) / 16) {
+  switch (per_share) {
     case 1: GO(1); break;
     case 2: GO(2); break;
     case 3: GO(3); break;
