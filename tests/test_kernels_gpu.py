@@ -607,6 +607,18 @@ def test_weight_streaming_product_with_two_column_blocks(ops, ref, shape, monkey
     assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
 
 
+@pytest.mark.parametrize("shape", [(1, 151, 37), (3, 50, 1000), (16, 33, 130), (9, 1000, 896), (16, 4, 8)])
+def test_linear_float32_of_few_rows(ops, ref, shape):
+    # Up to sixteen float32 rows take the kernel that walks the weights once: widths that end inside a wave's four
+    # weight rows, K that is and is not a multiple of four, rows of A with a stride.
+    m, n, k = shape
+    wide = rand((m, k + 12), torch.float32, 41)
+    x, w, bias = wide[:, 4:4 + k], rand((n, k), torch.float32, 42, 0.1), rand((n,), torch.float32, 43)
+    want = (x.double() @ w.double().t() + bias.double()).float()
+    torch.testing.assert_close(ops.linear(x, w, bias), want, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(ops.linear(x.contiguous(), w), (x.double() @ w.double().t()).float(), rtol=1e-5, atol=1e-5)
+
+
 def test_linear_float32_is_true_float32(ops):
     # Inputs that need 13 mantissa bits: a reduced-precision matrix mode (10 or 7 bits) would be off by
     # about 1e-2 here, float32 accumulation by less than 3e-4.
