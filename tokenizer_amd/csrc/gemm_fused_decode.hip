@@ -424,7 +424,11 @@ static int rows_per_workgroup(int n_rows, int rows_override) {
   if (rows_override >= 1 && rows_override <= 32) return rows_override;
   const int units = compute_units();
   const int rounds = (n_rows + units * 32 - 1) / (units * 32);
-  const int rows = (n_rows + units * rounds - 1) / (units * rounds);
+  int rows = (n_rows + units * rounds - 1) / (units * rounds);
+  // One round of 17 to 31 rows would be a block of sixteen and a nearly empty second one, one after the other:
+  // two workgroups of half the rows on every compute unit, one block each, are over sooner (measured at 4,864
+  // rows of 896: 19 rows 8.6 us, 10 rows 8.2 us; with two rounds, 8,960 rows of 1,536, the halves are slower).
+  if (rounds == 1 && rows > 16 && rows < 32) rows = (n_rows + 2 * units - 1) / (2 * units);
   return rows < 4 ? 4 : rows;
 }
 
