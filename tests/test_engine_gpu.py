@@ -544,3 +544,22 @@ def test_the_whole_model_at_half_a_billion_parameters(tmp_path):
             for rid in reqs:
                 close(got[rid], want[rid], dtype)
             del eng
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [8, 32, 48])
+def test_other_page_sizes(model_folders, oracle, dtype, page_size):
+    # Pages of 32 and 48 tokens take the matrix-core attention kernels as pages of 16 do; pages of 8 (no multiple
+    # of a key tile) go to the generic kernel.  Mixed batches with reused pages, configuration C with its window.
+    for name in ("B", "C"):
+        reqs = requests_for(name)
+        steps = tt.mixed(reqs, 7)
+        live = tt.peak_tokens(steps)
+        eng = engine_for(model_folders[name], dtype, num_pages=-(-live // page_size) + 4, page_size=page_size,
+                         max_requests=4)
+        eng.pools.poison()
+        got = tt.run_in_process(eng, steps)
+        for rid, ids in reqs.items():
+            close(got[rid], oracle(name, ids), dtype)
+        eng.cache.check_invariants()
+        assert not eng.cache.requests
