@@ -563,3 +563,28 @@ def test_other_page_sizes(model_folders, oracle, dtype, page_size):
             close(got[rid], oracle(name, ids), dtype)
         eng.cache.check_invariants()
         assert not eng.cache.requests
+
+
+@pytest.mark.parametrize("size", ["inner100", "group18", "wide", "window_inner44"])
+def test_decode_batches_of_dozens_at_sizes_away_from_every_tile(tmp_path, size):
+    # Decode batches of 20 and 64 requests (the kernels for 17 to 64 rows: K cut over workgroups with the parts
+    # left to the norm, two column blocks, the rotation epilogue with the rows in shares) at odd sizes, two steps
+    # each, in bfloat16 and in 32-bit, against the plain implementation.
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import StepEntry
+    raw = dict(TINY["A"][0], max_position_embeddings=512, **ODD_SIZES[size])
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 17, str(tmp_path / size))
+    cfg, tensors = plain.load_folder(folder)
+    for dtype in ("bfloat16", "float32"):
+        for batch in (20, 64):
+            eng = engine_for(folder, dtype, max_tokens=64 * batch, max_requests=batch)
+            prompts = [random_ids(raw["vocab_size"], 3 + (7 * i) % 40, 200 + i) for i in range(batch)]
+            for rid, ids in enumerate(prompts):
+                eng.add_request(rid)
+                eng.step([StepEntry(rid, ids[:-1], [])])
+            for _ in range(2):
+                logits = eng.step([StepEntry(rid, ids[-1:], [0]) for rid, ids in enumerate(prompts)]).float().cpu()
+                for rid, ids in enumerate(prompts):
+                    close(logits[rid:rid + 1], plain.all_logits(cfg, tensors, ids)[-1:], dtype)
+                prompts = [ids + [int(logits[rid].argmax())] for rid, ids in enumerate(prompts)]
