@@ -44,22 +44,25 @@ def test_embedding(ops, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden", [200, 896, 72])
-def test_add_rmsnorm(ops, ref, dtype, hidden):
-    residual = rand((33, hidden), torch.float32, 2, 3.0)
-    delta = rand((33, hidden), dtype, 3)
+@pytest.mark.parametrize("hidden", [200, 896, 72, 2048, 4100])
+@pytest.mark.parametrize("n", [33, 301])
+def test_add_rmsnorm(ops, ref, dtype, hidden, n):
+    # (few and many rows; rows that fit the registers of a workgroup and rows that do not)
+    residual = rand((n, hidden), torch.float32, 2, 3.0)
+    delta = rand((n, hidden), dtype, 3)
     weight = rand((hidden,), torch.float32, 4) + 1
     for use_delta in (True, False):
         res_a, res_b = residual.clone(), residual.clone()
-        out_a = torch.empty((33, hidden), dtype=dtype).cuda()
+        out_a = torch.empty((n, hidden), dtype=dtype).cuda()
         out_b = torch.empty_like(out_a)
         ops.add_rmsnorm(res_a, delta if use_delta else None, weight, 1e-5, out_a)
         ref.add_rmsnorm(res_b, delta if use_delta else None, weight, 1e-5, out_b)
         torch.testing.assert_close(res_a, res_b, rtol=1e-6, atol=1e-6)
         torch.testing.assert_close(out_a.float(), out_b.float(), **tol(dtype))
-    rows = torch.tensor([32, 0, 7, 7], dtype=torch.int32).cuda()
+    picked = [n - 1, 0, 7, 7] if n < 256 else [n - 1, 0, 7, 7] + list(range(2, 2 + 256))
+    rows = torch.tensor(picked, dtype=torch.int32).cuda()
     res_a = residual.clone()
-    out_a = torch.empty((4, hidden), dtype=dtype).cuda()
+    out_a = torch.empty((len(picked), hidden), dtype=dtype).cuda()
     out_b = torch.empty_like(out_a)
     ops.add_rmsnorm(res_a, delta, weight, 1e-6, out_a, rows, store_residual=False)
     ref.add_rmsnorm(residual.clone(), delta, weight, 1e-6, out_b, rows, store_residual=False)
