@@ -20,6 +20,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   __shared__ float q_s[ATT_MAX_D];
   __shared__ float acc_s[ATT_WAVES][ATT_MAX_D];
   __shared__ float m_s[ATT_WAVES], l_s[ATT_WAVES];
+  __shared__ float p_s[ATT_WAVES][WAVE];
   const int t = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
   const int pos = positions[t];
@@ -45,7 +46,15 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
       vbase = (page * n_kv + kvh) * page_size * d + (j % page_size);
       const T* kr = k_pages + (size_t)row * d;
       float dot = 0.f;
-      for (int i = 0; i < d; ++i) dot += q_s[i] * ld(kr + i);
+      if (sizeof(T) == 4 && d % 4 == 0) {
+        // A lane walks its key's row sixteen bytes at a time (rows are 16-byte aligned: d is a multiple of 4).
+        for (int i = 0; i < d; i += 4) {
+          const float4 kv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(kr) + i);
+          dot = fmaf(q_s[i], kv.x, fmaf(q_s[i + 1], kv.y, fmaf(q_s[i + 2], kv.z, fmaf(q_s[i + 3], kv.w, dot))));
+        }
+      } else {
+        for (int i = 0; i < d; ++i) dot += q_s[i] * ld(kr + i);
+      }
       s = dot * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -55,13 +64,53 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
 #pragma unroll
     for (int r = 0; r < ATT_MAX_D / WAVE; ++r) acc[r] *= corr;
     const int count = min(WAVE, n_keys - base);
-    for (int jj = 0; jj < count; ++jj) {
-      const float pj = __shfl(p, jj, WAVE);
-      const T* vr = v_pages + (size_t)__shfl(vbase, jj, WAVE);
+    if (sizeof(T) == 4 && page_size % 4 == 0) {
+      // Values lie transposed inside a page, [d, page_size]: lane i walks row i of the page sixteen bytes (four
+      // keys) at a time, so that the wave reads the page as one contiguous block; the keys' weights come through
+      // LDS.  (One key at a time, every lane's element would lie a row apart from its neighbour's.)
+      p_s[wave][lane] = p;
+      __builtin_amdgcn_wave_barrier();
+      int jj = 0;
+      while (jj < count) {
+        const int j = lo + base + jj;
+        const int off = j % page_size;
+        const int run = min(count - jj, page_size - off);
+        const float* page_v = reinterpret_cast<const float*>(v_pages) +
+                              ((size_t)table[j / page_size] * n_kv + kvh) * d * page_size + off;
+        if (off % 4 == 0 && run >= 4) {
+          for (int q4 = 0; q4 + 4 <= run; q4 += 4) {
+            const float p0 = p_s[wave][jj + q4], p1 = p_s[wave][jj + q4 + 1], p2 = p_s[wave][jj + q4 + 2],
+                        p3 = p_s[wave][jj + q4 + 3];
 #pragma unroll
-      for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
-        const int i = lane + r * WAVE;
-        if (i < d) acc[r] += pj * ld(vr + (size_t)i * page_size);
+            for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
+              const int i = lane + r * WAVE;
+              if (i < d) {
+                const float4 v4 = *reinterpret_cast<const float4*>(page_v + (size_t)i * page_size + q4);
+                acc[r] = fmaf(p0, v4.x, fmaf(p1, v4.y, fmaf(p2, v4.z, fmaf(p3, v4.w, acc[r]))));
+              }
+            }
+          }
+          jj += run / 4 * 4;
+        } else {
+          const float pj = p_s[wave][jj];
+#pragma unroll
+          for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
+            const int i = lane + r * WAVE;
+            if (i < d) acc[r] += pj * page_v[(size_t)i * page_size];
+          }
+          ++jj;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    } else {
+      for (int jj = 0; jj < count; ++jj) {
+        const float pj = __shfl(p, jj, WAVE);
+        const T* vr = v_pages + (size_t)__shfl(vbase, jj, WAVE);
+#pragma unroll
+        for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
+          const int i = lane + r * WAVE;
+          if (i < d) acc[r] += pj * ld(vr + (size_t)i * page_size);
+        }
       }
     }
     m = m_new;
