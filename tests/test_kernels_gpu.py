@@ -278,9 +278,13 @@ def test_prefill_attention_with_all_heads_of_a_group_in_one_wave(ops, ref, geome
     torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("target", [1024, 16])
 @pytest.mark.parametrize("window", [None, 1000])
-def test_decode_attention_long_contexts_and_many_splits(ops, ref, window):
-    # Batches of single tokens at long, unequal contexts: the key range is cut into many splits.
+def test_decode_attention_long_contexts_and_many_splits(ops, ref, window, target, monkeypatch):
+    # Batches of single tokens at long, unequal contexts: the key range is cut into many splits (a wave has a few
+    # blocks and asks for the next one ahead), or, aiming at few workgroups, into one or two long ones (a wave
+    # walks dozens of blocks one after the other).
+    monkeypatch.setattr(ops, "target_workgroups", target)
     n_q, n_kv, d, page_size = 14, 2, 64, 16
     for lengths in ([3000], [2049, 1, 777, 4096, 31, 32, 33, 2500]):
         qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(

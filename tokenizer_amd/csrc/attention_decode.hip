@@ -26,7 +26,8 @@ __device__ __forceinline__ bf16x8 zero8() {
 // Token at position p sees keys max(0, p - window)..p (window < 0: from 0).
 // Partials: part_o [n_items, n_q, splits, D] (unnormalised), part_ml [n_items, n_q, splits, 2] (max, sum);
 // with splits == 1 the result goes straight to `out` [n_tokens, n_q * D].
-template <int D, int DEC_WAVES>
+// AHEAD: a wave asks for its next block of keys while it works on the current one (see below).
+template <int D, int DEC_WAVES, bool AHEAD>
 __global__ void __launch_bounds__(DEC_WAVES * WAVE)
 decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
@@ -151,24 +152,34 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
       acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[db].v, pf, acc[db], 0, 0, 0);
     }
   };
-  // Two blocks in turn: while one is worked on, the next one's keys and values are on their way (a wave that
-  // asked for them only when it got there would wait a trip to memory in every block).
   constexpr int STRIDE = DEC_WAVES * 32;
   int kb = first + wave * 32;
-  if (kb <= last) {
-    KeyBlock one, two;
-    load_block(one, kb);
-    while (true) {
-      const bool more = kb + STRIDE <= last;
-      if (more) load_block(two, kb + STRIDE);
+  if constexpr (AHEAD) {
+    // Two blocks in turn: while one is worked on, the next one's keys and values are on their way (a wave that
+    // asked for them only when it got there would wait a trip to memory in every block).  That pays while a wave
+    // has a few blocks; over dozens of blocks the second set of registers costs more in waves a SIMD holds
+    // (measured at batch 64, head size 64: 1.03x at a context of 2,048, level at 8,192, 0.89x at 30,000).
+    if (kb <= last) {
+      KeyBlock one, two;
+      load_block(one, kb);
+      while (true) {
+        const bool more = kb + STRIDE <= last;
+        if (more) load_block(two, kb + STRIDE);
+        attend(one, kb);
+        kb += STRIDE;
+        if (!more) break;
+        const bool further = kb + STRIDE <= last;
+        if (further) load_block(one, kb + STRIDE);
+        attend(two, kb);
+        kb += STRIDE;
+        if (!further) break;
+      }
+    }
+  } else {
+    for (; kb <= last; kb += STRIDE) {
+      KeyBlock one;
+      load_block(one, kb);
       attend(one, kb);
-      kb += STRIDE;
-      if (!more) break;
-      const bool further = kb + STRIDE <= last;
-      if (further) load_block(one, kb + STRIDE);
-      attend(two, kb);
-      kb += STRIDE;
-      if (!further) break;
     }
   }
   // Sum of the lane groups' partial denominators (the maximum is already common to them).
@@ -282,10 +293,12 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
   const int group = n_q / n_kv;
   dim3 grid(splits, n_kv * ((group + 15) / 16), n_items);
   constexpr int NW = D > 128 ? 2 : 4;   // keeps the merge buffer within 64 KB of LDS
-  decode_attention_kernel<D, NW><<<grid, NW * WAVE, 0, stream>>>(
-      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)rows,
-      (const int*)positions, (const int*)entry_of_token, (const int*)block_table, table_stride, (float*)part_o,
-      (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits);
+#define GO(AHEAD) decode_attention_kernel<D, NW, AHEAD><<<grid, NW * WAVE, 0, stream>>>( \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)rows, \
+      (const int*)positions, (const int*)entry_of_token, (const int*)block_table, table_stride, (float*)part_o, \
+      (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits)
+  if (split_keys <= 32 * NW * 8) GO(true); else GO(false);      // up to eight blocks a wave
+#undef GO
   int status = LAUNCH_STATUS();
   if (status == 0 && splits > 1) {
     decode_attention_merge<<<n_items * n_q, 64, 0, stream>>>((const float*)part_o, (const float*)part_ml,
