@@ -15,7 +15,9 @@ def pytest_configure(config):
 
 @pytest.fixture(scope="session")
 def model_folders(tmp_path_factory):
-    """Model folders of the tiny configurations, written once per session by the random-weights mode."""
+    """Model folders of the tiny configurations, written once per session by the random-weights mode.  The
+    norms' scales lie well away from 1, so that a norm's weight taken from the wrong tensor, or not at all,
+    changes the logits."""
     from tiny_configs import TINY
     import tokenizer_amd as ta
     from tokenizer_amd.config import Qwen2Config
@@ -24,6 +26,6 @@ def model_folders(tmp_path_factory):
     folders = {}
     for name, (raw, seed) in TINY.items():
         folder = str(root / name)
-        ta.write_random_model(Qwen2Config.from_dict(raw), seed, folder)
+        ta.write_random_model(Qwen2Config.from_dict(raw), seed, folder, norm_spread=0.3)
         folders[name] = folder
     return folders

@@ -13,9 +13,9 @@ def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_si
 
     inner = engine.step
 
-    def step(entries):
+    def step(entries, **kw):
         engine.forwards.append([len(e.tokens) for e in entries])
-        return inner(entries)
+        return inner(entries, **kw)
 
     if counting:
         engine.step = step

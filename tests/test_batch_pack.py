@@ -42,7 +42,7 @@ def expected_parts(manager, entries, table_width):
             slots += [table[p // page] * page + p % page for p in range(start, start + len(entry.tokens))]
         flat = []
         for table in tables:
-            flat += table + [-1] * (width - len(table))
+            flat += table[:width] + [-1] * (width - len(table))     # pages held beyond a fixed width are left out
         parts += [slots, flat]
     return parts
 
@@ -82,6 +82,23 @@ def test_packed_batch_matches_its_definition(seed, table_width):
     assert ctx.max_q_len == max(len(e.tokens) for e in entries)
     assert ctx.max_position == max(manager.seq_len(e.rid) + len(e.tokens) - 1 for e in entries)
     manager.check_invariants()
+
+
+def test_a_fixed_width_leaves_out_pages_beyond_the_steps_last_token():
+    """A prompt's pages are reserved whole while its first portions run: the request's table is then wider than a
+    step's fixed width needs to be, and only the pages up to the step's last token are written."""
+    manager = CacheManager([CacheNeed("full", 2, 16)], num_pages=40, page_size=16, max_requests=2)
+    manager.add_request("a")
+    assert manager.reserve("a", 200)                               # thirteen pages
+    entry = StepEntry("a", list(range(32)), [31])
+    ctx = build_context([entry], manager, "cpu", table_width=4)
+    assert ctx.block_tables[0].tolist() == [manager.table("a", 0)[:4]]
+    manager.advance("a", 32)
+    ctx = build_context([StepEntry("a", list(range(32)), [31])], manager, "cpu", table_width=4)
+    assert ctx.block_tables[0].tolist() == [manager.table("a", 0)[:4]] and ctx.positions.tolist() == list(range(32, 64))
+    manager.advance("a", 64)
+    with pytest.raises(ValueError, match="wider"):                 # tokens 64..95 need a fifth and a sixth page
+        build_context([StepEntry("a", list(range(32)), [31])], manager, "cpu", table_width=4)
 
 
 def test_packing_refuses_what_does_not_fit():

@@ -198,6 +198,41 @@ def test_groups_follow_the_needs():
     assert CacheManager([FULL, FULL], 8, P, 2, prefix_cache=True).prefix_cache
 
 
+def test_no_prefix_sharing_beside_state_of_fixed_size():
+    """A layer that keeps state in the request's slot has seen every token; a request that attached a shared
+    prefix would skip those tokens, so sharing is off whatever was asked for."""
+    manager = CacheManager([NONE, FULL], 8, P, 2, prefix_cache=True)
+    assert not manager.prefix_cache
+    prompt = list(range(40))
+    manager.add_request(1)
+    manager.reserve(1, 40), manager.advance(1, 40), manager.publish(1, prompt)
+    manager.add_request(2)
+    assert manager.attach_shared_prefix(2, prompt + [7]) == 0 and manager.seq_len(2) == 0
+    state_and_pages = CacheNeed("full", 2, 16, state_shape=(3,))
+    assert not CacheManager([state_and_pages, FULL], 8, P, 2, prefix_cache=True).prefix_cache
+
+
+def test_a_kind_of_cache_is_a_rule_for_what_is_kept():
+    """Another kind registers how far behind a query its keys are read; the bookkeeping needs nothing else."""
+    from tokenizer_amd.cache import manager as manager_module
+    manager_module.CACHE_KINDS["twice_the_window"] = lambda need: 2 * need.window
+    try:
+        manager = CacheManager([CacheNeed("twice_the_window", 2, 16, window=10), FULL], 16, P, 1)
+        assert manager.group_of_layer == [0, 1]
+        manager.add_request("a")
+        manager.reserve("a", 100), manager.advance("a", 100)
+        assert manager.first_needed_position(0, 100) == 80 and manager.first_needed_position(1, 100) == 0
+        assert [p >= 0 for p in manager.table("a", 0)] == [False] * 5 + [True] * 2     # positions below 80 are gone
+        manager.release("a")
+        manager.check_invariants()
+    finally:
+        del manager_module.CACHE_KINDS["twice_the_window"]
+    with pytest.raises(ValueError, match="unknown cache kind"):
+        CacheManager([CacheNeed("twice_the_window", 2, 16, window=10)], 16, P, 1)
+    with pytest.raises(ValueError, match="needs a window"):
+        CacheManager([CacheNeed("window", 2, 16)], 16, P, 1)
+
+
 def test_reserve_is_all_or_nothing_and_release_returns_everything():
     manager = CacheManager([FULL, WIN], num_pages=4, page_size=P, max_requests=2)
     manager.add_request("a")

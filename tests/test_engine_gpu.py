@@ -125,7 +125,7 @@ def test_thousands_of_tokens_of_context(tmp_path, dtype):
     from tokenizer_amd.config import Qwen2Config
     from tokenizer_amd.engine import StepEntry
     raw = dict(TINY["A"][0], max_position_embeddings=8192, sliding_window=8192, rope_theta=1000000.0)
-    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 11, str(tmp_path / "long"))
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 11, str(tmp_path / "long"), norm_spread=0.3)
     cfg, tensors = plain.load_folder(folder)
     long_ids, short_ids = random_ids(256, 5200, 31), random_ids(256, 60, 32)
     if "long" not in _LONG_ORACLE:                                # the same weights for both dtypes: computed once
@@ -226,8 +226,6 @@ def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
         else:
             entries = [StepEntry(rid, [rng_tokens[at + i]], [0]) for i, rid in enumerate(action)]
             at += len(action)
-        if action == [0]:
-            entries = [StepEntry(rid, e.tokens, e.want) if True else e for rid, e in zip(action, entries)]
         got = []
         for eng in engines:
             if not all(eng.cache.seq_len(e.rid) for e in entries):          # first use: run the prompt
@@ -394,7 +392,7 @@ def test_greedy_generation_through_the_entry_points(model_folders, tmp_path, dty
                          capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr
     assert f"prompt ids ({len(prompt)}): {prompt}" in run.stderr
-    assert "max_tokens 8 temperature 0.0 top_p 1.0 seed 0 eos []" in run.stderr
+    assert "max_tokens 8 temperature 0 top_p 1 seed 0 eos []" in run.stderr
     assert f"generated ids: {out.tokens}" in run.stderr and "stop: MaxTokens" in run.stderr
     assert "tok/s (8 tokens, KV cache, total" in run.stderr
     assert run.stdout.split() == [str(t) for t in out.tokens]
@@ -464,7 +462,7 @@ def test_layers_of_real_sizes(tmp_path, size):
     from tokenizer_amd.config import Qwen2Config
     raw = dict(TINY["A"][0], num_hidden_layers=2, vocab_size=1000, max_position_embeddings=512,
                tie_word_embeddings=(size != "7b"), **REAL_SIZES[size])
-    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 11, str(tmp_path / size))
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 11, str(tmp_path / size), norm_spread=0.3)
     cfg, tensors = plain.load_folder(folder)
     reqs = {f"r{i}": random_ids(1000, n, 20 + i) for i, n in enumerate([150, 47, 80])}
     want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
@@ -511,7 +509,7 @@ def test_sizes_away_from_every_tile(tmp_path, size):
     import tokenizer_amd as ta
     from tokenizer_amd.config import Qwen2Config
     raw = dict(TINY["A"][0], max_position_embeddings=512, **ODD_SIZES[size])
-    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 13, str(tmp_path / size))
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 13, str(tmp_path / size), norm_spread=0.3)
     cfg, tensors = plain.load_folder(folder)
     reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 30 + i) for i, n in enumerate([70, 33, 100, 9])}
     want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
@@ -532,7 +530,7 @@ def test_the_whole_model_at_half_a_billion_parameters(tmp_path):
     raw = dict(TINY["A"][0], num_hidden_layers=24, vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6,
                tie_word_embeddings=True, max_position_embeddings=32768, sliding_window=32768, max_window_layers=24,
                **REAL_SIZES["0.5b"])
-    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 0, str(tmp_path / "half_b"))
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 0, str(tmp_path / "half_b"), norm_spread=0.3)
     cfg, tensors = plain.load_folder(folder)
     reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 50 + i) for i, n in enumerate([150, 70, 33])}
     want = {rid: plain.all_logits(cfg, tensors, ids) for rid, ids in reqs.items()}
@@ -574,7 +572,7 @@ def test_decode_batches_of_dozens_at_sizes_away_from_every_tile(tmp_path, size):
     from tokenizer_amd.config import Qwen2Config
     from tokenizer_amd.engine import StepEntry
     raw = dict(TINY["A"][0], max_position_embeddings=512, **ODD_SIZES[size])
-    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 17, str(tmp_path / size))
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 17, str(tmp_path / size), norm_spread=0.3)
     cfg, tensors = plain.load_folder(folder)
     for dtype in ("bfloat16", "float32"):
         for batch in (20, 64):

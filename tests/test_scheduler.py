@@ -228,3 +228,17 @@ def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed
             continue
         assert result.tokens == solo(folder, prompt, GenerateParams.greedy(n)).tokens, (rid, len(prompt), n)
     sched.assert_idle()
+
+
+def test_a_step_that_may_not_reserve_refuses_an_entry_without_pages(model_folders):
+    """The scheduler reserves while it plans; the step it then runs takes nothing from the pool."""
+    from tokenizer_amd.engine import StepEntry
+    engine = cpu_engine(model_folders["A"], num_pages=4, counting=False)
+    engine.add_request("a")
+    with pytest.raises(RuntimeError, match="too few pages"):
+        engine.step([StepEntry("a", [1, 2, 3], [2])], reserve=False)
+    assert engine.cache.seq_len("a") == 0 and engine.cache.groups[0].allocator.live_count() == 0
+    assert engine.cache.reserve("a", 3)
+    assert engine.step([StepEntry("a", [1, 2, 3], [2])], reserve=False).shape == (1, 256)
+    assert engine.cache.seq_len("a") == 3 and engine.cache.groups[0].allocator.live_count() == 1
+    engine.end_request("a")

@@ -84,6 +84,24 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert word in text
 
 
+def test_tensors_the_model_does_not_read_are_a_warning_alone(tmp_path):
+    # A tied model saved with a redundant head, an export with rotary buffers: the reference takes what it asks
+    # for by name and never looks at the rest (qwen-infer/src/model.rs:776-786).
+    from tokenizer_amd.weights import UnexpectedTensors
+    tensors = random_tensors(expected(), 0)
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    path = str(tmp_path / "model.safetensors")
+    save_safetensors(path, tensors)
+    with pytest.warns(UnexpectedTensors, match="lm_head.weight") as caught:
+        out = load_weights(path, expected(), torch.bfloat16)
+    assert "rotary_emb.inv_freq" in str(caught[0].message) and set(out) == set(expected())
+    with pytest.raises(WeightError) as err:
+        load_weights(path, expected(), torch.bfloat16, strict=True)
+    assert err.value.unexpected == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert not err.value.missing
+
+
 def test_untied_model_needs_its_head(tmp_path):
     tensors = random_tensors(expected("B"), 2)
     del tensors["lm_head.weight"]

@@ -40,6 +40,31 @@ class RequestCache:
     slot: int = -1
 
 
+def _window_of_window_kind(need: CacheNeed) -> int:
+    if need.window is None or need.window < 0:
+        raise ValueError("a window cache needs a window")
+    return int(need.window)
+
+
+# What a kind of cache keeps, as the one number the bookkeeping works with: None = the keys and values of
+# every position; w >= 0 = a query reads at most w positions behind itself, and pages wholly behind every
+# later query are given back.  A mixer with another name for its need (or another way to derive the window
+# from its `CacheNeed`) adds its kind here; kind "none" asks for no pages at all.
+CACHE_KINDS: dict[str, "callable"] = {
+    "full": lambda need: None,
+    "window": _window_of_window_kind,
+}
+
+
+def retention_window(need: CacheNeed) -> int | None:
+    """The window behind which a group of this need gives pages back (None: never)."""
+    try:
+        rule = CACHE_KINDS[need.kind]
+    except KeyError:
+        raise ValueError(f"unknown cache kind {need.kind!r}; known: none, {', '.join(sorted(CACHE_KINDS))}") from None
+    return rule(need)
+
+
 def plan_groups(needs: list[CacheNeed]) -> tuple[list[tuple[CacheNeed, list[int]]], list[int | None]]:
     """Group the layers by what they need.  Returns the groups and, per layer, its group index."""
     groups: list[tuple[CacheNeed, list[int]]] = []
@@ -49,10 +74,10 @@ def plan_groups(needs: list[CacheNeed]) -> tuple[list[tuple[CacheNeed, list[int]
         if need.kind == "none":
             group_of.append(None)
             continue
-        if need.kind not in ("full", "window"):
-            raise ValueError(f"layer {layer} asks for an unknown cache kind {need.kind!r}")
-        if need.kind == "window" and (need.window is None or need.window < 0):
-            raise ValueError(f"layer {layer} asks for a window cache without a window")
+        try:
+            retention_window(need)
+        except ValueError as err:
+            raise ValueError(f"layer {layer}: {err}") from None
         key = need.page_key()
         if key not in keys:
             keys[key] = len(groups)
@@ -121,11 +146,11 @@ class CacheManager:
         self.num_pages = num_pages
         self.max_requests = max_requests
         self._lib = _host.lib()
-        kinds = (ctypes.c_int32 * max(1, len(planned)))(*[1 if need.kind == "window" else 0 for need, _ in planned])
-        windows = (ctypes.c_int32 * max(1, len(planned)))(*[need.window if need.kind == "window" else -1
-                                                           for need, _ in planned])
-        self._core = self._lib.ta_cache_new(len(planned), kinds, windows, num_pages, page_size, max_requests,
-                                            1 if prefix_cache else 0)
+        kept = [retention_window(need) for need, _ in planned]
+        windows = (ctypes.c_int32 * max(1, len(planned)))(*[-1 if w is None else w for w in kept])
+        self.state_layers = [i for i, need in enumerate(needs) if need.state_shape is not None]
+        self._core = self._lib.ta_cache_new(len(planned), windows, num_pages, page_size, max_requests,
+                                            1 if prefix_cache else 0, len(self.state_layers))
         if not self._core:
             raise ValueError("num_pages and max_requests must not be negative and page_size must be positive")
         self._core_owner = _CoreOwner(self._lib, self._core)
@@ -133,9 +158,9 @@ class CacheManager:
                                                               _borrowed=self._lib.ta_cache_allocator(self._core, g),
                                                               _owner=self._core_owner))
                        for g, (need, layers) in enumerate(planned)]
-        # Sharing a prefix needs every group to keep all positions (a window group drops pages).
+        # Sharing a prefix needs every group to keep all positions (a window group drops pages) and no layer
+        # that keeps state of its own in the request's slot (it would never see an attached prefix's tokens).
         self.prefix_cache = bool(self._lib.ta_cache_prefix_enabled(self._core))
-        self.state_layers = [i for i, need in enumerate(needs) if need.state_shape is not None]
         # A request id that is a small non-negative integer is its own handle in the core (so the scheduler core,
         # which numbers its sequences, and this class speak of the same requests); any other id gets one here.
         self._ids: dict[object, int] = {}

@@ -89,6 +89,13 @@ def parse_args(argv: list[str]) -> dict:
     return args
 
 
+def _plain_number(value: float) -> str:
+    """A float as the reference's `{}` prints it (qwen-infer/src/main.rs:33-36): whole numbers without a
+    fraction ("0", "1"), others as short as they read back ("0.7")."""
+    text = repr(float(value))
+    return text[:-2] if text.endswith(".0") else text
+
+
 def main(argv: list[str] | None = None) -> int:
     try:
         args = parse_args(sys.argv[1:] if argv is None else argv)
@@ -125,8 +132,8 @@ def main(argv: list[str] | None = None) -> int:
     eos_path = os.path.join(folder, "generation_config.json")
     if os.path.exists(eos_path):
         params.eos = load_eos_token_ids(eos_path)
-    print(f"max_tokens {params.max_tokens} temperature {params.temperature} top_p {params.top_p} "
-          f"seed {params.seed} eos {params.eos}", file=sys.stderr)
+    print(f"max_tokens {params.max_tokens} temperature {_plain_number(params.temperature)} "
+          f"top_p {_plain_number(params.top_p)} seed {params.seed} eos {params.eos}", file=sys.stderr)
 
     if args["random_weights"] is not None:      # the folder then needs its config.json only
         model = random_model(load_config(folder), args["random_weights"], args["dtype"])

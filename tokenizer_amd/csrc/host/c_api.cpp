@@ -90,10 +90,11 @@ int ta_alloc_check(void* a) {
 }
 
 // ------------------------------------------------------------------------------------------- cache
-void* ta_cache_new(int n_groups, const int* kinds, const int* windows, int num_pages, int page_size,
-                   int max_requests, int prefix_cache) {
-  if (n_groups < 0 || num_pages < 0 || page_size <= 0 || max_requests < 0) return nullptr;
-  return new CacheCore(n_groups, kinds, windows, num_pages, page_size, max_requests, prefix_cache != 0);
+// windows[g] < 0: group g keeps every position; else the window behind which its pages are given back.
+void* ta_cache_new(int n_groups, const int* windows, int num_pages, int page_size, int max_requests,
+                   int prefix_cache, int n_state_layers) {
+  if (n_groups < 0 || num_pages < 0 || page_size <= 0 || max_requests < 0 || n_state_layers < 0) return nullptr;
+  return new CacheCore(n_groups, windows, num_pages, page_size, max_requests, prefix_cache != 0, n_state_layers);
 }
 void ta_cache_delete(void* c) { delete (CacheCore*)c; }
 void* ta_cache_allocator(void* c, int group) { return ((CacheCore*)c)->allocator(group); }   // borrowed
@@ -164,7 +165,7 @@ int ta_sched_append_token(void* s, int64_t id, int32_t token) { return ((Schedul
 // (-1: empty), 6 pages to admit `id`, 7 tokens of `id` in the cache, 8 tokens `id` holds, 9 whether `id` runs.
 int64_t ta_sched_get(void* s, int what, int64_t id) {
   const SchedulerCore& core = *(SchedulerCore*)s;
-  const Sequence* seq = what >= 7 ? core.find(id) : nullptr;
+  const Sequence* seq = what >= 7 && what <= 9 ? core.find(id) : nullptr;
   switch (what) {
     case 0: return core.n_running();
     case 1: return core.n_waiting();
@@ -176,6 +177,8 @@ int64_t ta_sched_get(void* s, int what, int64_t id) {
     case 7: return seq ? seq->computed : -1;
     case 8: return seq ? (int64_t)seq->tokens.size() : -1;
     case 9: return seq ? (seq->running ? 1 : 0) : -1;
+    case 10: return core.prefix_hits();
+    case 11: return core.prefix_tokens_reused();
     default: return -1;
   }
 }

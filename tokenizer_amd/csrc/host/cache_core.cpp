@@ -6,16 +6,17 @@ namespace ta {
 
 static int pages_for_len(int length, int page_size) { return (length + page_size - 1) / page_size; }
 
-CacheCore::CacheCore(int n_groups, const int* kinds, const int* windows, int num_pages, int page_size,
-                     int max_requests, bool prefix_cache)
+CacheCore::CacheCore(int n_groups, const int* windows, int num_pages, int page_size, int max_requests,
+                     bool prefix_cache, int n_state_layers)
     : page_size_(page_size), max_requests_(max_requests) {
-  bool all_full = true;
+  bool all_kept = true;
   for (int g = 0; g < n_groups; ++g) {
-    groups_.emplace_back(new Group(kinds[g], windows[g], num_pages, page_size));
-    all_full = all_full && kinds[g] == CACHE_FULL;
+    groups_.emplace_back(new Group(windows[g], num_pages, page_size));
+    all_kept = all_kept && groups_.back()->keeps_all();
   }
-  // Sharing a prefix needs every group to keep all positions (a window group drops pages).
-  prefix_cache_ = prefix_cache && all_full;
+  // Sharing a prefix needs every group to keep all positions (a window group drops pages) and no layer with
+  // state of its own in the slot (it would never see the tokens of an attached prefix).
+  prefix_cache_ = prefix_cache && all_kept && n_state_layers == 0;
   for (int slot = max_requests - 1; slot >= 0; --slot) free_slots_.push_back(slot);
 }
 
@@ -50,7 +51,7 @@ int CacheCore::add_request(int64_t id) {
 
 int CacheCore::first_needed_position(int group, int seq_len) const {
   const Group& g = *groups_[group];
-  return g.kind == CACHE_WINDOW ? std::max(0, seq_len - g.window) : 0;
+  return g.keeps_all() ? 0 : std::max(0, seq_len - g.window);
 }
 
 int CacheCore::pages_missing(int64_t id, int new_len, int* per_group) const {
@@ -89,7 +90,7 @@ int CacheCore::advance(int64_t id, int new_len) {
     if (pages_for_len(new_len, page_size_) > (int)table.size()) return CACHE_TOO_FEW_PAGES;
   request->seq_len = new_len;
   for (size_t g = 0; g < groups_.size(); ++g) {
-    if (groups_[g]->kind != CACHE_WINDOW) continue;
+    if (groups_[g]->keeps_all()) continue;
     // Pages no later query reads again go back to the pool.
     const int first = first_needed_position((int)g, new_len);
     std::vector<int>& table = request->tables[g];
@@ -211,10 +212,14 @@ int64_t CacheCore::pack_batch(int n_entries, const int64_t* ids, const int* n_to
   }
   for (int g = 0; g < n_groups; ++g) {
     int width = 1;
-    for (int e = 0; e < n_entries; ++e) width = std::max(width, (int)requests[e]->tables[g].size());
     if (table_width >= 0) {
-      if (width > table_width) return CACHE_TABLE_TOO_WIDE;
+      // A fixed width has to hold the pages up to each request's last token of this step; pages a request holds
+      // beyond that are left out.
+      for (int e = 0; e < n_entries; ++e)
+        if (pages_for_len(requests[e]->seq_len + n_tokens[e], page_size_) > table_width) return CACHE_TABLE_TOO_WIDE;
       width = table_width;
+    } else {
+      for (int e = 0; e < n_entries; ++e) width = std::max(width, (int)requests[e]->tables[g].size());
     }
     widths[g] = width;
   }
@@ -280,8 +285,9 @@ int64_t CacheCore::pack_batch(int n_entries, const int64_t* ids, const int* n_to
         slots[at++] = page * page_size_ + p % page_size_;
       }
       int32_t* dst = table_out + (int64_t)e * widths[g];
-      std::copy(table.begin(), table.end(), dst);
-      std::fill(dst + table.size(), dst + widths[g], -1);
+      const size_t copied = std::min(table.size(), (size_t)widths[g]);
+      std::copy(table.begin(), table.begin() + copied, dst);
+      std::fill(dst + copied, dst + widths[g], -1);
     }
   }
   return total;

@@ -12,17 +12,20 @@
 
 namespace ta {
 
-enum CacheKind { CACHE_FULL = 0, CACHE_WINDOW = 1 };
 enum CacheStatus {
   CACHE_OK = 0, CACHE_ALREADY_LIVE = -1, CACHE_NO_SLOT = -2, CACHE_UNKNOWN_REQUEST = -3, CACHE_SHRINKS = -4,
   CACHE_TOO_FEW_PAGES = -5, CACHE_PAGE_GIVEN_BACK = -6, CACHE_TABLE_TOO_WIDE = -7, CACHE_BUFFER_TOO_SMALL = -8,
   CACHE_BAD_ARGUMENT = -9
 };
 
+// A group of layers with one need: `window` < 0 keeps the keys of every position; a window w >= 0 means that a
+// query reads the keys at most w positions behind it, so pages wholly behind every later query are given back.
+// (Whatever a mixer calls its kind of cache, it reaches this class as that one number.)
 struct Group {
-  int kind, window;
+  int window;
   PageAllocator allocator;
-  Group(int kind, int window, int num_pages, int page_size) : kind(kind), window(window), allocator(num_pages, page_size) {}
+  bool keeps_all() const { return window < 0; }
+  Group(int window, int num_pages, int page_size) : window(window), allocator(num_pages, page_size) {}
 };
 
 struct Request {
@@ -33,8 +36,11 @@ struct Request {
 
 class CacheCore {
  public:
-  CacheCore(int n_groups, const int* kinds, const int* windows, int num_pages, int page_size, int max_requests,
-            bool prefix_cache);
+  // `n_state_layers`: how many layers keep per-request state of fixed size in the request's slot.  A prefix can
+  // be shared only when what a request holds after it is a function of its pages alone: every group keeps all
+  // positions and no layer keeps such state (a state slot has seen every token; an attached prefix would skip them).
+  CacheCore(int n_groups, const int* windows, int num_pages, int page_size, int max_requests, bool prefix_cache,
+            int n_state_layers);
 
   int n_groups() const { return (int)groups_.size(); }
   int page_size() const { return page_size_; }
@@ -61,7 +67,10 @@ class CacheCore {
   // `tokens`) and n_want[i] wanted places among them (flattened in `want`).  The parts are written one after
   // the other into `out`: token ids, positions, entry of token, cu_q, first position, state slot, wanted rows,
   // tiles of 16 prompt tokens as (entry, offset), rows of single tokens, then per group the cache slot of every
-  // token and the block tables [n_entries, width].  table_width < 0: the widest table of the batch (at least 1).
+  // token and the block tables [n_entries, width].  table_width < 0: the widest table of the batch (at least 1);
+  // else every table is written that wide: a request may hold more pages than that (a prompt's pages are
+  // reserved whole while its first portions run), as long as the pages up to its last token of this step fit,
+  // since no later one is read or written in the step.
   // sizes: 9 + 2 * groups part lengths; widths: per group.  Returns the total length or a CacheStatus.
   int64_t pack_batch(int n_entries, const int64_t* ids, const int* n_tokens, const int32_t* tokens,
                      const int* n_want, const int* want, int table_width, int32_t* out, int64_t capacity,

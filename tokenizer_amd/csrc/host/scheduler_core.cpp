@@ -69,6 +69,7 @@ void SchedulerCore::admit(std::vector<FailedEntry>* failed) {
       break;
     }
     waiting_.pop_front();
+    if (shared > 0) { ++prefix_hits_; prefix_tokens_ += shared; }
     seq.computed = shared;
     seq.running = true;
     running_.push_back(id);

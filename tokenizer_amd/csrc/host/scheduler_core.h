@@ -43,6 +43,8 @@ class SchedulerCore {
   int max_running() const { return max_running_; }
   int preemptions() const { return preemptions_; }
   int64_t last_preempted_id() const { return last_preempted_; }
+  int prefix_hits() const { return prefix_hits_; }                   // admissions that found shared pages
+  int64_t prefix_tokens_reused() const { return prefix_tokens_; }    // tokens those pages held
   int64_t front_waiting() const { return waiting_.empty() ? -1 : waiting_.front(); }
   int pages_to_admit(int64_t id) const;
   const std::vector<int64_t>& running() const { return running_; }
@@ -65,7 +67,8 @@ class SchedulerCore {
   std::unordered_map<int64_t, Sequence> sequences_;
   std::deque<int64_t> waiting_;
   std::vector<int64_t> running_;          // in order of admission
-  int max_running_ = 0, preemptions_ = 0;
+  int max_running_ = 0, preemptions_ = 0, prefix_hits_ = 0;
+  int64_t prefix_tokens_ = 0;
   int64_t last_preempted_ = 0;
 };
 

@@ -409,9 +409,15 @@ class Engine:
                 raise OutOfPages(f"no pages left for request {entry.rid!r} to reach {new_len} tokens "
                                  f"({self.cache.num_pages} pages of {self.cache.page_size})")
 
-    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+    def step(self, entries: list[StepEntry], reserve: bool = True) -> torch.Tensor:
+        """Run the entries' tokens as one batch; float32 logits [wanted, vocab].  The step itself works on pages
+        that are there: `reserve=True` (callers without a scheduler: replay, `generate`, tests) first asks the
+        cache manager for the pages of the new tokens and raises `OutOfPages` if there are none;
+        `reserve=False` (the scheduler, which reserves while it plans and preempts when pages run out) takes
+        nothing from the pool, and an entry whose pages are missing is refused."""
         self.validate(entries)
-        self.reserve(entries)
+        if reserve:
+            self.reserve(entries)
         self._graph_result = None
         if self._replays(entries):
             logits = self._graph_step(entries)

@@ -51,6 +51,8 @@ class EngineStats:
     last_preempted_id: int = 0
     peak_blocks: int = 0
     peak_occupied: int = 0
+    prefix_hits: int = 0             # admissions that took over pages another request had computed
+    prefix_tokens_reused: int = 0    # tokens those pages held (never forwarded again)
     steps: int = 0
     tokens_forwarded: int = 0
 
@@ -80,13 +82,13 @@ class Sequence:
 
 
 _RUNNING, _WAITING, _MAX_RUNNING, _PREEMPTIONS, _LAST_PREEMPTED, _FRONT, _PAGES_TO_ADMIT, _COMPUTED, _N_TOKENS, \
-    _IS_RUNNING = range(10)
+    _IS_RUNNING, _PREFIX_HITS, _PREFIX_TOKENS = range(12)
 
 
 class Scheduler:
     """Admits requests, cuts prompts into portions, decodes, finishes and frees.
 
-    `engine` needs: `.cache` (a CacheManager), `.step(entries) -> logits`, `.argmax(logits, rows) ->
+    `engine` needs: `.cache` (a CacheManager), `.step(entries, reserve=False) -> logits`, `.argmax(logits, rows) ->
     list[int]`, `.max_positions`, and for warm requests `.sample(logits, rows, temperature, top_p, uniform)
     -> list[int]` or, without it, `.rows_to_host(logits, rows) -> float32 array` (drawn on the host then).
     """
@@ -212,7 +214,7 @@ class Scheduler:
             if wants:
                 wanting.append(seq)
         started = time.perf_counter()
-        logits = self.engine.step(entries)
+        logits = self.engine.step(entries, reserve=False)       # the plan reserved every page
         greedy_rows = [row for row, seq in enumerate(wanting) if seq.cursor.is_greedy]
         warm_rows = [row for row, seq in enumerate(wanting) if not seq.cursor.is_greedy]
         picked: dict[int, int] = {}
@@ -272,6 +274,8 @@ class Scheduler:
         self.stats.max_running = self._get(_MAX_RUNNING)
         self.stats.preemptions = self._get(_PREEMPTIONS)
         self.stats.last_preempted_id = self._get(_LAST_PREEMPTED)
+        self.stats.prefix_hits = self._get(_PREFIX_HITS)
+        self.stats.prefix_tokens_reused = self._get(_PREFIX_TOKENS)
         for group in self.cache.groups:
             self.stats.peak_blocks = max(self.stats.peak_blocks, group.allocator.peak_live)
             self.stats.peak_occupied = max(self.stats.peak_occupied, group.allocator.peak_occupied)

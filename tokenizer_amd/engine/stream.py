@@ -7,18 +7,6 @@ one U+FFFD each time they are met; `finish` decodes whatever is left, lossily.
 from __future__ import annotations
 
 
-def _expected_length(first: int) -> int:
-    if first < 0x80:
-        return 1
-    if 0xC2 <= first <= 0xDF:
-        return 2
-    if 0xE0 <= first <= 0xEF:
-        return 3
-    if 0xF0 <= first <= 0xF4:
-        return 4
-    return 0
-
-
 class StreamDecoder:
     def __init__(self):
         self.pending = bytearray()

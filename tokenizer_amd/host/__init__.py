@@ -33,7 +33,7 @@ _SIGNATURES = {
     "ta_alloc_publish_prompt_pages": (None, [_vp, _i32p, _int, _i32p, _int]),
     "ta_alloc_reclaim_cached": (None, [_vp]),
     "ta_alloc_check": (_int, [_vp]),
-    "ta_cache_new": (_vp, [_int, _i32p, _i32p, _int, _int, _int, _int]),
+    "ta_cache_new": (_vp, [_int, _i32p, _int, _int, _int, _int, _int]),
     "ta_cache_delete": (None, [_vp]),
     "ta_cache_allocator": (_vp, [_vp, _int]),
     "ta_cache_prefix_enabled": (_int, [_vp]),

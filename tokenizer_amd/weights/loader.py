@@ -2,6 +2,13 @@
 
 The file is matched to the expectation in one pass and every problem is
 reported together: missing tensors, unexpected tensors and wrong shapes.
+Tensors the model does not read are no reason to refuse a file that holds
+everything else (the reference's loader takes what it asks for by name and never
+looks at the rest, qwen-infer/src/model.rs:776-786: a tied model saved with a
+redundant `lm_head.weight`, an export with `rotary_emb.inv_freq` buffers): alone
+they are a warning; beside a real misfit they are listed in the same error,
+since a misnamed tensor shows up as one missing and one unexpected name.
+`strict=True` makes them an error on their own.
 Tensors are not renamed; a part that wants two matrices side by side joins
 them itself after loading (the reference keeps q, k, v and gate, up apart,
 qwen-infer/src/model.rs:263-276).
@@ -9,11 +16,16 @@ qwen-infer/src/model.rs:263-276).
 from __future__ import annotations
 
 import os
+import warnings
 
 import torch
 
 from ..parts.spec import TensorSpec
 from .safetensors_io import SafetensorsError, SafetensorsFile
+
+
+class UnexpectedTensors(UserWarning):
+    """The weight file holds tensors that the model does not read."""
 
 
 class WeightError(ValueError):
@@ -67,8 +79,10 @@ def weight_path(folder: str) -> str:
 
 
 def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: torch.dtype,
-                 device: torch.device | str = "cpu") -> dict[str, torch.Tensor]:
-    """Load exactly the tensors in `expected`, or raise one `WeightError` naming every misfit."""
+                 device: torch.device | str = "cpu", strict: bool = False) -> dict[str, torch.Tensor]:
+    """Load the tensors in `expected`, or raise one `WeightError` naming every misfit (missing, wrong shape,
+    unusable dtype, and the unexpected names beside them).  Unexpected tensors alone: an `UnexpectedTensors`
+    warning that lists them, or the same error with `strict=True`."""
     path = weight_path(folder)
     try:
         source = SafetensorsFile(path)
@@ -87,8 +101,11 @@ def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: to
             wrong_dtype.append((name, dtype))
         if spec.role == "table" and dtype not in _INTS:
             wrong_dtype.append((name, dtype))
-    if missing or unexpected or wrong_shape or wrong_dtype:
+    if missing or wrong_shape or wrong_dtype or (unexpected and strict):
         raise WeightError(path, missing, unexpected, wrong_shape, wrong_dtype)
+    if unexpected:
+        warnings.warn(UnexpectedTensors(f"{path} holds {len(unexpected)} tensors the model does not read: "
+                                        + ", ".join(unexpected)), stacklevel=2)
     out = {}
     for name, spec in expected.items():
         out[name] = stored_form(source.tensor(name), spec, compute_dtype).to(device).contiguous()

@@ -3,7 +3,9 @@
 Every tensor is drawn from its own generator keyed by (seed, tensor name), so
 the values of a tensor do not depend on which other tensors exist.  Matrices,
 biases and the embedding are N(0, std) rounded to bfloat16 (the dtype model
-files are stored in); norm scales are 1.
+files are stored in); norm scales are 1, or 1 + spread * N(0, 1) when a spread
+is asked for (tests do: with every scale equal to 1 two norms could be swapped,
+or one left out, and no logit would change).
 """
 from __future__ import annotations
 
@@ -24,11 +26,14 @@ def _generator(seed: int, name: str) -> torch.Generator:
     return gen
 
 
-def random_tensor(name: str, spec: TensorSpec, seed: int) -> torch.Tensor:
+def random_tensor(name: str, spec: TensorSpec, seed: int, norm_spread: float = 0.0) -> torch.Tensor:
     if spec.role == "table":
         return torch.zeros(spec.shape, dtype=torch.int32)
     if spec.init == "ones":
-        return torch.ones(spec.shape, dtype=torch.bfloat16)
+        if not norm_spread:
+            return torch.ones(spec.shape, dtype=torch.bfloat16)
+        noise = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=_generator(seed, name))
+        return (1.0 + float(norm_spread) * noise).to(torch.bfloat16)
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=torch.bfloat16)
     if spec.init != "normal":
@@ -40,12 +45,13 @@ def random_tensor(name: str, spec: TensorSpec, seed: int) -> torch.Tensor:
     return values if spec.role == "keep" else values.to(torch.bfloat16)
 
 
-def random_tensors(expected: dict[str, TensorSpec], seed: int) -> dict[str, torch.Tensor]:
-    return {name: random_tensor(name, spec, seed) for name, spec in expected.items()}
+def random_tensors(expected: dict[str, TensorSpec], seed: int, norm_spread: float = 0.0) -> dict[str, torch.Tensor]:
+    return {name: random_tensor(name, spec, seed, norm_spread) for name, spec in expected.items()}
 
 
-def write_random_model(config: ModelConfig, seed: int, folder: str) -> str:
-    """Write config.json and model.safetensors for `config` with weights from `seed`."""
+def write_random_model(config: ModelConfig, seed: int, folder: str, norm_spread: float = 0.0) -> str:
+    """Write config.json and model.safetensors for `config` with weights from `seed`.  `norm_spread`: how far
+    the norms' scales lie from 1 (standard deviation; 0 = all equal to 1)."""
     from ..config.registry import get_architecture
     from ..parts.model import expected_tensors
 
@@ -53,6 +59,6 @@ def write_random_model(config: ModelConfig, seed: int, folder: str) -> str:
     os.makedirs(folder, exist_ok=True)
     config.save(folder)
     save_safetensors(os.path.join(folder, "model.safetensors"),
-                     random_tensors(expected_tensors(spec), seed),
+                     random_tensors(expected_tensors(spec), seed, norm_spread),
                      metadata={"format": "pt", "seed": str(seed)})
     return folder
