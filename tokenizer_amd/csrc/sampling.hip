@@ -1,5 +1,8 @@
 // Greedy pick on the device: the first maximum wins, as a scan with `>` from -inf does.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 #define ARGMAX_THREADS 256
 
@@ -75,6 +78,48 @@ extern "C" int ta_argmax(const void* logits, void* out, void* partial_v, void* p
   if (status) return status;
   argmax_rows<<<n_rows, ARGMAX_THREADS, 0, stream>>>((const float*)partial_v, (const int*)partial_i, (int*)out, chunks);
   return LAUNCH_STATUS();
+}
+
+// The same pick for callers that cannot allocate (see no_alloc.h): the pieces' maxima live in this array.  In
+// host code its name is only a stand-in; the address kernels can use is looked up per device, once, below.
+static __device__ __align__(256) unsigned char argmax_scratch[TA_ARGMAX_STATIC_PAIRS * (sizeof(float) + sizeof(int))];
+
+#define TA_MAX_DEVICES 64
+static void* g_argmax_scratch[TA_MAX_DEVICES];      // each GPU holds its own copy of the array at its own address
+static std::mutex g_argmax_scratch_lock;
+
+// The device address of `argmax_scratch` on the current device; 0 and a HIP error code in *status on failure.
+static void* argmax_scratch_here(int* status) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) { *status = (int)err; return nullptr; }
+  if (device < 0 || device >= TA_MAX_DEVICES) { *status = (int)hipErrorInvalidDevice; return nullptr; }
+  std::lock_guard<std::mutex> hold(g_argmax_scratch_lock);
+  if (!g_argmax_scratch[device]) {
+    void* found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(argmax_scratch));
+    if (err != hipSuccess || !found) { *status = err != hipSuccess ? (int)err : (int)hipErrorInvalidSymbol; return nullptr; }
+    g_argmax_scratch[device] = found;
+  }
+  *status = 0;
+  return g_argmax_scratch[device];
+}
+
+extern "C" int ta_argmax_static(const void* logits, void* out, int n_rows, int vocab, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (vocab < 1) return -1;
+  if (n_rows > TA_ARGMAX_STATIC_PAIRS) return TA_STATIC_TOO_LARGE;
+  // Pieces per row as the allocating wrapper chooses them, within what the array holds.
+  int chunks = vocab / 2048;
+  if (chunks > 256) chunks = 256;
+  if (chunks > TA_ARGMAX_STATIC_PAIRS / n_rows) chunks = TA_ARGMAX_STATIC_PAIRS / n_rows;
+  if (chunks < 1) chunks = 1;
+  int status = 0;
+  unsigned char* scratch = (unsigned char*)argmax_scratch_here(&status);
+  if (!scratch) return status;
+  float* partial_v = (float*)scratch;
+  int* partial_i = (int*)(scratch + TA_ARGMAX_STATIC_PAIRS * sizeof(float));
+  return ta_argmax(logits, out, partial_v, partial_i, n_rows, vocab, chunks, stream);
 }
 
 // ------------------------------------------------------------------------------------------------
