@@ -55,7 +55,24 @@ def test_gaps_the_pattern_leaves_are_pieces_too():
     assert tok.encode("ab ab")[:1] == [256]
 
 
+def test_added_tokens_are_found_leftmost_first_and_the_longest_of_those_that_start_together():
+    # src/rank.rs:368-447
+    data = tiny_file()
+    data["added_tokens"] += [{"id": 301, "content": "<|end", "normalized": False},
+                             {"id": 302, "content": "<|endoftext|>x", "normalized": False}]
+    tok = Tokenizer.from_json(data)
+    assert tok.encode("a<|endoftext|>xb<|endq") == [ord("a"), 302, ord("b"), 301, ord("q")]
+    assert tok.encode("<|endoftext|>") == [300] and tok.encode("") == []
+    assert tok.decode(tok.encode("ab<|end<|endoftext|>")) == "ab<|end<|endoftext|>"
+    assert tok.vocab_size() == 303
+
+
 @pytest.mark.parametrize("change, word", [
+    (lambda f: f["added_tokens"].append(dict(f["added_tokens"][0], id=301)), "listed twice"),
+    (lambda f: f["added_tokens"][0].update(id=97), "token id 97 is given to"),
+    (lambda f: f["model"]["vocab"].update({"\u00ad": 400}), "spells no byte"),
+    (lambda f: f["model"].update(merges=["a b", "a b"]), "produce the same bytes"),
+    (lambda f: f["pre_tokenizer"]["pretokenizers"].pop(1), "no ByteLevel step"),
     (lambda f: f["added_tokens"][0].update(normalized=True), "normalized"),
     (lambda f: f.update(normalizer={"type": "NFKC"}), "NFC"),
     (lambda f: f.update(normalizer=None), "no normalizer"),

@@ -1,15 +1,16 @@
 """Byte-level BPE read from a Hugging Face `tokenizer.json` of the Qwen kind.
 
-Loader rules follow src/qwen.rs:143-297 of the reference: the normalizer must be NFC; the
-pre-tokenizer a Sequence with a Split step (a Regex, behaviour Isolated, not inverted) and a
-ByteLevel step without its own regex; the model BPE.  Vocabulary strings are mapped back to
-bytes through the inverse of GPT-2's `bytes_to_unicode` (src/qwen.rs:96-121); all 256 single
-bytes must be tokens; a merge's rank is its index in the list; added tokens must be
-`normalized: false` and are matched literally before anything else.
+What the file must look like is the reference's (src/qwen.rs:143-297): normalizer NFC; pre-tokenizer a
+Sequence holding a Split step (its pattern a Regex, behaviour Isolated, not inverted) and a ByteLevel
+step that brings no regex of its own; model BPE.  A vocabulary entry spells its bytes in the printable
+alphabet of byte-level BPE (src/qwen.rs:96-121): every byte value must be a token; a merge ranks by its
+place in the list and is looked up by the bytes it produces; added tokens are literals (`normalized:
+false`), found in the text before anything else.
 
-Encoding follows src/rank.rs:368-447,536-586: split out the earliest added token (the longest
-on a tie), NFC the text between, split it with the regex keeping unmatched gaps as pieces,
-and in every piece merge the adjacent pair of lowest rank (leftmost on a tie) until none is left.
+Encoding (src/rank.rs:368-447,536-586): cut the text at added tokens (leftmost first, the longest of
+those that start at the same place), bring what lies between to NFC, cut that with the regex (what the
+regex skips is a piece too), and inside every piece join the neighbouring pair of lowest rank (the
+leftmost of equals) until no pair has a rank.
 """
 from __future__ import annotations
 
@@ -29,17 +30,135 @@ class UnknownToken(TokenizerError):
         self.token = token
 
 
+# ------------------------------------------------------------------------------------ the byte alphabet
+_SELF_SPELLED = (range(0x21, 0x7F), range(0xA1, 0xAD), range(0xAE, 0x100))     # printable, kept as they are
+
+
+def _byte_alphabet() -> list[str]:
+    """The character that spells each byte value: printable Latin-1 bytes spell themselves, the other 68
+    are numbered upwards from U+0100 in byte order."""
+    spelled = [None] * 256
+    for span in _SELF_SPELLED:
+        for byte in span:
+            spelled[byte] = chr(byte)
+    following = 0x100
+    for byte in range(256):
+        if spelled[byte] is None:
+            spelled[byte] = chr(following)
+            following += 1
+    return spelled
+
+
 def bytes_to_unicode_reverse() -> dict[str, int]:
     """Character of a vocabulary string -> the byte it stands for."""
-    keep = list(range(ord("!"), ord("~") + 1)) + list(range(0xA1, 0xAD)) + list(range(0xAE, 0x100))
-    codes = list(keep)
-    extra = 0
-    for byte in range(256):
-        if byte not in keep:
-            keep.append(byte)
-            codes.append(256 + extra)
-            extra += 1
-    return {chr(code): byte for byte, code in zip(keep, codes)}
+    return {ch: byte for byte, ch in enumerate(_byte_alphabet())}
+
+
+# ------------------------------------------------------------------------------------- reading the file
+class _Section:
+    """One object of the file with a name for messages: `section["key"]` complains with the path to it."""
+
+    def __init__(self, data, path: str):
+        if not isinstance(data, dict):
+            raise TokenizerError(f"{path} is missing or not an object")
+        self.data, self.path = data, path
+
+    def get(self, key: str, default=None):
+        return self.data.get(key, default)
+
+    def want(self, key: str, value, why: str = ""):
+        found = self.data.get(key)
+        if found != value:
+            raise TokenizerError(f"{self.path}.{key} is {found!r} where {value!r} is needed" + (f" ({why})" if why else ""))
+
+    def child(self, key: str) -> "_Section":
+        return _Section(self.data.get(key), f"{self.path}.{key}")
+
+
+class _TokenizerFile:
+    """The parts of a parsed tokenizer.json that this tokenizer uses, each checked where it is read."""
+
+    def __init__(self, data: dict):
+        self.root = _Section(data, "tokenizer.json")
+        self.alphabet = bytes_to_unicode_reverse()
+
+    def check_normalizer(self) -> None:
+        if not self.root.get("normalizer"):
+            raise TokenizerError("tokenizer.json has no normalizer; texts are brought to NFC and the file must say so")
+        self.root.child("normalizer").want("type", "NFC", "no other normalisation is applied")
+
+    def split_regex(self) -> str:
+        pre = self.root.child("pre_tokenizer")
+        pre.want("type", "Sequence")
+        steps = {}
+        for index, step in enumerate(pre.get("pretokenizers") or []):
+            section = _Section(step, f"{pre.path}.pretokenizers[{index}]")
+            steps.setdefault(section.get("type"), section)
+        for kind in ("Split", "ByteLevel"):
+            if kind not in steps:
+                raise TokenizerError(f"{pre.path} has no {kind} step")
+        split, byte_level = steps["Split"], steps["ByteLevel"]
+        split.want("behavior", "Isolated", "matches and the text between them are both kept as pieces")
+        if split.get("invert"):
+            raise TokenizerError(f"{split.path}.invert is set; an inverted split is not handled")
+        pattern = split.child("pattern").get("Regex")
+        if not isinstance(pattern, str):
+            raise TokenizerError(f"{split.path}.pattern holds no Regex")
+        if byte_level.get("use_regex"):
+            raise TokenizerError(f"{byte_level.path}.use_regex is set; pieces are cut by the Split step's regex alone")
+        return pattern
+
+    def spell(self, text: str, what: str) -> bytes:
+        try:
+            return bytes(self.alphabet[ch] for ch in text)
+        except KeyError as stray:
+            raise TokenizerError(f"{what} {text!r} holds U+{ord(stray.args[0]):04X}, which spells no byte") from None
+
+    def byte_vocab(self) -> dict[bytes, int]:
+        model = self.root.child("model")
+        model.want("type", "BPE")
+        ids: dict[bytes, int] = {}
+        for text, token in (model.get("vocab") or {}).items():
+            raw = self.spell(text, "vocabulary entry")
+            if raw in ids:
+                raise TokenizerError(f"vocabulary ids {ids[raw]} and {token} spell the same bytes")
+            ids[raw] = token
+        absent = [byte for byte in range(256) if bytes([byte]) not in ids]
+        if absent:
+            raise TokenizerError(f"missing single-byte token {absent[0]}"
+                                 + (f" (and {len(absent) - 1} more)" if len(absent) > 1 else ""))
+        return ids
+
+    def merge_ranks(self, ids: dict[bytes, int]) -> dict[bytes, int]:
+        ranks: dict[bytes, int] = {}
+        for rank, entry in enumerate(self.root.child("model").get("merges") or []):
+            halves = entry.split(" ") if isinstance(entry, str) else list(entry)
+            if len(halves) == 1:
+                raise TokenizerError(f"merge {rank} ({entry!r}) has no space between its halves")
+            if len(halves) != 2 or not all(halves):
+                raise TokenizerError(f"merge {rank} ({entry!r}) is not a pair")
+            left, right = (self.spell(half, f"merge {rank}:") for half in halves)
+            for side in (left, right, left + right):
+                if side not in ids:
+                    raise TokenizerError(f"merge {rank} ({entry!r}): {side!r} is not in the vocab")
+            if left + right in ranks:
+                raise TokenizerError(f"merges {ranks[left + right]} and {rank} produce the same bytes")
+            ranks[left + right] = rank
+        return ranks
+
+    def literals(self) -> dict[str, int]:
+        found: dict[str, int] = {}
+        for index, entry in enumerate(self.root.get("added_tokens") or []):
+            item = _Section(entry, f"tokenizer.json.added_tokens[{index}]")
+            content, token = item.get("content"), item.get("id")
+            if not content or not isinstance(token, int):
+                raise TokenizerError(f"{item.path} needs a content that is not empty and an id")
+            if item.get("normalized", True):
+                raise TokenizerError(f"{item.path} ({content!r}) is normalized; added tokens are matched as literals only")
+            if content in found:
+                raise TokenizerError(f"{item.path} ({content!r}) is listed twice")
+            found[content] = token
+        return found
 
 
 class Tokenizer:
@@ -52,6 +171,9 @@ class Tokenizer:
             self.pattern = regex.compile(pattern)
         except regex.error as err:
             raise TokenizerError(f"split pattern does not compile: {err}") from None
+        # Leftmost match, and among literals that start there the longest: the alternatives are tried in order.
+        by_length = sorted(specials, key=len, reverse=True)
+        self._literal = regex.compile("|".join(regex.escape(text) for text in by_length)) if specials else None
 
     # -------------------------------------------------------------------- loading
     @classmethod
@@ -67,96 +189,24 @@ class Tokenizer:
 
     @classmethod
     def from_json(cls, data: dict) -> "Tokenizer":
-        normalizer = data.get("normalizer")
-        if not normalizer:
-            raise TokenizerError("tokenizer.json has no normalizer")
-        if normalizer.get("type") != "NFC":
-            raise TokenizerError(f"expected an NFC normalizer, found {normalizer.get('type')}")
-        pre = data.get("pre_tokenizer") or {}
-        if pre.get("type") != "Sequence":
-            raise TokenizerError(f"expected a Sequence pre-tokenizer, found {pre.get('type')}")
-        pattern = cls._split_pattern(pre)
-        model = data.get("model") or {}
-        if model.get("type") != "BPE":
-            raise TokenizerError(f"expected a BPE model, found {model.get('type')}")
-        reverse = bytes_to_unicode_reverse()
-
-        def unmap(token: str) -> bytes:
-            try:
-                return bytes(reverse[ch] for ch in token)
-            except KeyError as err:
-                raise TokenizerError(f"vocab char U+{ord(err.args[0]):04X} is not a bytes_to_unicode scalar") from None
-
-        encoder: dict[bytes, int] = {}
-        max_id = 0
-        for token, token_id in model.get("vocab", {}).items():
-            raw = unmap(token)
-            if raw in encoder:
-                raise TokenizerError(f"duplicate vocab bytes for id {token_id}")
-            encoder[raw] = token_id
-            max_id = max(max_id, token_id)
-        for byte in range(256):
-            if bytes([byte]) not in encoder:
-                raise TokenizerError(f"missing single-byte token {byte}")
-        ranks: dict[bytes, int] = {}
-        for index, merge in enumerate(model.get("merges", [])):
-            if isinstance(merge, list):
-                merge = " ".join(merge)
-            left, sep, right = merge.partition(" ")
-            if not sep:
-                raise TokenizerError(f"merge {index} has no space")
-            if not left or not right or " " in right:
-                raise TokenizerError(f"merge {index} is not two bytes_to_unicode tokens")
-            left_b, right_b = unmap(left), unmap(right)
-            if left_b not in encoder or right_b not in encoder:
-                raise TokenizerError(f"merge {index} names a token that is not in the vocab")
-            merged = left_b + right_b
-            if merged not in encoder:
-                raise TokenizerError(f"merge {index} concatenation is not in the vocab")
-            if merged in ranks:
-                raise TokenizerError(f"merge {index} repeats a byte string")
-            ranks[merged] = index
-        added = data.get("added_tokens", [])
-        for item in added:
-            max_id = max(max_id, item["id"])
-        decoder: list[bytes | None] = [None] * (max_id + 1)
-        for raw, token_id in encoder.items():
-            if decoder[token_id] is not None:
-                raise TokenizerError(f"duplicate token id {token_id}")
-            decoder[token_id] = raw
-        specials: dict[str, int] = {}
-        for item in added:
-            if item.get("normalized", True):
-                raise TokenizerError(f"added token {item['content']!r} is normalized; only normalized=false is supported")
-            if not item["content"]:
-                raise TokenizerError("added token content is empty")
-            if decoder[item["id"]] is not None:
-                raise TokenizerError(f"added token id {item['id']} already belongs to a vocab token")
-            decoder[item["id"]] = item["content"].encode("utf-8")
-            if item["content"] in specials:
-                raise TokenizerError(f"duplicate added token {item['content']!r}")
-            specials[item["content"]] = item["id"]
-        return cls(encoder, decoder, ranks, specials, pattern)
-
-    @staticmethod
-    def _split_pattern(pre: dict) -> str:
-        steps = pre.get("pretokenizers", [])
-        split = next((s for s in steps if s.get("type") == "Split"), None)
-        if split is None:
-            raise TokenizerError("pre-tokenizer has no Split step")
-        if split.get("behavior") != "Isolated":
-            raise TokenizerError(f"expected Split behavior Isolated, found {split.get('behavior')!r}")
-        if split.get("invert", False):
-            raise TokenizerError("Split invert=true is not supported")
-        pattern = (split.get("pattern") or {}).get("Regex")
-        if pattern is None:
-            raise TokenizerError("Split step has no Regex pattern")
-        byte_level = next((s for s in steps if s.get("type") == "ByteLevel"), None)
-        if byte_level is None:
-            raise TokenizerError("pre-tokenizer has no ByteLevel step")
-        if byte_level.get("use_regex", False):
-            raise TokenizerError("ByteLevel use_regex must be false; the Split step owns the regex")
-        return pattern
+        source = _TokenizerFile(data)
+        source.check_normalizer()
+        pattern = source.split_regex()
+        ids = source.byte_vocab()
+        ranks = source.merge_ranks(ids)
+        literals = source.literals()
+        # id -> bytes for both kinds of token; no id may mean two things.
+        table: dict[int, bytes] = {}
+        for raw, token in list(ids.items()) + [(text.encode("utf-8"), token) for text, token in literals.items()]:
+            if token in table:
+                raise TokenizerError(f"token id {token} is given to {table[token]!r} and to {raw!r}")
+            table[token] = raw
+        decoder: list[bytes | None] = [None] * (max(table) + 1)
+        for token, raw in table.items():
+            if token < 0:
+                raise TokenizerError(f"token id {token} is negative")
+            decoder[token] = raw
+        return cls(ids, decoder, ranks, literals, pattern)
 
     # ------------------------------------------------------------------- encoding
     def vocab_size(self) -> int:
@@ -164,54 +214,43 @@ class Tokenizer:
 
     def encode(self, text: str) -> list[int]:
         ids: list[int] = []
-        rest = text
-        while True:
-            found = self._earliest_special(rest)
-            if found is None:
-                self._push_ordinary(rest, ids)
-                return ids
-            start, token = found
-            self._push_ordinary(rest[:start], ids)
-            ids.append(self.specials[token])
-            rest = rest[start + len(token):]
+        at = 0
+        if self._literal is not None:
+            for match in self._literal.finditer(text):
+                self._encode_ordinary(text[at:match.start()], ids)
+                ids.append(self.specials[match.group()])
+                at = match.end()
+        self._encode_ordinary(text[at:], ids)
+        return ids
 
-    def _earliest_special(self, text: str):
-        best = None
-        for token in self.specials:
-            at = text.find(token)
-            if at < 0:
-                continue
-            if best is None or at < best[0] or (at == best[0] and len(token) > len(best[1])):
-                best = (at, token)
-        return best
-
-    def _push_ordinary(self, text: str, ids: list[int]) -> None:
+    def _encode_ordinary(self, text: str, ids: list[int]) -> None:
         if not text:
             return
         text = unicodedata.normalize("NFC", text)
         at = 0
         for match in self.pattern.finditer(text):
+            if match.end() == match.start():
+                continue
             if match.start() > at:
-                self._push_piece(text[at:match.start()].encode("utf-8"), ids)   # a gap is a piece too
-            if match.end() > match.start():
-                self._push_piece(match.group().encode("utf-8"), ids)
-            at = max(at, match.end())
+                self._encode_piece(text[at:match.start()].encode("utf-8"), ids)    # what the regex skipped
+            self._encode_piece(match.group().encode("utf-8"), ids)
+            at = match.end()
         if at < len(text):
-            self._push_piece(text[at:].encode("utf-8"), ids)
+            self._encode_piece(text[at:].encode("utf-8"), ids)
 
-    def _push_piece(self, piece: bytes, ids: list[int]) -> None:
-        if not piece:
+    def _encode_piece(self, piece: bytes, ids: list[int]) -> None:
+        whole = self.encoder.get(piece) if len(piece) == 1 else None
+        if whole is not None:
+            ids.append(whole)
             return
         parts = [piece[i:i + 1] for i in range(len(piece))]
         while len(parts) > 1:
-            best_rank, best_at = None, -1
-            for i in range(len(parts) - 1):
-                rank = self.ranks.get(parts[i] + parts[i + 1])
-                if rank is not None and (best_rank is None or rank < best_rank):
-                    best_rank, best_at = rank, i
-            if best_rank is None:
+            ranked = [(self.ranks.get(left + right), i) for i, (left, right) in enumerate(zip(parts, parts[1:]))]
+            ranked = [pair for pair in ranked if pair[0] is not None]
+            if not ranked:
                 break
-            parts[best_at:best_at + 2] = [parts[best_at] + parts[best_at + 1]]
+            _, at = min(ranked)                          # lowest rank; the leftmost of equal ranks
+            parts[at:at + 2] = [parts[at] + parts[at + 1]]
         ids.extend(self.encoder[part] for part in parts)
 
     # ------------------------------------------------------------------- decoding
