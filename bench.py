@@ -54,7 +54,8 @@ def weight_bytes_per_step(model) -> int:
     tensors = [decoder.head]
     for block in decoder.blocks:
         for part in (block.mixer_norm, block.mixer, block.feed_forward_norm, block.feed_forward):
-            tensors.extend(v for v in vars(part).values() if isinstance(v, torch.Tensor))
+            if part is not None:
+                tensors.extend(v for v in vars(part).values() if isinstance(v, torch.Tensor))
     tensors.extend(v for v in vars(decoder.final_norm).values() if isinstance(v, torch.Tensor))
     for tensor in tensors:
         if tensor.data_ptr() not in seen:

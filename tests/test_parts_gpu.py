@@ -532,3 +532,157 @@ def test_toy_routed_architecture(tmp_path, dtype):
         err = float((got[rid] - want).abs().max())
         assert err <= (3e-5 if dtype == "float32" else 4e-2) * max(1.0, float(want.abs().max())), (rid, err)
     engine.cache.check_invariants()
+
+
+# ------------------------------------------------------------------------------------------------
+# A third toy architecture: layers that lack a sub-layer, and a norm and a position encoding defined here
+# that say themselves that the fused decode kernels can compute them.  Layer 0 is attention alone, layer 1 a
+# feed-forward alone, layer 2 has both.
+def register_chain_toys():
+    from tokenizer_amd.config import get_architecture, register_architecture, registered_architectures
+    from tokenizer_amd.config.base import ModelConfig
+    if "ToyChainForCausalLM" in registered_architectures():
+        return get_architecture("ToyChainForCausalLM").config_class
+    from tokenizer_amd.parts import (NORMS, POSITIONS, FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, Norm,
+                                     NormFold, NormSpec, PositionEncoding, PositionSpec, ScheduleEntry, StoreEpilogue,
+                                     TensorSpec)
+
+    if "rms_one_plus" not in NORMS.kinds():
+        @NORMS.register("rms_one_plus")
+        class OnePlus(Norm):
+            """x / sqrt(mean(x^2) + eps) * (1 + gain): the file holds the gain's distance from one."""
+            graph_safe = True
+
+            def __init__(self, spec, tensors, rt):
+                self.size, self.eps, self.rt = spec.size, float(spec.eps), rt
+                self.scale = (1.0 + tensors["gain"].float()).contiguous()
+
+            @staticmethod
+            def tensor_specs(spec):
+                return {"gain": TensorSpec((spec.size,), std=0.3, role="vector")}
+
+            def fold(self):
+                return NormFold(self.scale, self.eps)
+
+            def apply(self, residual, delta, rows=None):
+                n_rows = residual.shape[0] if rows is None else rows.numel()
+                out = torch.empty((n_rows, self.size), dtype=self.rt.dtype, device=residual.device)
+                return self.rt.ops.add_rmsnorm(residual, delta, self.scale, self.eps, out, rows,
+                                               store_residual=rows is None)
+
+    if "rope_half_speed" not in POSITIONS.kinds():
+        @POSITIONS.register("rope_half_speed")
+        class HalfSpeed(PositionEncoding):
+            """The half-split rotation with every angle halved: another table, the same kernels."""
+            graph_safe = True
+
+            def __init__(self, spec, rt):
+                self.rt = rt
+                cos, sin = half_speed_tables(spec.theta, spec.head_dim, spec.max_positions)
+                self.cos_sin = torch.cat([cos, sin], dim=1).contiguous().to(rt.device)
+
+            def epilogue(self):
+                return StoreEpilogue(self.cos_sin)
+
+            def encode_and_store(self, qkv, bias, n_q, n_kv, head_dim, ctx, cache):
+                slots = ctx.slots[cache.group] if cache.writes else None
+                self.rt.ops.rope_store(qkv, bias, ctx.positions, self.cos_sin, slots,
+                                       cache.k_pages if cache.writes else None,
+                                       cache.v_pages if cache.writes else None, n_q, n_kv, head_dim)
+
+    @dataclasses.dataclass(frozen=True)
+    class ChainConfig(ModelConfig):
+        vocab_size: int
+        hidden_size: int
+        heads: int
+        inner: int
+
+    def chain_spec(cfg):
+        d = cfg.hidden_size // cfg.heads
+        norm = NormSpec("rms_one_plus", cfg.hidden_size, 1e-4)
+        mixer = MixerSpec("gqa_attention", cfg.hidden_size, cfg.heads, 1, d, qkv_bias=True,
+                          position=PositionSpec("rope_half_speed", d, 100.0, 256))
+        ff = FeedForwardSpec("gated_dense", cfg.hidden_size, cfg.inner, "silu")
+        layers = (LayerSpec("pre_norm", mixer, None, norm, None, mixer_prefix="l.0.mix", mixer_norm_prefix="l.0.n1"),
+                  LayerSpec("pre_norm", None, ff, None, norm, feed_forward_prefix="l.1.ff", feed_forward_norm_prefix="l.1.n2"),
+                  LayerSpec("pre_norm", mixer, ff, norm, norm, "l.2.mix", "l.2.ff", "l.2.n1", "l.2.n2"))
+        return ModelSpec("ToyChainForCausalLM", cfg.vocab_size, cfg.hidden_size, 256, "emb.weight", layers,
+                         tuple(ScheduleEntry(i) for i in range(3)), norm, "final", tied_head=True, head_name="head.weight")
+
+    register_architecture("ToyChainForCausalLM", ChainConfig, chain_spec)
+    return ChainConfig
+
+
+def half_speed_tables(theta, d, n_positions):
+    inv_freq = torch.tensor([1.0 / (float(theta) ** (i / d)) for i in range(0, d, 2)], dtype=torch.float64).float()
+    angles = torch.arange(n_positions, dtype=torch.float32)[:, None] * 0.5 * inv_freq[None, :]
+    return angles.cos(), angles.sin()
+
+
+def chain_plain_logits(tensors, ids, heads):
+    t = {k: v.float() for k, v in tensors.items()}
+    hidden = t["emb.weight"].shape[1]
+    d, n = hidden // heads, len(ids)
+    pos = list(range(n))
+    cos, sin = half_speed_tables(100.0, d, 256)
+    norm = lambda x, name: plain.rms_norm(x, 1.0 + t[f"{name}.gain"], 1e-4)
+
+    def attention(x, i):
+        named = {f"a.{k[len(f'l.{i}.mix.'):]}": v for k, v in t.items() if k.startswith(f"l.{i}.mix.")}
+        return x + plain.self_attention(norm(x, f"l.{i}.n1"), named, "a", heads, 1, d, cos, sin, pos, None)
+
+    def feed_forward(x, i):
+        named = {f"m.{k[len(f'l.{i}.ff.'):]}": v for k, v in t.items() if k.startswith(f"l.{i}.ff.")}
+        return x + plain.mlp(norm(x, f"l.{i}.n2"), named, "m")
+
+    x = feed_forward(attention(feed_forward(attention(t["emb.weight"][ids], 0), 1), 2), 2)
+    return norm(x, "final") @ t["emb.weight"].t()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_without_a_sub_layer_and_parts_that_offer_their_fused_form(tmp_path, dtype):
+    import trace_tools as tt
+    import tokenizer_amd as ta
+    from safetensors.torch import load_file
+    from tokenizer_amd.engine import Engine, load_model
+
+    config_cls = register_chain_toys()
+    cfg = config_cls.from_dict({"vocab_size": 72, "hidden_size": 64, "heads": 2, "inner": 40})
+    folder = ta.write_random_model(cfg, 8, str(tmp_path / "chain"))
+    tensors = load_file(folder + "/model.safetensors")
+    assert "l.0.mix.q_proj.weight" in tensors and "l.1.ff.down_proj.weight" in tensors and "l.2.n2.gain" in tensors
+    assert not any(k.startswith(("l.0.ff", "l.0.n2", "l.1.mix", "l.1.n1")) for k in tensors)
+    model = load_model(folder, dtype)
+    assert [n.kind for n in model.cache_needs] == ["full", "none", "full"] and model.decoder.graph_safe
+    ops = model.runtime.ops
+    folded = {"qkv": 0, "gated": 0}
+    inner_qkv, inner_gated = ops.fused_norm_qkv_rope, ops.fused_norm_gated
+
+    def count_qkv(rows, norm_weight, *rest, **kw):
+        folded["qkv"] += norm_weight is not None
+        return inner_qkv(rows, norm_weight, *rest, **kw)
+
+    def count_gated(rows, norm_weight, *rest, **kw):
+        folded["gated"] += norm_weight is not None
+        return inner_gated(rows, norm_weight, *rest, **kw)
+
+    ops.fused_norm_qkv_rope, ops.fused_norm_gated = count_qkv, count_gated
+    try:
+        requests = {f"r{i}": random_ids(72, n, 130 + i) for i, n in enumerate([2, 31, 64, 17, 40])}
+        steps = tt.mixed(requests, 11, max_live=3)
+        engine = Engine(model, max_tokens=tt.peak_tokens(steps), max_requests=3)
+        engine.pools.poison()
+        got = tt.run_in_process(engine, steps)
+    finally:
+        del ops.fused_norm_qkv_rope, ops.fused_norm_gated          # back to the class's methods
+    for rid, ids in requests.items():
+        want = chain_plain_logits(tensors, ids, 2)
+        err = float((got[rid] - want).abs().max())
+        assert err <= (3e-5 if dtype == "float32" else 4e-2) * max(1.0, float(want.abs().max())), (rid, err)
+    engine.cache.check_invariants()
+    if dtype == "bfloat16":
+        # Steps of few rows took the norm into the products' prologue and the rotation into their epilogue,
+        # for parts the package has never heard of.
+        assert folded["qkv"] >= 2 and folded["gated"] >= 2, folded
+    else:
+        assert folded == {"qkv": 0, "gated": 0}

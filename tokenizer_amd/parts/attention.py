@@ -7,8 +7,6 @@ import torch
 
 from .base import can_fuse_decode as _can_fuse
 from .base import MIXERS, POSITIONS, Mixer, Runtime
-from .norm import RMSNorm
-from .position import NoPosition, RotaryHalfSplit
 from .spec import CacheNeed, MixerSpec, PositionSpec, TensorSpec
 
 
@@ -65,19 +63,21 @@ class GQAttention(Mixer):
         """Decode batches of few bfloat16 rows: norm + q/k/v product + bias + rotation + cache write in one
         kernel, attention, then the output product added straight into the residual stream."""
         ops = self.runtime.ops
-        fused = (delta is None and type(norm) is RMSNorm and type(self.position) in (NoPosition, RotaryHalfSplit)
-                 and self.d % 32 == 0 and cache.group is not None
+        # The norm and the position encoding say themselves whether they have the form the fused kernels compute.
+        fold = norm.fold() if delta is None else None
+        behind = self.position.epilogue() if fold is not None else None
+        fused = (behind is not None and self.d % 32 == 0 and cache.group is not None
                  and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
             # The output is handed on as a delta: an output product whose K is cut over workgroups may stay in
             # parts, and the norm that takes it next adds them in its own kernel.
             return self._run(norm.apply(residual, delta), ctx, cache, pending=getattr(ops, "takes_pending", False))
         if getattr(ops, "fold_norm", lambda hidden: True)(residual.shape[1]):
-            rows, norm_weight = residual, norm.weight
+            rows, norm_weight = residual, fold.weight
         else:                       # a wide model: the norm's own kernel once, not again in every workgroup
             rows, norm_weight = norm.apply(residual, None), None
-        q = ops.fused_norm_qkv_rope(rows, norm_weight, norm.eps, self.w_qkv, self.b_qkv, ctx.positions,
-                                    self.position.table(), ctx.slots[cache.group] if cache.writes else None,
+        q = ops.fused_norm_qkv_rope(rows, norm_weight, fold.eps, self.w_qkv, self.b_qkv, ctx.positions,
+                                    behind.cos_sin, ctx.slots[cache.group] if cache.writes else None,
                                     cache.k_pages, cache.v_pages, self.n_q, self.n_kv, self.d)
         mixed = torch.empty((q.shape[0], self.n_q * self.d), dtype=q.dtype, device=q.device)
         ops.paged_attention(q, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
@@ -92,10 +92,12 @@ class GQAttention(Mixer):
     def _run(self, x, ctx, cache, pending: bool):
         ops = self.runtime.ops
         can = getattr(ops, "can_rope_store", None)
-        if (can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and type(self.position) in (NoPosition, RotaryHalfSplit)
-                and self.d % 32 == 0 and cache.group is not None):
+        behind = None
+        if can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and self.d % 32 == 0 and cache.group is not None:
+            behind = self.position.epilogue()
+        if behind is not None:
             # A few dozen rows: bias, rotation and the cache write ride in the projection's epilogue.
-            qkv = ops.fused_norm_qkv_rope(x, None, 0.0, self.w_qkv, self.b_qkv, ctx.positions, self.position.table(),
+            qkv = ops.fused_norm_qkv_rope(x, None, 0.0, self.w_qkv, self.b_qkv, ctx.positions, behind.cos_sin,
                                           ctx.slots[cache.group] if cache.writes else None, cache.k_pages,
                                           cache.v_pages, self.n_q, self.n_kv, self.d)
         else:

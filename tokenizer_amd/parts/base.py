@@ -7,6 +7,8 @@ Interfaces
 ----------
 Norm            tensor_specs(spec) -> {local name: TensorSpec}
                 apply(residual, delta, rows=None) -> normalised rows in the compute dtype.
+                Optional: fold() -> NormFold, if the norm is x / sqrt(mean(x^2) + eps) * weight for some weight:
+                a mixer or feed-forward may then take it into the prologue of its own product.
                 `residual` is the float32 stream [T, H]; `delta` (or None) is added to it first and,
                 unless `rows` picks a subset, the sum is stored back.  `delta` may also be a product still
                 in parts (`kernels.PendingSum`, which the kernel library's `add_rmsnorm` takes as it is): a
@@ -14,13 +16,16 @@ Norm            tensor_specs(spec) -> {local name: TensorSpec}
 PositionEncoding
                 encode_and_store(qkv, geometry, ctx, cache, bias): adds the projection bias, encodes
                 the query and key heads in place and writes keys and values of this step into `cache`.
+                Optional: epilogue() -> StoreEpilogue, if the encoding is a rotation of half-split pairs by a
+                table (or nothing at all): the fused projection then does it, and the store, in its epilogue.
 Mixer           tensor_specs(spec), cache_need(spec) -> CacheNeed
                 forward(x [T, H], ctx: StepContext, cache: LayerCache) -> [T, H] in the compute dtype.
                 Optional: forward_normed(residual, delta, norm, ctx, cache) to fold the norm before it and the
                 residual add after it into its own kernels (returns None when it added its output itself; what
                 it returns is only ever handed to a norm as its delta, so it may be a product still in parts).
 FeedForward     tensor_specs(spec); forward(x [T, H], ctx) -> [T, H]; optional forward_normed likewise.
-Block           arranges two norms, a mixer and a feed-forward around the residual stream:
+Block           arranges two norms, a mixer and a feed-forward around the residual stream (either sub-layer may
+                be absent: None for the part and its norm):
                 forward(residual, delta, ctx, cache) -> delta still to be added.
 """
 from __future__ import annotations
@@ -84,15 +89,41 @@ class Part:
         return {}
 
 
+@dataclasses.dataclass
+class NormFold:
+    """A norm in the form the fused products take into their prologue: y = x / sqrt(mean(x^2) + eps) * weight,
+    with `weight` float32 [H] on the device.  A norm of that form says so through `Norm.fold()`, whatever its
+    class and however it derives the weight from its tensors."""
+    weight: torch.Tensor
+    eps: float
+
+
+@dataclasses.dataclass
+class StoreEpilogue:
+    """What the fused q/k/v projection can do behind its bias: rotate the half-split pairs of every query and
+    key head by the row of `cos_sin` (float32 [positions, d]: cos half, then sin half) at the token's position,
+    `cos_sin` None meaning no rotation, and write keys and values into their pages.  A position encoding that is
+    of that form says so through `PositionEncoding.epilogue()`."""
+    cos_sin: torch.Tensor | None
+
+
 class Norm(Part):
     def apply(self, residual: torch.Tensor, delta: torch.Tensor | None,
               rows: torch.Tensor | None = None) -> torch.Tensor:
         raise NotImplementedError
 
+    def fold(self) -> NormFold | None:
+        """The norm as a product's prologue can compute it, or None (the parts then call `apply`)."""
+        return None
+
 
 class PositionEncoding(Part):
     def encode_and_store(self, qkv, bias, n_q: int, n_kv: int, head_dim: int, ctx, cache) -> None:
         raise NotImplementedError
+
+    def epilogue(self) -> StoreEpilogue | None:
+        """The encoding as the fused projection's epilogue can apply it, or None (`encode_and_store` is called)."""
+        return None
 
 
 class Mixer(Part):

@@ -10,6 +10,7 @@ class PreNormBlock(Block):
 
     The residual stream is float32.  Each sub-layer's output is handed on as a pending `delta`
     so that the add fuses into the next norm; a part that added its output itself hands on None.
+    A sub-layer that the layer does not have (None) is passed over.
     """
     graph_safe = True
 
@@ -19,5 +20,8 @@ class PreNormBlock(Block):
         self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
 
     def forward(self, residual, delta, ctx, cache):
-        mixed = self.mixer.forward_normed(residual, delta, self.mixer_norm, ctx, cache)
-        return self.feed_forward.forward_normed(residual, mixed, self.feed_forward_norm, ctx)
+        if self.mixer is not None:
+            delta = self.mixer.forward_normed(residual, delta, self.mixer_norm, ctx, cache)
+        if self.feed_forward is not None:
+            delta = self.feed_forward.forward_normed(residual, delta, self.feed_forward_norm, ctx)
+        return delta

@@ -5,7 +5,6 @@ import torch
 
 from .base import can_fuse_decode as _can_fuse
 from .base import FEED_FORWARDS, FeedForward, Runtime
-from .norm import RMSNorm
 from .spec import FeedForwardSpec, TensorSpec
 
 
@@ -45,16 +44,15 @@ class GatedDense(FeedForward):
         """Decode batches of few bfloat16 rows: norm + gate/up product + activation in one kernel, then the
         down product added straight into the residual stream."""
         ops = self.runtime.ops
-        fused = (delta is None and type(norm) is RMSNorm
-                 and _can_fuse(ops, residual, self.runtime.dtype))
-        if not fused:
+        fold = norm.fold() if delta is None else None      # the norm says whether it has the form the kernel computes
+        if fold is None or not _can_fuse(ops, residual, self.runtime.dtype):
             # The output is handed on as a delta: a down product whose K is cut over workgroups may stay in
             # parts, and the norm that takes it next adds them in its own kernel.
             return self._run(norm.apply(residual, delta), pending=getattr(ops, "takes_pending", False))
         if getattr(ops, "fold_norm", lambda hidden: True)(residual.shape[1]):
-            act = ops.fused_norm_gated(residual, norm.weight, norm.eps, self.w_gate_up)
+            act = ops.fused_norm_gated(residual, fold.weight, fold.eps, self.w_gate_up)
         else:                       # a wide model: the norm's own kernel once, not again in every workgroup
-            act = ops.fused_norm_gated(norm.apply(residual, None), None, norm.eps, self.w_gate_up)
+            act = ops.fused_norm_gated(norm.apply(residual, None), None, fold.eps, self.w_gate_up)
         ops.linear_add(act, self.w_down, None, residual)
         return None
 

@@ -17,12 +17,14 @@ def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
     """Every tensor name the model reads from the weight file, with its shape."""
     out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size), std=spec.embedding_std)}
     for layer in spec.layers:
-        out.update(_prefixed(layer.mixer_norm_prefix, NORMS.get(layer.mixer_norm.kind).tensor_specs(layer.mixer_norm)))
-        out.update(_prefixed(layer.mixer_prefix, MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer)))
-        out.update(_prefixed(layer.feed_forward_norm_prefix,
-                             NORMS.get(layer.feed_forward_norm.kind).tensor_specs(layer.feed_forward_norm)))
-        out.update(_prefixed(layer.feed_forward_prefix,
-                             FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward)))
+        if layer.mixer is not None:
+            out.update(_prefixed(layer.mixer_norm_prefix, NORMS.get(layer.mixer_norm.kind).tensor_specs(layer.mixer_norm)))
+            out.update(_prefixed(layer.mixer_prefix, MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer)))
+        if layer.feed_forward is not None:
+            out.update(_prefixed(layer.feed_forward_norm_prefix,
+                                 NORMS.get(layer.feed_forward_norm.kind).tensor_specs(layer.feed_forward_norm)))
+            out.update(_prefixed(layer.feed_forward_prefix,
+                                 FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward)))
     out.update(_prefixed(spec.final_norm_prefix, NORMS.get(spec.final_norm.kind).tensor_specs(spec.final_norm)))
     if not spec.tied_head:
         out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
@@ -30,8 +32,9 @@ def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
 
 
 def cache_needs(spec: ModelSpec) -> list[CacheNeed]:
-    """What each layer's mixer asks of the cache manager, by layer index."""
-    return [MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) for layer in spec.layers]
+    """What each layer's mixer asks of the cache manager, by layer index (a layer without a mixer: nothing)."""
+    return [MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) if layer.mixer is not None else CacheNeed()
+            for layer in spec.layers]
 
 
 def _strip(prefix: str, tensors: dict[str, torch.Tensor]) -> dict[str, torch.Tensor]:
@@ -58,17 +61,21 @@ class DecoderModel:
         self.embedding = tensors[spec.embedding_name]
         self.blocks = []
         for layer in spec.layers:
-            mixer_norm = NORMS.get(layer.mixer_norm.kind)(layer.mixer_norm, _strip(layer.mixer_norm_prefix, tensors), runtime)
-            mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _strip(layer.mixer_prefix, tensors), runtime)
-            ff_norm = NORMS.get(layer.feed_forward_norm.kind)(layer.feed_forward_norm,
-                                                              _strip(layer.feed_forward_norm_prefix, tensors), runtime)
-            feed_forward = FEED_FORWARDS.get(layer.feed_forward.kind)(layer.feed_forward,
-                                                                     _strip(layer.feed_forward_prefix, tensors), runtime)
+            mixer_norm = mixer = ff_norm = feed_forward = None
+            if layer.mixer is not None:
+                mixer_norm = NORMS.get(layer.mixer_norm.kind)(layer.mixer_norm, _strip(layer.mixer_norm_prefix, tensors), runtime)
+                mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _strip(layer.mixer_prefix, tensors), runtime)
+            if layer.feed_forward is not None:
+                ff_norm = NORMS.get(layer.feed_forward_norm.kind)(layer.feed_forward_norm,
+                                                                  _strip(layer.feed_forward_norm_prefix, tensors), runtime)
+                feed_forward = FEED_FORWARDS.get(layer.feed_forward.kind)(layer.feed_forward,
+                                                                         _strip(layer.feed_forward_prefix, tensors), runtime)
             self.blocks.append(BLOCKS.get(layer.block)(mixer_norm, mixer, ff_norm, feed_forward))
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)
         self.head = self.embedding if spec.tied_head else tensors[spec.head_name]
-        parts = [self.final_norm] + [p for b in self.blocks for p in (b, b.mixer_norm, b.mixer, b.feed_forward_norm,
-                                                                      b.feed_forward) if hasattr(b, "mixer")]
+        parts = [self.final_norm] + [p for b in self.blocks if hasattr(b, "mixer")
+                                     for p in (b, b.mixer_norm, b.mixer, b.feed_forward_norm, b.feed_forward)
+                                     if p is not None]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts) and \
             all(hasattr(b, "mixer") for b in self.blocks)
 

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import NORMS, Norm, Runtime
+from .base import NORMS, Norm, NormFold, Runtime
 from .spec import NormSpec, TensorSpec
 
 
@@ -21,6 +21,9 @@ class RMSNorm(Norm):
     @staticmethod
     def tensor_specs(spec: NormSpec) -> dict[str, TensorSpec]:
         return {"weight": TensorSpec((spec.size,), init="ones", role="vector")}
+
+    def fold(self):
+        return NormFold(self.weight, self.eps)
 
     def apply(self, residual, delta, rows=None):
         n_rows = residual.shape[0] if rows is None else rows.numel()

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import POSITIONS, PositionEncoding, Runtime
+from .base import POSITIONS, PositionEncoding, Runtime, StoreEpilogue
 from .spec import PositionSpec
 
 
@@ -18,6 +18,13 @@ class NoPosition(PositionEncoding):
 
     def table(self):
         return None
+
+    def epilogue(self):
+        # A subclass that encodes in its own way inherits this method but not the promise: it has to offer an
+        # epilogue of its own (or none).
+        if type(self).encode_and_store is not NoPosition.encode_and_store:
+            return None
+        return StoreEpilogue(self.table())
 
     def encode_and_store(self, qkv, bias, n_q, n_kv, head_dim, ctx, cache):
         slots = ctx.slots[cache.group] if cache.writes else None

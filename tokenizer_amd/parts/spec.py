@@ -94,16 +94,29 @@ class FeedForwardSpec:
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    """One layer: which block arrangement, which parts, and their tensor name prefixes."""
+    """One layer: which block arrangement, which parts, and their tensor name prefixes.
+
+    Either sub-layer may be absent (None for the part and for its norm; at least one is there): a layer of a
+    mixer alone, or of a feed-forward alone.  Since the schedule is a list of layers, any chain of sub-layers
+    (two mixers before one feed-forward, say) is a run of such layers.
+    """
     block: str                    # "pre_norm", ...
-    mixer: MixerSpec
-    feed_forward: FeedForwardSpec
-    mixer_norm: NormSpec
-    feed_forward_norm: NormSpec
-    mixer_prefix: str
-    feed_forward_prefix: str
-    mixer_norm_prefix: str
-    feed_forward_norm_prefix: str
+    mixer: MixerSpec | None
+    feed_forward: FeedForwardSpec | None
+    mixer_norm: NormSpec | None
+    feed_forward_norm: NormSpec | None
+    mixer_prefix: str = ""
+    feed_forward_prefix: str = ""
+    mixer_norm_prefix: str = ""
+    feed_forward_norm_prefix: str = ""
+
+    def __post_init__(self):
+        if self.mixer is None and self.feed_forward is None:
+            raise ValueError("a layer needs a mixer or a feed-forward")
+        for part, norm, what in ((self.mixer, self.mixer_norm, "mixer"),
+                                 (self.feed_forward, self.feed_forward_norm, "feed-forward")):
+            if (part is None) != (norm is None):
+                raise ValueError(f"a layer's {what} and its norm are there together or not at all")
 
 
 @dataclasses.dataclass(frozen=True)
