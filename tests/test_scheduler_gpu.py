@@ -90,3 +90,52 @@ def test_portions_of_long_prompts_replay_graphs_narrower_than_their_tables(tmp_p
     for use_graphs in (True, False):
         for prompt, got in zip(prompts, tokens[use_graphs]):
             check_greedy(cfg, tensors, prompt, got, dtype, 6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_back_to_back_give_what_single_steps_give(model_folders, dtype):
+    """Greedy decoding runs in bursts of steps whose ids stay on the device (the host reads them one step late).
+    A sequence that meets its end-of-sequence id, or a stop string, in the middle of a burst ends there, the
+    others keep the token of the step that was already under way, and every request gets what it gets with one
+    step at a time."""
+    from tokenizer_amd.engine import Generated, GenerateParams, Scheduler, SchedulerConfig, StopReason
+    name = "B"
+    cfg, tensors = plain.load_folder(model_folders[name])
+    vocab = cfg["vocab_size"]
+    prompts = [random_ids(vocab, n, 500 + n) for n in (7, 19, 33, 4, 12)]
+    budgets = [40, 25, 40, 9, 33]
+    want = [plain.greedy_generate(cfg, tensors, p, n) for p, n in zip(prompts, budgets)]
+    # An id that the first request meets for the first time some steps in: it ends there; others may meet it too.
+    ends_at = next(j for j in range(5, 40) if want[0][j] not in want[0][:j])
+    eos = want[0][ends_at]
+    token_bytes = lambda token: bytes([65 + token % 26])
+    stop = bytes([65 + want[2][20] % 26, 65 + want[2][21] % 26]).decode()    # two letters the third request spells
+
+    def run(burst):
+        eng = engine_for(model_folders[name], dtype, num_pages=40, max_requests=4)
+        eng.pools.poison()
+        sched = Scheduler(eng, SchedulerConfig(max_batch_size=4, num_blocks=40, prefix_cache=False, decode_burst=burst))
+        rids = []
+        for i, (prompt, budget) in enumerate(zip(prompts, budgets)):
+            params = GenerateParams.greedy(budget)
+            params.eos = [eos]
+            if i == 2:
+                params.stop = [stop]
+            rids.append(sched.add_request(prompt, params, token_bytes=token_bytes))
+        results = sched.run()
+        sched.assert_idle()
+        return [results[rid] for rid in rids], sched.stats
+
+    bursts, stats = run(16)
+    singles, single_stats = run(1)
+    assert stats.steps == single_stats.steps or dtype == "bfloat16"
+    for i, (a, b) in enumerate(zip(bursts, singles)):
+        assert isinstance(a, Generated) and isinstance(b, Generated)
+        if dtype == "float32":
+            assert (a.tokens, a.reason, a.text, a.completion_tokens) == (b.tokens, b.reason, b.text, b.completion_tokens), i
+            cut = want[i].index(eos) if eos in want[i] else len(want[i])
+            assert a.tokens[:cut] == want[i][:len(a.tokens[:cut])] and len(a.tokens) <= cut
+    if dtype == "float32":
+        assert bursts[0].reason == StopReason.Eos and len(bursts[0].tokens) == ends_at
+        assert bursts[2].reason in (StopReason.StopString, StopReason.Eos)
+        assert any(r.reason == StopReason.MaxTokens for r in bursts)

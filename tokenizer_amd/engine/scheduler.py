@@ -39,6 +39,7 @@ class SchedulerConfig:
     prefix_cache: bool = True
     max_num_batched_tokens: int = 2048
     prefill_chunk: int | None = None
+    decode_burst: int = 16       # greedy decode steps that may run back to back without the host in between
 
 
 @dataclasses.dataclass
@@ -197,7 +198,11 @@ class Scheduler:
         plan = [(self.sequences[int(planned[4 * i])], int(planned[4 * i + 1]), int(planned[4 * i + 2]),
                  bool(planned[4 * i + 3])) for i in range(n_planned)]
         if plan:
-            self._run(plan)
+            burst = self._burst_length(plan)
+            if burst > 1:
+                self._run_burst(plan, burst)
+            else:
+                self._run(plan)
         self._note_peaks()
         return bool(plan) or n_preempted > 0
 
@@ -255,6 +260,63 @@ class Scheduler:
         for seq, _, _, completes in plan:
             if seq.result is None and completes and seq.params.max_tokens == 0:
                 self._finish(seq, seq.cursor.finish_without_sample(seq.on_chunk))
+
+    # ---------------------------------------------------------------------- bursts
+    def _burst_length(self, plan: list[tuple[Sequence, int, int, bool]]) -> int:
+        """How many decode steps may follow each other on the device without a decision of the host between them:
+        more than one only when the step is nothing but greedy decoding (the ids a step picks feed the next one
+        there, `Engine.decode_greedy`), nothing waits that could join, no sequence reaches its last token before
+        the burst's last step, and the pages for all those tokens are there now."""
+        burst = min(self.config.decode_burst, 64)
+        if burst < 2 or not getattr(self.engine, "use_graphs", False) or not hasattr(self.engine, "decode_greedy"):
+            return 1
+        if self._get(_WAITING) and len(plan) < self.config.max_batch_size:
+            return 1                     # the queue's front waits for pages: a finished sequence should let it in at once
+        for seq, first, count, completes in plan:
+            if count != 1 or first < seq.prompt_len or not completes or not seq.cursor.is_greedy:
+                return 1
+            burst = min(burst, seq.params.max_tokens - seq.cursor.produced)
+        if burst < 2:
+            return 1
+        for seq, first, _, _ in plan:
+            if not self.cache.reserve(seq.id, first + burst):       # tokens first .. first + burst - 1 get their pages
+                return 1                  # (pages some of them took already are theirs a few steps early, no more)
+        return burst
+
+    def _run_burst(self, plan: list[tuple[Sequence, int, int, bool]], burst: int) -> None:
+        """`burst` greedy decode steps of the planned sequences back to back.  Ids reach the host one step late;
+        when one of them ends a sequence (end-of-sequence id, stop string, the caller's callback), the step after
+        it is already on its way: the others keep its tokens, the finished sequence's one is dropped."""
+        seqs = [seq for seq, _, _, _ in plan]
+        tokens = [self._tokens(seq.id, first, 1)[0] for seq, first, _, _ in plan]
+        handled = 0
+        started = time.perf_counter()
+
+        def take(ids) -> bool:
+            nonlocal handled, started
+            now = time.perf_counter()
+            elapsed, started = now - started, now
+            handled += 1
+            live = [seq for seq in seqs if seq.result is None]
+            go_on = True
+            self.stats.steps += 1
+            self.stats.tokens_forwarded += len(live)
+            for seq, token in zip(seqs, ids):
+                if seq.result is not None:
+                    continue              # ended earlier in this burst: what the step already under way picked for it is dropped
+                seq.decode += elapsed / len(live)
+                self._lib.ta_sched_commit(self._core, seq.id, 1)
+                outcome = seq.cursor.push_token(int(token), seq.token_bytes, seq.on_chunk)
+                if isinstance(outcome, Sampled):
+                    self._finish(seq, outcome)
+                    go_on = False
+                else:
+                    self._lib.ta_sched_append_token(self._core, seq.id, int(outcome))
+            return go_on
+
+        picked = self.engine.decode_greedy([seq.id for seq in seqs], tokens, burst, on_step=lambda k, ids: take(ids))
+        for ids in picked[handled:]:      # the step that was under way when a sequence ended
+            take(ids)
 
     def _finish(self, seq: Sequence, done: Sampled) -> None:
         seq.result = Generated(done.tokens, done.text, done.chunks, done.reason, done.completion_tokens,
