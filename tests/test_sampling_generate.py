@@ -100,7 +100,7 @@ def test_stop_hold_releases_a_suffix_that_was_not_the_stop():
     held = StopHold()
     assert held.push("aba", ["abc"]) == (False, "ab")
     assert held.push("bc", ["abc"]) == (True, "")
-    assert held.full[:held.emitted] == "ab"
+    assert held.handed_out == 2 and held.tail == "" and held.push("more", ["abc"]) == (True, "")
 
 
 # ---- generation loop -----------------------------------------------------------------------------

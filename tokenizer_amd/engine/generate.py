@@ -70,52 +70,59 @@ def validate(params: GenerateParams) -> None:
         raise SampleError("stop strings must be non-empty")
 
 
-def earliest_stop(text: str, stops: list[str]) -> int | None:
-    found = None
-    for stop in stops:
-        pos = text.find(stop)
-        if pos >= 0 and (found is None or pos < found):
-            found = pos
-    return found
-
-
-def prefix_hold(text: str, stops: list[str]) -> int:
-    """Length of the longest suffix of `text` that is a proper prefix of some stop string."""
-    hold = 0
-    for stop in stops:
-        for length in range(1, min(len(text), len(stop) - 1) + 1):
-            if text.endswith(stop[:length]):
-                hold = max(hold, length)
-    return hold
-
-
 class StopHold:
-    """The decoded text and how much of it has been handed out.  A suffix that may still grow into a
-    stop string is held back; a completed stop string ends the stream and is never shown."""
+    """Decoded text on its way out, with stop strings watched for (behaviour of generate.rs:433-501).
+
+    Only the text that has not been handed out yet is kept: the `tail`.  After every push it is the longest end
+    of the text that could still be the beginning of a stop string, and nothing else; so a stop string, which
+    never starts inside text that was let go, is always found inside tail + new chunk, and a push costs what
+    the chunk and the stop strings are long, however much text went before.  A completed stop string ends the
+    stream: the text before it goes out, the stop string itself and what follows never do.
+    """
 
     def __init__(self):
-        self.full = ""
-        self.emitted = 0
+        self.tail = ""
+        self.handed_out = 0          # characters given to the caller so far
+        self.stopped = False
+
+    @staticmethod
+    def _first_stop(window: str, stops: list[str]) -> int:
+        """Where the earliest stop string starts in `window`, or -1."""
+        starts = [at for at in (window.find(stop) for stop in stops) if at >= 0]
+        return min(starts) if starts else -1
+
+    @staticmethod
+    def _open_end(window: str, stops: list[str]) -> int:
+        """How many characters at the end of `window` begin a stop string without completing it."""
+        longest = 0
+        for stop in stops:
+            for size in range(min(len(window), len(stop) - 1), longest, -1):
+                if window.endswith(stop[:size]):
+                    longest = size
+                    break
+        return longest
 
     def push(self, chunk: str, stops: list[str]) -> tuple[bool, str]:
-        """Returns (stopped, text safe to emit now)."""
-        self.full += chunk
-        pos = earliest_stop(self.full, stops)
-        if pos is not None:
-            emit = self.full[self.emitted:pos] if pos > self.emitted else ""
-            self.emitted = pos
-            return True, emit
-        safe = len(self.full) - prefix_hold(self.full, stops)
-        if safe < self.emitted:
-            return False, ""
-        emit = self.full[self.emitted:safe]
-        self.emitted = safe
-        return False, emit
+        """Returns (a stop string was completed, text that may go out now)."""
+        if self.stopped:
+            return True, ""
+        window = self.tail + chunk
+        cut = self._first_stop(window, stops) if stops else -1
+        if cut >= 0:
+            self.stopped, self.tail = True, ""
+            self.handed_out += cut
+            return True, window[:cut]
+        keep = self._open_end(window, stops) if stops else 0
+        out = window[:len(window) - keep]
+        self.tail = window[len(window) - keep:]
+        self.handed_out += len(out)
+        return False, out
 
     def finish(self) -> str:
-        emit = self.full[self.emitted:]
-        self.emitted = len(self.full)
-        return emit
+        """What was held back in case it grew into a stop string, now that nothing more comes."""
+        out, self.tail = self.tail, ""
+        self.handed_out += len(out)
+        return out
 
 
 TokenBytes = Callable[[int], bytes]
