@@ -71,43 +71,61 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   for (int db = 0; db < DB; ++db) acc[db] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  // A block of 32 keys (two tiles of 16, each inside one page) as the matrix instructions want it.
+  // A block of 32 keys as the matrix instructions want it.  Key kb + k is index k of the second product's
+  // contraction (lane group g holds k = 8g .. 8g+7), so a lane's eight values of a row of V^T are sixteen
+  // contiguous bytes of one page: one load.  For that the first product's two instructions take the keys in an
+  // order of their own: row r of instruction t is key kb + 8 (r / 4) + 4 t + r % 4, whose score then lands in
+  // the lane group that holds that key in the second product.  Keys kb .. kb+15 lie in one page, kb+16 .. kb+31
+  // in one (page sizes are multiples of 16).
   struct KeyBlock {
     bf16x8 kf[2][KS];
-    union VFrag { uint2 half[2]; bf16x8 v; } vf[DB];
-    bool active[2];
+    union VFrag { uint4 bits; bf16x8 v; } vf[DB];
+    bool active;
   };
   // All loads of a block are issued together: keys, and values (whose addresses do not wait for the scores).
   auto load_block = [&](KeyBlock& blk, int kb) {
+    blk.active = (kb <= last) && (kb + 31 >= lo);
 #pragma unroll
-    for (int tile = 0; tile < 2; ++tile) {
-      const int k0 = kb + tile * 16;                       // 16 keys of one page
-      blk.active[tile] = (k0 <= last) && (k0 + 15 >= lo);
-      if (blk.active[tile]) {
-        const int page = table[k0 / page_size];
-        const size_t base = ((size_t)page * n_kv + kvh) * page_size * D;   // same element count for K and V^T pages
-        const bf16_t* kr = k_pages + base + (size_t)((k0 % page_size) + col) * D + 8 * g;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          if (ks * 32 + 8 * g < D) blk.kf[tile][ks] = *reinterpret_cast<const bf16x8*>(kr + ks * 32);
-          else blk.kf[tile][ks] = zero8();
-        }
-        const bf16_t* vr = vt_pages + base + (size_t)col * page_size + (k0 % page_size) + 4 * g;
-        const int left = last - (k0 + 4 * g);              // keys of this lane that exist: 0..left
+      for (int ks = 0; ks < KS; ++ks) blk.kf[t][ks] = zero8();
+#pragma unroll
+    for (int db = 0; db < DB; ++db) blk.vf[db].bits = make_uint4(0, 0, 0, 0);
+    if (blk.active) {
+      // The two halves of sixteen keys: a half that holds no key of the range (before `lo`: its page may have been
+      // given back; after `last`: it may not exist yet) borrows the other half's page, which is a valid address;
+      // what is read there never counts (scores outside lo..last are masked, such values are set to zero).  So
+      // the branch is the same for the whole wave, and the addresses are a page number a lane away from scalars.
+      const bool there0 = kb + 15 >= lo, there1 = kb + 16 <= last;
+      const int page0 = table[(there0 ? kb : kb + 16) / page_size];
+      const int page1 = table[(there1 ? kb + 16 : kb) / page_size];
+      const uint32_t page_elems = (uint32_t)page_size * D;                  // same element count for K and V^T pages
+      {
+        const int half = col >> 3;
+        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems +
+                            (uint32_t)(((kb + 16 * half) % page_size) + 8 * ((col >> 2) & 1) + (col & 3)) * D + 8 * g;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            if (ks * 32 + 8 * g < D) blk.kf[t][ks] = *reinterpret_cast<const bf16x8*>(k_pages + at + t * 4 * D + ks * 32);
+      }
+      {
+        const int half = g >> 1;
+        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems + (uint32_t)col * page_size +
+                            ((kb + 16 * half) % page_size) + 8 * (g & 1);
+        const int left = (half ? there1 : there0) ? last - (kb + 8 * g) : -1;   // keys of this lane that exist: 0..left
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          uint2 v = *reinterpret_cast<const uint2*>(vr + (size_t)db * 16 * page_size);
-          if (left < 3) {                                  // slots nobody wrote may hold anything: 0 * NaN would poison the sum
+          uint4 v = *reinterpret_cast<const uint4*>(vt_pages + at + db * 16 * page_size);
+          if (left < 7) {                                    // slots nobody wrote may hold anything: 0 * NaN would poison the sum
             if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
-            if (left < 2) v.y = 0; else v.y &= 0xffffu;
+            if (left < 2) v.y = 0; else if (left < 3) v.y &= 0xffffu;
+            if (left < 4) v.z = 0; else if (left < 5) v.z &= 0xffffu;
+            if (left < 6) v.w = 0; else v.w &= 0xffffu;
           }
-          blk.vf[db].half[tile] = v;
+          blk.vf[db].bits = v;
         }
-      } else {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) blk.kf[tile][ks] = zero8();
-#pragma unroll
-        for (int db = 0; db < DB; ++db) blk.vf[db].half[tile] = make_uint2(0, 0);
       }
     }
   };
@@ -115,15 +133,15 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   auto attend = [&](const KeyBlock& blk, int kb) {
     float s[2][4];
 #pragma unroll
-    for (int tile = 0; tile < 2; ++tile) {
+    for (int t = 0; t < 2; ++t) {
       floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
-        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[tile][ks], qf[ks], st, 0, 0, 0);
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[t][ks], qf[ks], st, 0, 0, 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int key = kb + tile * 16 + 4 * g + r;
-        s[tile][r] = (blk.active[tile] && key >= lo && key <= last) ? st[r] * scale : -INFINITY;
+        const int key = kb + 8 * g + 4 * t + r;
+        s[t][r] = (blk.active && key >= lo && key <= last) ? st[r] * scale : -INFINITY;
       }
     }
     float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
@@ -136,12 +154,12 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     bf16x8 pf;
     float psum = 0.f;
 #pragma unroll
-    for (int tile = 0; tile < 2; ++tile)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __expf(s[tile][r] - m_new);        // exp(-inf) = 0 for masked keys
+        const float p = __expf(s[t][r] - m_new);           // exp(-inf) = 0 for masked keys
         psum += p;
-        pf[tile * 4 + r] = (__bf16)p;
+        pf[t * 4 + r] = (__bf16)p;
       }
     l = l * corr + psum;
     m = m_new;

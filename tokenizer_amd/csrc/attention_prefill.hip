@@ -19,7 +19,7 @@ __device__ __forceinline__ bf16x8 pf_zero8() {
   return z;
 }
 
-// One step of the online softmax over 64 keys (four 16-key tiles, each inside one page) for the HG heads of
+// One step of the online softmax over 64 keys (sixteen consecutive keys lie inside one page) for the HG heads of
 // the wave.  FULL: every key of the block is visible to every token of the tile, so nothing is masked.
 // Scores stay unscaled; `c` = scale * log2(e) enters in exp2(s*c - m*c).
 template <int D, int HG, bool FULL>
@@ -29,40 +29,61 @@ __device__ __forceinline__ void prefill_block(
     float c, const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16], float (&m)[HG], float (&l)[HG]) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
-  bf16x8 kf[4][KS];
-  union VFrag { uint2 half[2]; bf16x8 v; } vf[2][DB];
-  bool active[4];
+  // The block is two halves of 32 keys.  Key base + k of a half is index k of the second product's contraction
+  // (lane group g holds k = 8g .. 8g+7), so a lane's eight values of a row of V^T are sixteen contiguous bytes
+  // of one page: one load.  For that the first product's instructions take a half's keys in an order of their
+  // own: row r of instruction t is key base + 8 (r / 4) + 4 t + r % 4, whose score then lands in the lane group
+  // that holds that key in the second product.  Sixteen consecutive keys lie in one page.
+  bf16x8 kf[4][KS];                                    // [2 u + t]: instruction t of half u
+  union VFrag { uint4 bits; bf16x8 v; } vf[2][DB];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int k0 = kb + t * 16;
-    active[t] = FULL || ((k0 <= hi) && (k0 + 15 >= lo));
-    if (active[t]) {
-      const int page = table[k0 / page_size];
-      const size_t base = ((size_t)page * n_kv + kvh) * page_size * D;
-      const bf16_t* kr = k_pages + base + (size_t)((k0 % page_size) + col) * D + 8 * g;
+  for (int u = 0; u < 2; ++u) {
+    const int base_key = kb + 32 * u;
+    const bool active = FULL || ((base_key <= hi) && (base_key + 31 >= lo));      // the same for the whole wave
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks * 32 + 8 * g < D) kf[t][ks] = *reinterpret_cast<const bf16x8*>(kr + ks * 32);
-        else kf[t][ks] = pf_zero8();
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kf[2 * u + t][ks] = pf_zero8();
+#pragma unroll
+    for (int db = 0; db < DB; ++db) vf[u][db].bits = make_uint4(0, 0, 0, 0);
+    if (active) {
+      // A half's two runs of sixteen keys: one that holds no key of the range (before `lo`: its page may have been
+      // given back; after `hi`: it may not exist yet) borrows the other's page, a valid address; what is read
+      // there never counts (scores outside the range are masked, such values are set to zero).
+      const bool there0 = FULL || base_key + 15 >= lo, there1 = FULL || base_key + 16 <= hi;
+      const int page0 = table[(there0 ? base_key : base_key + 16) / page_size];
+      const int page1 = table[(there1 ? base_key + 16 : base_key) / page_size];
+      const uint32_t page_elems = (uint32_t)page_size * D;
+      {
+        const int half = col >> 3;
+        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems +
+                            (uint32_t)(((base_key + 16 * half) % page_size) + 8 * ((col >> 2) & 1) + (col & 3)) * D + 8 * g;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            if (ks * 32 + 8 * g < D)
+              kf[2 * u + t][ks] = *reinterpret_cast<const bf16x8*>(k_pages + at + t * 4 * D + ks * 32);
       }
-      const bf16_t* vr = vt_pages + base + (size_t)col * page_size + (k0 % page_size) + 4 * g;
+      {
+        const int half = g >> 1;
+        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems + (uint32_t)col * page_size +
+                            ((base_key + 16 * half) % page_size) + 8 * (g & 1);
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        uint2 v = *reinterpret_cast<const uint2*>(vr + (size_t)db * 16 * page_size);
-        if (!FULL) {                                   // slots past the last key may never have been written
-          const int left = hi - (k0 + 4 * g);          // keys of this lane that exist: 0..left
-          if (left < 3) {
-            if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
-            if (left < 2) v.y = 0; else v.y &= 0xffffu;
+        for (int db = 0; db < DB; ++db) {
+          uint4 v = *reinterpret_cast<const uint4*>(vt_pages + at + db * 16 * page_size);
+          if (!FULL) {                                 // slots past the last key may never have been written
+            const int left = (half ? there1 : there0) ? hi - (base_key + 8 * g) : -1;    // keys of this lane that exist: 0..left
+            if (left < 7) {
+              if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
+              if (left < 2) v.y = 0; else if (left < 3) v.y &= 0xffffu;
+              if (left < 4) v.z = 0; else if (left < 5) v.z &= 0xffffu;
+              if (left < 6) v.w = 0; else v.w &= 0xffffu;
+            }
           }
+          vf[u][db].bits = v;
         }
-        vf[t >> 1][db].half[t & 1] = v;
       }
-    } else {
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) kf[t][ks] = pf_zero8();
-#pragma unroll
-      for (int db = 0; db < DB; ++db) vf[t >> 1][db].half[t & 1] = make_uint2(0, 0);
     }
   }
 #pragma unroll
@@ -80,8 +101,8 @@ __device__ __forceinline__ void prefill_block(
         if (FULL) {
           s[t * 4 + r] = st[r];
         } else {
-          const int key = kb + t * 16 + 4 * g + r;
-          s[t * 4 + r] = (active[t] && key <= my_pos && key >= my_lo) ? st[r] : -INFINITY;
+          const int key = kb + 32 * (t >> 1) + 8 * g + 4 * (t & 1) + r;     // (keys outside lo..hi lie outside my_lo..my_pos)
+          s[t * 4 + r] = (key <= my_pos && key >= my_lo) ? st[r] : -INFINITY;
         }
       }
     }
@@ -307,10 +328,10 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
   if (d == 64 && heads_per_wave == 0 && (n_q / n_kv) % 7 == 0 && planned_reach(max_keys, window) > 768) {
     // Seven query heads per kv head (or fourteen) and enough tiles to fill the device with a quarter of the
     // workgroups: a wave takes all seven heads, so that every key tile is read once instead of four times and no
-    // head slot of a wave stays empty (measured at 14 / 2 heads: level at 3,072 tokens, 1.2x at 4,096, 1.3x from
-    // 8,192 on; with fewer tiles the device runs out of workgroups).
+    // head slot of a wave stays empty (measured at 14 / 2 heads: level at 2,560 tokens, 1.13x at 3,072, 1.2x at
+    // 4,096, 1.3x from 8,192 on; with fewer tiles the device runs out of workgroups: 0.86x at 2,048).
     const long workgroups = (long)n_tiles * n_kv * (n_q / n_kv / 7);
-    if (workgroups >= 512) {
+    if (workgroups >= 384) {
       heads_per_wave = 7;
       if (waves == 0) waves = workgroups < 1024 ? 4 : 2;
     }
