@@ -372,6 +372,41 @@ def test_peaked_attention_over_hundreds_of_keys(model_folders, tmp_path, name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_far_token_moves_the_last_logits_as_the_plain_model_says(model_folders, tmp_path, dtype):
+    """In both dtypes, through the whole engine: with attention sharpened (not to one-hot: bfloat16 rounding must
+    not decide), one token changed some two hundred positions back moves the last logits by several times the
+    bfloat16 bound.  The engine has to show the same move, decoding token by token and in mixed batches with
+    reused pages: a key read from a wrong page, a split of the key range left out or a block table row mixed up
+    would lose it, where the nearly uniform attention of the other tests' weights would hide that."""
+    name = "B"
+    folder = sharpened(model_folders[name], str(tmp_path / "sharp"), 8.0)
+    cfg, tensors64 = plain.load_folder(folder, torch.float64)
+    vocab = cfg["vocab_size"]
+    ids = random_ids(vocab, 250, 91)
+    base = plain.all_logits(cfg, tensors64, ids).float()
+    moves = []
+    for at in (2, 5, 9, 14, 20, 33, 47):
+        other = list(ids)
+        other[at] = (other[at] + 101) % vocab
+        moved = plain.all_logits(cfg, tensors64, other).float()
+        moves.append((float((moved[-16:] - base[-16:]).abs().max()), at, other, moved))
+    effect, at, other, moved = max(moves, key=lambda item: item[0])
+    bound = TOL[dtype] * max(1.0, float(base.abs().max()))
+    assert effect > 5 * TOL["bfloat16"], "the weights and inputs should make one far token matter"
+    reqs = {"base": ids, "moved": other, "beside": random_ids(vocab, 120, 92)}
+    for steps in (tt.decode_tail(reqs, 32), tt.mixed(reqs, 12, max_live=3)):
+        eng = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=3)
+        eng.pools.poison()
+        got = tt.run_in_process(eng, steps)
+        close(got["base"], base, dtype)
+        close(got["moved"], moved, dtype)
+        shown = got["moved"][-16:] - got["base"][-16:]
+        assert float((shown - (moved[-16:] - base[-16:])).abs().max()) <= 2 * bound
+        assert float(shown.abs().max()) >= effect - 2 * bound
+        eng.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_entry_points(model_folders, tmp_path, dtype):
     import subprocess
     import sys
