@@ -95,11 +95,33 @@ def test_tensors_the_model_does_not_read_are_a_warning_alone(tmp_path):
     save_safetensors(path, tensors)
     with pytest.warns(UnexpectedTensors, match="lm_head.weight") as caught:
         out = load_weights(path, expected(), torch.bfloat16)
-    assert "rotary_emb.inv_freq" in str(caught[0].message) and set(out) == set(expected())
+    ours = [str(w.message) for w in caught if isinstance(w.message, UnexpectedTensors)]
+    assert len(ours) == 1 and "rotary_emb.inv_freq" in ours[0] and set(out) == set(expected())
     with pytest.raises(WeightError) as err:
         load_weights(path, expected(), torch.bfloat16, strict=True)
     assert err.value.unexpected == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
     assert not err.value.missing
+
+
+def test_a_model_in_shards_beside_an_index(tmp_path):
+    import json
+    tensors = random_tensors(expected("B"), 2)
+    names = sorted(tensors)
+    shards = {"model-00001-of-00002.safetensors": names[::2], "model-00002-of-00002.safetensors": names[1::2]}
+    for file_name, held in shards.items():
+        save_safetensors(str(tmp_path / file_name), {n: tensors[n] for n in held})
+    index = {"metadata": {}, "weight_map": {n: f for f, held in shards.items() for n in held}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    out = load_weights(str(tmp_path), expected("B"), torch.bfloat16)
+    assert set(out) == set(names) and all(torch.equal(out[n].float(), tensors[n].float()) for n in names)
+    # A tensor the index promises but its shard does not hold is missing; a shard that is not there says so.
+    save_safetensors(str(tmp_path / "model-00002-of-00002.safetensors"), {n: tensors[n] for n in names[1::2][1:]})
+    with pytest.raises(WeightError) as err:
+        load_weights(str(tmp_path), expected("B"), torch.bfloat16)
+    assert err.value.missing == [names[1]]
+    (tmp_path / "model-00001-of-00002.safetensors").unlink()
+    with pytest.raises(WeightError, match="no weight file"):
+        load_weights(str(tmp_path), expected("B"), torch.bfloat16)
 
 
 def test_untied_model_needs_its_head(tmp_path):

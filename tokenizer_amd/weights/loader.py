@@ -15,6 +15,7 @@ qwen-infer/src/model.rs:263-276).
 """
 from __future__ import annotations
 
+import json
 import os
 import warnings
 
@@ -78,6 +79,54 @@ def weight_path(folder: str) -> str:
     return os.path.join(folder, "model.safetensors") if os.path.isdir(folder) else folder
 
 
+class ShardedWeights:
+    """A model stored in several safetensors files beside `model.safetensors.index.json`, whose `weight_map`
+    says which file holds which tensor (larger checkpoints are published that way; the reference reads a single
+    file, qwen-infer/src/lib.rs:56-60).  Same face as `SafetensorsFile`; a shard is mapped when first asked for."""
+
+    def __init__(self, index_path: str):
+        self.path = index_path
+        try:
+            with open(index_path, encoding="utf-8") as fh:
+                weight_map = json.load(fh)["weight_map"]
+        except (OSError, ValueError, KeyError, TypeError) as err:
+            raise SafetensorsError(f"{index_path} is no shard index: {err}") from None
+        if not isinstance(weight_map, dict):
+            raise SafetensorsError(f"{index_path}: weight_map is not an object")
+        self._folder = os.path.dirname(index_path)
+        self._file_of = weight_map
+        self._shards: dict[str, SafetensorsFile] = {}
+
+    def _shard(self, name: str) -> SafetensorsFile:
+        file_name = self._file_of[name]
+        if file_name not in self._shards:
+            self._shards[file_name] = SafetensorsFile(os.path.join(self._folder, file_name))
+        return self._shards[file_name]
+
+    def names(self) -> list[str]:
+        # What the shards really hold: a name the index promises but its file lacks is then reported as missing.
+        return [name for name in self._file_of if name in self._shard(name)._entries]
+
+    def info(self, name: str):
+        return self._shard(name).info(name)
+
+    def tensor(self, name: str):
+        return self._shard(name).tensor(name)
+
+    def close(self) -> None:
+        for shard in self._shards.values():
+            shard.close()
+
+
+def open_weights(folder: str):
+    """The weights of a model folder: `model.safetensors`, or the shards that `model.safetensors.index.json` lists."""
+    path = weight_path(folder)
+    index = path + ".index.json"
+    if not os.path.exists(path) and os.path.exists(index):
+        return ShardedWeights(index)
+    return SafetensorsFile(path)
+
+
 def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: torch.dtype,
                  device: torch.device | str = "cpu", strict: bool = False) -> dict[str, torch.Tensor]:
     """Load the tensors in `expected`, or raise one `WeightError` naming every misfit (missing, wrong shape,
@@ -85,10 +134,11 @@ def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: to
     warning that lists them, or the same error with `strict=True`."""
     path = weight_path(folder)
     try:
-        source = SafetensorsFile(path)
+        source = open_weights(folder)
+        path = source.path
+        names = set(source.names())
     except SafetensorsError as err:
         raise WeightError(path, other=[str(err)]) from None
-    names = set(source.names())
     missing = sorted(set(expected) - names)
     unexpected = sorted(names - set(expected))
     wrong_shape, wrong_dtype = [], []
@@ -102,6 +152,7 @@ def load_weights(folder: str, expected: dict[str, TensorSpec], compute_dtype: to
         if spec.role == "table" and dtype not in _INTS:
             wrong_dtype.append((name, dtype))
     if missing or wrong_shape or wrong_dtype or (unexpected and strict):
+        source.close()
         raise WeightError(path, missing, unexpected, wrong_shape, wrong_dtype)
     if unexpected:
         warnings.warn(UnexpectedTensors(f"{path} holds {len(unexpected)} tensors the model does not read: "
