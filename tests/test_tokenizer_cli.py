@@ -118,3 +118,49 @@ def test_generate_takes_text_with_a_tokenizer(model_folders):
     assert from_text.text == tok.decode_bytes(from_text.tokens).decode("utf-8", errors="replace")
     with pytest.raises(ValueError):
         generate(engine, "abba", GenerateParams.greedy(1))
+
+
+def test_merges_in_the_host_library_follow_the_rule_spelled_out_here():
+    """Random vocabularies over a small alphabet: the ids the tokenizer gives (its merge loop runs in the C++ host
+    library) against the rule written out plainly: join the neighbouring pair whose joined bytes have the lowest
+    rank, the leftmost of equals, until no pair has a rank (src/rank.rs:536-586)."""
+    import random
+    reverse = bytes_to_unicode_reverse()
+    of_byte = {byte: ch for ch, byte in reverse.items()}
+    spell = lambda raw: "".join(of_byte[b] for b in raw)
+
+    def plainly(piece, ranks, ids):
+        parts = [piece[i:i + 1] for i in range(len(piece))]
+        while True:
+            ranked = [(ranks[a + b], i) for i, (a, b) in enumerate(zip(parts, parts[1:])) if a + b in ranks]
+            if not ranked:
+                return [ids[p] for p in parts]
+            _, at = min(ranked)
+            parts[at:at + 2] = [parts[at] + parts[at + 1]]
+
+    for seed in range(8):
+        rng = random.Random(seed)
+        ids = {bytes([b]): b for b in range(256)}
+        merges, ranks = [], {}
+        tokens = [b"a", b"b", b"c", b" "]
+        for _ in range(rng.randint(3, 40)):
+            left, right = rng.choice(tokens), rng.choice(tokens)
+            if left + right in ranks or len(left + right) > 6:
+                continue
+            ranks[left + right] = len(merges)
+            ids[left + right] = 256 + len(merges)
+            merges.append(f"{spell(left)} {spell(right)}")
+            tokens.append(left + right)
+        data = tiny_file(pattern=" ?[abc]+| +")
+        data["model"]["vocab"] = {spell(raw): token for raw, token in ids.items()}
+        data["model"]["merges"] = merges
+        tok = Tokenizer.from_json(data)
+        for _ in range(30):
+            text = "".join(rng.choice("abc ") for _ in range(rng.randint(1, 40)))
+            want = []
+            for piece in tok.pattern.findall(text):
+                want += plainly(piece.encode(), ranks, ids)
+            assert tok.encode(text) == want, (seed, text)
+            assert tok.decode(want) == text
+    long_piece = "ab" * 400                                    # more parts than the first buffer holds
+    assert tok.decode(tok.encode(long_piece)) == long_piece

@@ -4,6 +4,7 @@
 #include <cstring>
 #include <string>
 
+#include "bpe_core.h"
 #include "cache_core.h"
 #include "page_allocator.h"
 #include "sampler.h"
@@ -222,6 +223,23 @@ float ta_uniform_f32(uint64_t seed, uint64_t counter) { return uniform_f32(seed,
 int ta_greedy_token(const float* logits, int64_t count) { return greedy_token(logits, count); }
 int ta_sample_with_uniform(const float* logits, int64_t count, float temperature, float top_p, float uniform) {
   return sample_with_uniform(logits, count, temperature, top_p, uniform);
+}
+
+// ---------------------------------------------------------------------------------------- tokenizer
+void* ta_bpe_new() { return new BpeCore(); }
+void ta_bpe_delete(void* b) { delete (BpeCore*)b; }
+int ta_bpe_add_token(void* b, int32_t id, const uint8_t* bytes, int len, int findable) {
+  return ((BpeCore*)b)->add_token(id, bytes, len, findable != 0);
+}
+int ta_bpe_add_merge(void* b, const uint8_t* merged, int len, int rank) {
+  return ((BpeCore*)b)->add_merge(merged, len, rank);
+}
+int ta_bpe_vocab_size(void* b) { return ((BpeCore*)b)->vocab_size(); }
+int ta_bpe_encode_piece(void* b, const uint8_t* piece, int len, int32_t* out, int capacity) {
+  return ((BpeCore*)b)->encode_piece(piece, len, out, capacity);
+}
+int64_t ta_bpe_decode(void* b, const int32_t* ids, int count, uint8_t* out, int64_t capacity, int* bad_at) {
+  return ((BpeCore*)b)->decode(ids, count, out, capacity, bad_at);
 }
 
 }  // extern "C"

@@ -68,6 +68,13 @@ _SIGNATURES = {
     "ta_sched_tokens": (_int, [_vp, _i64, _int, _int, _i32p]),
     "ta_sched_commit": (_int, [_vp, _i64, _int]),
     "ta_sched_finish": (_int, [_vp, _i64]),
+    "ta_bpe_new": (_vp, []),
+    "ta_bpe_delete": (None, [_vp]),
+    "ta_bpe_add_token": (_int, [_vp, ctypes.c_int32, ctypes.c_char_p, _int, _int]),
+    "ta_bpe_add_merge": (_int, [_vp, ctypes.c_char_p, _int, _int]),
+    "ta_bpe_vocab_size": (_int, [_vp]),
+    "ta_bpe_encode_piece": (_int, [_vp, ctypes.c_char_p, _int, _i32p, _int]),
+    "ta_bpe_decode": (_i64, [_vp, _i32p, _int, ctypes.c_char_p, _i64, _i32p]),
     "ta_uniform_f32": (_f32, [_u64, _u64]),
     "ta_greedy_token": (_int, [_f32p, _i64]),
     "ta_sample_with_uniform": (_int, [_f32p, _i64, _f32, _f32, _f32]),

@@ -14,10 +14,13 @@ leftmost of equals) until no pair has a rank.
 """
 from __future__ import annotations
 
+import ctypes
 import json
 import unicodedata
 
 import regex
+
+from .. import host as _host
 
 
 class TokenizerError(ValueError):
@@ -161,12 +164,60 @@ class _TokenizerFile:
         return found
 
 
+class _MergeCore:
+    """The merges inside a piece and the way back from ids to bytes, in the host library (csrc/host/bpe_core.cpp)."""
+
+    def __init__(self, encoder: dict[bytes, int], ranks: dict[bytes, int], specials: dict[str, int]):
+        self._lib = _host.lib()
+        self._core = self._lib.ta_bpe_new()
+        for raw, token in encoder.items():
+            if self._lib.ta_bpe_add_token(self._core, token, raw, len(raw), 1) != 0:
+                raise TokenizerError(f"token id {token} or its bytes {raw!r} are taken already")
+        for text, token in specials.items():
+            raw = text.encode("utf-8")
+            if self._lib.ta_bpe_add_token(self._core, token, raw, len(raw), 0) != 0:
+                raise TokenizerError(f"token id {token} of {text!r} is taken already")
+        for merged, rank in ranks.items():
+            self._lib.ta_bpe_add_merge(self._core, merged, len(merged), rank)
+        self._ids = (ctypes.c_int32 * 256)()
+
+    def __del__(self):
+        if getattr(self, "_core", None):
+            self._lib.ta_bpe_delete(self._core)
+            self._core = None
+
+    def piece(self, piece: bytes, ids: list[int]) -> None:
+        count = self._lib.ta_bpe_encode_piece(self._core, piece, len(piece), self._ids, len(self._ids))
+        if count < 0 and count > -(1 << 31):                 # the piece has more parts than the buffer holds
+            self._ids = (ctypes.c_int32 * (-count))()
+            count = self._lib.ta_bpe_encode_piece(self._core, piece, len(piece), self._ids, len(self._ids))
+        if count < 0:
+            raise TokenizerError(f"piece {piece!r} does not break down into tokens of the vocabulary")
+        ids.extend(self._ids[:count])
+
+    def bytes_of(self, ids) -> bytes:
+        tokens = [int(t) for t in ids]
+        if any(not -(1 << 31) <= t < (1 << 31) for t in tokens):
+            raise UnknownToken(next(t for t in tokens if not -(1 << 31) <= t < (1 << 31)))
+        array = (ctypes.c_int32 * max(1, len(tokens)))(*tokens)
+        bad = ctypes.c_int32(0)
+        out = ctypes.create_string_buffer(max(1, 8 * len(tokens)))
+        size = self._lib.ta_bpe_decode(self._core, array, len(tokens), out, len(out), ctypes.byref(bad))
+        if size < 0 and size > -(1 << 31):
+            out = ctypes.create_string_buffer(-size)
+            size = self._lib.ta_bpe_decode(self._core, array, len(tokens), out, len(out), ctypes.byref(bad))
+        if size < 0:
+            raise UnknownToken(tokens[bad.value])
+        return out.raw[:size]
+
+
 class Tokenizer:
     def __init__(self, encoder, decoder, ranks, specials, pattern: str):
         self.encoder: dict[bytes, int] = encoder
         self.decoder: list[bytes | None] = decoder
         self.ranks: dict[bytes, int] = ranks
         self.specials: dict[str, int] = specials
+        self._core = _MergeCore(encoder, ranks, specials)
         try:
             self.pattern = regex.compile(pattern)
         except regex.error as err:
@@ -239,29 +290,11 @@ class Tokenizer:
             self._encode_piece(text[at:].encode("utf-8"), ids)
 
     def _encode_piece(self, piece: bytes, ids: list[int]) -> None:
-        whole = self.encoder.get(piece) if len(piece) == 1 else None
-        if whole is not None:
-            ids.append(whole)
-            return
-        parts = [piece[i:i + 1] for i in range(len(piece))]
-        while len(parts) > 1:
-            ranked = [(self.ranks.get(left + right), i) for i, (left, right) in enumerate(zip(parts, parts[1:]))]
-            ranked = [pair for pair in ranked if pair[0] is not None]
-            if not ranked:
-                break
-            _, at = min(ranked)                          # lowest rank; the leftmost of equal ranks
-            parts[at:at + 2] = [parts[at] + parts[at + 1]]
-        ids.extend(self.encoder[part] for part in parts)
+        self._core.piece(piece, ids)
 
     # ------------------------------------------------------------------- decoding
     def decode_bytes(self, ids) -> bytes:
-        out = bytearray()
-        for token in ids:
-            raw = self.decoder[token] if 0 <= token < len(self.decoder) else None
-            if raw is None:
-                raise UnknownToken(token)
-            out.extend(raw)
-        return bytes(out)
+        return self._core.bytes_of(ids)
 
     def decode(self, ids) -> str:
         return self.decode_bytes(ids).decode("utf-8", errors="replace")
