@@ -12,6 +12,10 @@ class StepEntry:
     rid: object
     tokens: list[int]
     want: list[int] = dataclasses.field(default_factory=list)
+    token_array: object = dataclasses.field(default=None, repr=False, compare=False)   # `tokens` as an array, once made
+
+    def packed_tokens(self):
+        return self.tokens if self.token_array is None else self.token_array
 
 
 @dataclasses.dataclass
@@ -57,7 +61,7 @@ def build_context(entries: list[StepEntry], manager, device, table_width: int | 
     page_size = manager.page_size
     n_groups = len(manager.groups)
     rids = [entry.rid for entry in entries]
-    token_lists = [entry.tokens for entry in entries]
+    token_lists = [entry.packed_tokens() for entry in entries]
     want_lists = [entry.want for entry in entries]
     if into is not None:
         host, dev = into

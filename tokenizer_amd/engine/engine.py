@@ -1,6 +1,7 @@
 """The engine: a model, its cache and the one step function everything else is built on."""
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager, CachePools, OutOfPages
@@ -137,7 +138,7 @@ class StepGraph:
         else:
             self.uploaded = torch.cuda.Event()
         manager = engine.cache
-        total, _, _, _ = manager.pack_batch([e.rid for e in entries], [e.tokens for e in entries],
+        total, _, _, _ = manager.pack_batch([e.rid for e in entries], [e.packed_tokens() for e in entries],
                                             [e.want for e in entries], self.host.numpy(), self.width)
         if total != self.host.numel():
             raise ValueError("the packed batch does not fit the graph's buffers")
@@ -390,9 +391,14 @@ class Engine:
             seen.add(entry.rid)
             if not self.cache.has_request(entry.rid):
                 raise KeyError(f"request {entry.rid!r} is not live")
-            if not entry.tokens:
+            if len(entry.tokens) == 0:
                 raise ValueError(f"request {entry.rid!r} brings no tokens")
-            if not (0 <= min(entry.tokens) and max(entry.tokens) < vocab):
+            if len(entry.tokens) > 64:                     # long portions: one conversion, kept for the packing
+                entry.token_array = np.asarray(entry.tokens, dtype=np.int64)
+                low, high = int(entry.token_array.min()), int(entry.token_array.max())
+            else:
+                low, high = min(entry.tokens), max(entry.tokens)
+            if not (0 <= low and high < vocab):
                 raise ValueError(f"request {entry.rid!r} has a token id outside 0..{vocab - 1}")
             end = self.cache.seq_len(entry.rid) + len(entry.tokens)
             if end > limit:
