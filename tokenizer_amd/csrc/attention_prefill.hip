@@ -143,7 +143,7 @@ __device__ __forceinline__ void prefill_block(
 // cu_q[e]: first row of entry e; first_position[e]: position of that row.
 // K pages [n_pages, n_kv, page_size, D]; V^T pages [n_pages, n_kv, D, page_size]; page_size % 16 == 0.
 template <int D, int HG, int NWV>
-__global__ void __launch_bounds__(NWV * WAVE)
+__global__ void __launch_bounds__(NWV * WAVE, (D <= 64 && HG <= 2) ? 3 : 1)
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
