@@ -139,3 +139,50 @@ def test_decode_steps_back_to_back_give_what_single_steps_give(model_folders, dt
         assert bursts[0].reason == StopReason.Eos and len(bursts[0].tokens) == ends_at
         assert bursts[2].reason in (StopReason.StopString, StopReason.Eos)
         assert any(r.reason == StopReason.MaxTokens for r in bursts)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_arrivals_pools_and_budgets_on_the_device(model_folders, seed):
+    """Random prompts (some with a shared beginning), output lengths, pool sizes, batch caps, token budgets,
+    portion sizes, burst lengths and arrival times, in float32 on the kernels with graphs: whatever the scheduler
+    decides, every request gets the plain implementation's tokens, and in the end nothing is left over."""
+    import random
+    from tokenizer_amd.engine import Failure, GenerateParams, Scheduler, SchedulerConfig
+    rng = random.Random(seed)
+    name = "B"
+    cfg, tensors = plain.load_folder(model_folders[name])
+    vocab, page = cfg["vocab_size"], 16
+    num_pages = rng.choice([5, 7, 10, 24])
+    config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 3, 5]), num_blocks=num_pages,
+                             prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 16, 40]),
+                             prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64,
+                             decode_burst=rng.choice([1, 3, 16]))
+    eng = engine_for(model_folders[name], "float32", num_pages=num_pages, max_requests=config.max_batch_size,
+                     prefix_cache=config.prefix_cache)
+    eng.pools.poison()
+    sched = Scheduler(eng, config)
+    shared = random_ids(vocab, 35, 900 + seed)
+    plan = []
+    for i in range(rng.randint(4, 8)):
+        prompt = random_ids(vocab, rng.choice([1, 2, 7, 16, 17, 33, 48]), 100 * seed + i)
+        if rng.random() < 0.4:
+            prompt = shared[:rng.choice([16, 32, 35])] + prompt
+        plan.append((rng.randint(0, 6), prompt, rng.randint(0, 9)))
+    ids, step = {}, 0
+    pending = sorted(plan, key=lambda item: item[0])
+    while pending or sched.has_work():
+        while pending and pending[0][0] <= step:
+            _, prompt, n = pending.pop(0)
+            ids[sched.add_request(prompt, GenerateParams.greedy(n))] = (prompt, n)
+        if sched.has_work():
+            sched.run(max_steps=1)
+        step += 1
+        assert step < 2000
+        eng.cache.check_invariants()
+    for rid, (prompt, n) in ids.items():
+        result = sched.finished[rid]
+        if isinstance(result, Failure):
+            assert "kv pool has" in result.message and -(-(len(prompt) + n) // page) > num_pages
+            continue
+        assert result.tokens == plain.greedy_generate(cfg, tensors, prompt, n), (rid, len(prompt), n)
+    sched.assert_idle()

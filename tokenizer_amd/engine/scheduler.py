@@ -272,6 +272,8 @@ class Scheduler:
             return 1
         if self._get(_WAITING) and len(plan) < self.config.max_batch_size:
             return 1                     # the queue's front waits for pages: a finished sequence should let it in at once
+        if len(plan) != self._get(_RUNNING):
+            return 1                     # the token budget left a running sequence out of this step: it is next
         for seq, first, count, completes in plan:
             if count != 1 or first < seq.prompt_len or not completes or not seq.cursor.is_greedy:
                 return 1
