@@ -278,6 +278,59 @@ def test_prefill_attention_with_all_heads_of_a_group_in_one_wave(ops, ref, geome
     torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("geometry", [(28, 4, 128, 16), (12, 2, 128, 32), (5, 1, 96, 48), (16, 2, 128, 16),
+                                      (24, 2, 128, 64), (3, 1, 128, 16)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, geometry, window, monkeypatch):
+    # The kernel whose four waves take one block of keys from LDS for up to eight query heads of a kv head: five,
+    # six, seven and eight heads (a wave with one head, a wave without any), twelve (two workgroups a tile) and
+    # three; portions that start in the middle of a page, end in the middle of a tile, lie under a window whose
+    # first pages hold nothing any more, and unwritten slots that hold NaN.
+    monkeypatch.setattr(ops, "prefill_shared", 1)
+    n_q, n_kv, d, page_size = geometry
+    lengths, q_lens = [700, 333, 40, 16, 1000], [700, 50, 33, 16, 2]
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=29)
+    scale = 1.0 / math.sqrt(d)
+    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    out_b = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
+    torch.testing.assert_close(out_a.float(), out_b, **attention_tol(torch.bfloat16, True))
+    rows = torch.tensor([0, 17, 699, 700, 749, 750, qkv.shape[0] - 1]).cuda()
+    out_c = torch.empty((len(rows), n_q * d), dtype=torch.bfloat16).cuda()
+    ref.paged_attention(qkv[rows], out_c, k_pages, v_pages, positions[rows], entry_of_token[rows], table, n_q, n_kv, d,
+                        window, scale)
+    torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
+    # The other prompt kernel rounds at other places; both stay within the same distance of the float32 result.
+    monkeypatch.setattr(ops, "prefill_shared", -1)
+    out_d = torch.full_like(out_a, float("nan"))
+    ops.paged_attention(qkv, out_d, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    torch.testing.assert_close(out_d.float(), out_b, **attention_tol(torch.bfloat16, True))
+
+
+@pytest.mark.parametrize("window", [None, 1000])
+def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles_of_large_heads(ops, ref, window):
+    # Seven heads of size 128 per kv head and more than 512 workgroups: the launcher's own choice.  A prompt
+    # that starts inside a page after 100 cached tokens, beside a short one.
+    n_q, n_kv, d, page_size = 28, 4, 128, 16
+    lengths, q_lens = [2300, 40], [2200, 33]
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=31)
+    batch = make_batch(lengths, q_lens)
+    assert ops.prefill_shared == 0 and ops.prefill_waves == 0 and ops.prefill_heads_per_wave == 0
+    assert ops.lib.ta_prefill_attention_shared_pays(batch.q_tiles.shape[0], n_q, n_kv, d) == 1
+    assert ops.lib.ta_prefill_attention_shared_pays(batch.q_tiles.shape[0], n_q, n_kv, 64) == 0
+    assert ops.lib.ta_prefill_attention_shared_pays(100, n_q, n_kv, d) == 0
+    scale = 1.0 / math.sqrt(d)
+    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=batch)
+    out_b = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
+    torch.testing.assert_close(out_a.float(), out_b, **attention_tol(torch.bfloat16, True))
+
+
 @pytest.mark.parametrize("target", [1024, 16])
 @pytest.mark.parametrize("window", [None, 1000])
 def test_decode_attention_long_contexts_and_many_splits(ops, ref, window, target, monkeypatch):
@@ -326,14 +379,15 @@ def test_paged_attention_finds_one_far_key(ops, attention_mode):
 
 
 @pytest.mark.parametrize("attention_mode", ATTENTION_MODES, indirect=True)
-@pytest.mark.parametrize("waves", [0, 1])
-def test_every_row_of_a_portion_sees_exactly_to_its_window_edge(ops, attention_mode, waves, monkeypatch):
+@pytest.mark.parametrize("waves,heads,shared", [(0, (4, 2, 64), 0), (1, (4, 2, 64), 0), (0, (10, 2, 128), 1)])
+def test_every_row_of_a_portion_sees_exactly_to_its_window_edge(ops, attention_mode, waves, heads, shared, monkeypatch):
     """A portion of 100 prompt tokens under a window of 77: the query at position p is made to look at the key
     at p - 77, the farthest it may see; those keys cross page and tile edges.  The output must be that key's
     value row; with a window of 76 the key is out of sight and the output is something else."""
     dtype = attention_mode
     monkeypatch.setattr(ops, "prefill_waves", waves)
-    n_q, n_kv, d, page_size, window = 4, 2, 64, 16, 77
+    monkeypatch.setattr(ops, "prefill_shared", shared)
+    (n_q, n_kv, d), page_size, window = heads, 16, 77
     lengths, q_lens = [700], [100]
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         dtype, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=21)

@@ -82,6 +82,7 @@ class Ops:
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16",
+                     "ta_prefill_attention_shared_pays",
                      "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16",
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
@@ -262,7 +263,7 @@ class Ops:
                 batch.q_tiles.shape[0], _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
                 block_table.shape[1], n_q, n_kv, head_dim, page_size, -1 if window is None else int(window),
                 ctypes.c_float(scale), self.prefill_heads_per_wave, int(batch.max_position) + 1,
-                self.prefill_waves, self._stream()), "prefill_attention")
+                self.prefill_waves, self.prefill_shared, self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
                 self._decode_attention(*args, rows=batch.decode_rows)
             return out
@@ -277,6 +278,8 @@ class Ops:
     use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
     prefill_waves = 0          # waves that share a tile's keys in the prompt kernel: 0 lets the launcher choose
     prefill_heads_per_wave = 0    # 0: the kernel's own choice for the head size
+    prefill_shared = 0            # the prompt kernel whose waves share a block of keys through LDS: 1 = wherever it has
+    #                               an instance, -1 = never, 0 = where the launcher expects it to be the faster one
     target_workgroups = 1024      # what the split of the key range aims at
     PLAN_KEYS = 512               # launch shapes depend on the context only through its multiple of this
 
