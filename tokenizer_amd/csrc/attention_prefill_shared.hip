@@ -53,10 +53,17 @@ struct Carrier {
   bool mine[ROUNDS];
   int v_first[ROUNDS];                                      // first key of the value piece, within its run
   piece_t k[4][ROUNDS], v[4][ROUNDS];
-  int at_page, at_slot;                                     // where the next run to fetch lies: index into the block table, slot in the page
+  int at_page, at_slot;                                     // where the next run to look up lies: index into the block table, slot in the page
+  int page[4], slot[4];                                     // of the runs of the block to fetch next (the same for all threads)
+  bool there[4];                                            // whether the run holds a key of lo..hi
+  int page_size;
+  uint32_t page_elements, first_element;                    // elements of a page (all kv heads); where this kv head's begin
 
-  // first_key: the first key of the first block that will be fetched; blocks are fetched in order.
-  __device__ __forceinline__ void plan(int tid, int page_size, int first_key) {
+  // first_key: the first key of the first block.
+  __device__ __forceinline__ void plan(int tid, const SharedTile& tile, int first_key) {
+    page_size = tile.page_size;
+    page_elements = (uint32_t)tile.n_kv * page_size * D;
+    first_element = (uint32_t)tile.kvh * page_size * D;
     at_page = first_key / page_size;
     at_slot = first_key % page_size;
 #pragma unroll
@@ -73,48 +80,75 @@ struct Carrier {
     }
   }
 
-  // Block `kb` from the pages into registers.  `full`: every key of the block exists and is seen by every
-  // token.  Otherwise a run without a key of lo..hi (before `lo`: its page may have been given back; after
-  // `hi`: it may not exist yet) borrows the page of `lo` or `hi`, a valid address, and its values become zero,
-  // as do values past `hi` (slots never written): a probability of zero times whatever lies there must stay
-  // zero.  Keys need no such care, their scores are masked by selection.
-  __device__ __forceinline__ void fetch(const SharedTile& tile, int kb, bool full) {
+  // Where the four runs of block `kb` lie: their pages and slots, looked up a turn before the block is fetched,
+  // so that no wave waits for a page number.  Blocks are looked up in order.  `full`: every key of the block
+  // exists and is seen by every token.  Otherwise a run without a key of lo..hi (before `lo`: its page may have
+  // been given back; after `hi`: it may not exist yet) borrows the page of `lo` or `hi`, a valid address.
+  __device__ __forceinline__ void look_up(const SharedTile& tile, int kb, bool full) {
+    if (full) {                                            // the usual block: nothing to decide per run
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        page[q] = tile.table[at_page];
+        slot[q] = at_slot;
+        there[q] = true;
+        step();
+      }
+      return;
+    }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int key = kb + 16 * q;
       int index = at_page;
-      bool there = true;
-      if (!full) {
-        there = key + 15 >= tile.lo && key <= tile.hi;
-        if (key + 15 < tile.lo) index = tile.lo_page;
-        if (key > tile.hi) index = tile.hi_page;
-      }
-      const uint32_t page = (uint32_t)__builtin_amdgcn_readfirstlane(tile.table[index]);
-      const uint32_t head = (page * tile.n_kv + tile.kvh) * (uint32_t)tile.page_size * D;
-      const bf16_t* k_run = tile.k_pages + (head + (uint32_t)at_slot * D);
-      const bf16_t* v_run = tile.vt_pages + (head + (uint32_t)at_slot);
-      at_slot += 16;                                     // on to the next run: pages hold whole runs
-      if (at_slot >= tile.page_size) {
-        at_slot = 0;
-        ++at_page;
-      }
+      there[q] = key + 15 >= tile.lo && key <= tile.hi;
+      if (key + 15 < tile.lo) index = tile.lo_page;
+      if (key > tile.hi) index = tile.hi_page;
+      page[q] = tile.table[index];
+      slot[q] = at_slot;
+      step();
+    }
+  }
+
+  // On to the next run: pages hold whole runs.
+  __device__ __forceinline__ void step() {
+    at_slot += 16;
+    if (at_slot >= page_size) {
+      at_slot = 0;
+      ++at_page;
+    }
+  }
+
+  // The block that was looked up last, from the pages into registers.  Unless the block is `full`, the values
+  // of a borrowed run become zero, as do values past `hi` (slots never written): a probability of zero times
+  // whatever lies there must stay zero.  Keys need no such care, their scores are masked by selection.
+  __device__ __forceinline__ void fetch(const SharedTile& tile, int kb, bool full) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t head = (uint32_t)page[q] * page_elements + first_element;
+      const bf16_t* k_run = tile.k_pages + (head + (uint32_t)slot[q] * D);
+      const bf16_t* v_run = tile.vt_pages + (head + (uint32_t)slot[q]);
 #pragma unroll
       for (int r = 0; r < ROUNDS; ++r) {
         if (!mine[r]) continue;
         k[q][r] = *reinterpret_cast<const piece_t*>(k_run + k_from[r]);
-        piece_t x = *reinterpret_cast<const piece_t*>(v_run + v_from[r]);
-        if (!full) {
-          const int left = there ? tile.hi - (key + v_first[r]) : -1;     // keys of this piece that exist: 0..left
-          if (left < 7) {
-            if (left < 0) x.x = 0; else if (left < 1) x.x &= 0xffffu;
-            if (left < 2) x.y = 0; else if (left < 3) x.y &= 0xffffu;
-            if (left < 4) x.z = 0; else if (left < 5) x.z &= 0xffffu;
-            if (left < 6) x.w = 0; else x.w &= 0xffffu;
-          }
-        }
-        v[q][r] = x;
+        v[q][r] = *reinterpret_cast<const piece_t*>(v_run + v_from[r]);
       }
     }
+    if (full) return;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int r = 0; r < ROUNDS; ++r) {
+        if (!mine[r]) continue;
+        const int left = there[q] ? tile.hi - (kb + 16 * q + v_first[r]) : -1;     // keys of this piece that exist: 0..left
+        if (left < 7) {
+          piece_t x = v[q][r];
+          if (left < 0) x.x = 0; else if (left < 1) x.x &= 0xffffu;
+          if (left < 2) x.y = 0; else if (left < 3) x.y &= 0xffffu;
+          if (left < 4) x.z = 0; else if (left < 5) x.z &= 0xffffu;
+          if (left < 6) x.w = 0; else x.w &= 0xffffu;
+          v[q][r] = x;
+        }
+      }
   }
 
   __device__ __forceinline__ void put(char* buf) const {
@@ -280,18 +314,22 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   int kb = (lo / 64) * 64;
   int cur = 0;
   Carrier<D, THREADS> carrier;
-  carrier.plan(tid, page_size, kb);
-  carrier.fetch(tile, kb, kb >= lo_all && kb + 63 <= p0);
+  carrier.plan(tid, tile, kb);
+  const auto whole = [&](int block) { return block >= lo_all && block + 63 <= p0; };
+  carrier.look_up(tile, kb, whole(kb));
+  carrier.fetch(tile, kb, whole(kb));
+  if (kb + 64 <= hi) carrier.look_up(tile, kb + 64, whole(kb + 64));
   carrier.put(staged);
   __syncthreads();
 #define TURN(FULL)                                                                                            \
   {                                                                                                           \
     const int next = kb + 64;                                                                                 \
     const bool more = next <= hi;                                                                             \
-    if (more) carrier.fetch(tile, next, next >= lo_all && next + 63 <= p0);                                  \
+    if (more) carrier.fetch(tile, next, whole(next));                                                         \
+    if (next + 64 <= hi) carrier.look_up(tile, next + 64, whole(next + 64));                                  \
     if (heads_here > 0)                                                                                       \
       shared_block<D, HG, FULL>(staged + cur * Staged<D>::BYTES, kb, col, g, my_pos, my_lo, scale_log2, qf, acc, m, l); \
-    if (more) carrier.put(staged + (cur ^ 1) * Staged<D>::BYTES);                                            \
+    if (more) carrier.put(staged + (cur ^ 1) * Staged<D>::BYTES);                                             \
     __syncthreads();                                                                                          \
     cur ^= 1;                                                                                                 \
   }
