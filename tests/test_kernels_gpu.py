@@ -257,9 +257,12 @@ def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, windo
 @pytest.mark.parametrize("geometry,lengths,q_lens", [((14, 2, 64, 16), [4500, 333], [4400, 50]),
                                                      ((28, 2, 64, 16), [2300, 40], [2200, 33])])
 @pytest.mark.parametrize("window", [None, 1000])
-def test_prefill_attention_with_all_heads_of_a_group_in_one_wave(ops, ref, geometry, lengths, q_lens, window):
+def test_prefill_attention_with_all_heads_of_a_group_in_one_wave(ops, ref, geometry, lengths, q_lens, window,
+                                                                 monkeypatch):
     # Head size 64, seven (or twice seven) query heads per kv head and so many tiles that the launcher gives a
     # wave all seven heads: portions that start and end inside pages and tiles, with and without a window.
+    # (With this many tiles the launcher itself would take the kernel whose waves share their blocks.)
+    monkeypatch.setattr(ops, "prefill_shared", -1)
     n_q, n_kv, d, page_size = geometry
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=23)
@@ -278,8 +281,8 @@ def test_prefill_attention_with_all_heads_of_a_group_in_one_wave(ops, ref, geome
     torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
 
 
-@pytest.mark.parametrize("geometry", [(28, 4, 128, 16), (12, 2, 128, 32), (5, 1, 96, 48), (16, 2, 128, 16),
-                                      (24, 2, 128, 64), (3, 1, 128, 16)])
+@pytest.mark.parametrize("geometry", [(28, 4, 128, 16), (12, 2, 128, 32), (5, 1, 64, 48), (16, 2, 128, 16),
+                                      (24, 2, 128, 64), (3, 1, 128, 16), (14, 2, 64, 16)])
 @pytest.mark.parametrize("window", [None, 100])
 def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, geometry, window, monkeypatch):
     # The kernel whose four waves take one block of keys from LDS for up to eight query heads of a kv head: five,
@@ -320,9 +323,10 @@ def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles_of_large_
         torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=31)
     batch = make_batch(lengths, q_lens)
     assert ops.prefill_shared == 0 and ops.prefill_waves == 0 and ops.prefill_heads_per_wave == 0
-    assert ops.lib.ta_prefill_attention_shared_pays(batch.q_tiles.shape[0], n_q, n_kv, d) == 1
-    assert ops.lib.ta_prefill_attention_shared_pays(batch.q_tiles.shape[0], n_q, n_kv, 64) == 0
-    assert ops.lib.ta_prefill_attention_shared_pays(100, n_q, n_kv, d) == 0
+    pays = ops.lib.ta_prefill_attention_shared_pays
+    assert pays(batch.q_tiles.shape[0], n_q, n_kv, d, 2560) == 1
+    assert pays(batch.q_tiles.shape[0], n_q, n_kv, 96, 2560) == 0 and pays(batch.q_tiles.shape[0], 16, 4, d, 2560) == 0
+    assert pays(64, n_q, n_kv, d, 2048) == 0 and pays(64, n_q, n_kv, d, 4096) == 1 and pays(63, n_q, n_kv, d, 4096) == 0
     scale = 1.0 / math.sqrt(d)
     out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
     ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,

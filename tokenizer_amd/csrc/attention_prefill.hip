@@ -317,7 +317,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const void* k_
 }
 
 // The kernel whose waves share a block of keys through LDS (attention_prefill_shared.hip).
-extern "C" int ta_prefill_attention_shared_pays(int n_tiles, int n_q, int n_kv, int d);
+extern "C" int ta_prefill_attention_shared_pays(int n_tiles, int n_q, int n_kv, int d, int reach);
 extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                                 const void* vt_pages, const void* tiles, int n_tiles,
                                                 const void* cu_q, const void* first_position,
@@ -327,8 +327,8 @@ extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, voi
 // Returns -2 for a head size without an instance (the caller then uses another kernel).
 // max_keys: the highest position of the batch + 1 (a hint for the number of waves per tile).
 // shared: 1 = the workgroup-shared kernel wherever it has an instance, -1 = never, 0 = where it is the faster one
-// (which depends on the shape of the launch only, never on the context, so that a launch recorded for a range of
-// contexts and a launch for the exact context make the same choice).
+// (by the shape of the launch and the planned reach, so that a launch recorded for a range of contexts and a
+// launch for the exact context make the same choice).
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
@@ -338,7 +338,7 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
   if (shared > 0 || (shared == 0 && heads_per_wave == 0 && waves == 0 &&
-                     ta_prefill_attention_shared_pays(n_tiles, n_q, n_kv, d))) {
+                     ta_prefill_attention_shared_pays(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window)))) {
     const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
                                                         first_position, block_table, table_stride, n_q, n_kv, d,
                                                         page_size, window, scale, stream);

@@ -1,28 +1,39 @@
 // Prompt attention for many query heads per kv head and long reaches: the workgroup of a tile of 16 tokens and one
-// kv head holds NW waves, each with HG of the query heads that share the kv head, and all of them walk the
-// same blocks of 64 keys.  A block's keys and values come from the pages once for the whole workgroup, through
-// registers into LDS, two buffers deep: the next block is on its way while the matrix cores work on the
-// current one, and every wave takes its fragments from LDS.  Against the kernel in attention_prefill.hip
-// (each wave fetches its own blocks for its own two heads) a key is read from the cache 1/NW as often and
-// no wave waits for memory with nothing else to do; it pays where the pages' traffic or its latency bound
-// that kernel: large heads, long prompts.  Same fragment layouts and key order as there: S^T = K Q^T and
-// O^T = V^T P^T with 16x16x32 MFMAs, token index in `lane % 16`, softmax online in float, probabilities
-// rounded to bfloat16 for the second product.
+// kv head holds four waves, each with HG of the query heads that share the kv head, and all of them walk the
+// same blocks of 64 keys.  A block's keys and values come from the pages once for the whole workgroup, by loads
+// that write straight into LDS (no register on the way), two buffers deep: the next block is on its way while
+// the matrix cores work on the current one, and every wave takes its fragments from LDS.  Against the kernel in
+// attention_prefill.hip (each wave fetches its own blocks for its own two heads) a key is read from the cache a
+// quarter as often and no wave waits for memory with nothing else to do; it pays where the pages' traffic or
+// its latency bound that kernel: large heads, long prompts.  Same fragment layouts and key order as there:
+// S^T = K Q^T and O^T = V^T P^T with 16x16x32 MFMAs, token index in `lane % 16`, softmax online in float,
+// probabilities rounded to bfloat16 for the second product.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef uint32_t piece_t __attribute__((ext_vector_type(4)));   // sixteen bytes on their way from a page to LDS
 
-// A block in LDS: 64 rows of keys, then D rows of 64 values each (V^T).  Rows are 16 bytes longer than their
-// contents, so that the rows which eight neighbouring lanes read at once start four banks apart.
+#define SHARED_WAVES 4       // waves of a workgroup: each brings one of a block's four runs of sixteen keys
+
+// A block in LDS.  A load that writes into LDS puts lane i's sixteen bytes at its base + 16 i, so what one
+// instruction brings is one KB on end, and where a piece lands is decided by which lane asks for it.
+// Keys: 64 rows of D / 8 pieces, no padding; the piece that holds elements 8 p .. 8 p + 7 of key k stands at
+// place p ^ swizzle(k), so that the eight rows which neighbouring lanes read at once lie in different banks.
+// Values: run by run, D rows of the run's sixteen keys (32 bytes), which neighbouring lanes read 32 bytes apart.
 template <int D>
 struct Staged {
-  static constexpr int K_ROW = 2 * D + 16;
-  static constexpr int V_ROW = 2 * 64 + 16;
+  static_assert(D == 64 || D == 128, "a key row must be a power of two of pieces for the swizzle");
+  static constexpr int PIECES = D / 8;                      // 16-byte pieces of a key row
+  static constexpr int K_ROW = 2 * D;
   static constexpr int K_BYTES = 64 * K_ROW;
-  static constexpr int BYTES = K_BYTES + D * V_ROW;
+  static constexpr int V_RUN = 32 * D;
+  static constexpr int BYTES = K_BYTES + 4 * V_RUN;
+  static constexpr int KEYS_A_LOAD = 64 / PIECES;           // key rows that one instruction of a wave brings
+  static constexpr int K_LOADS = 16 / KEYS_A_LOAD;          // instructions for a run's keys
+  static constexpr int V_LOADS = D / 32;                    // and for its values (32 rows of D each)
+  // Keys k, k + 1, k + 2, k + 3 and k + 8 .. k + 11 (k a multiple of 4) are read at once.
+  __device__ static constexpr int swizzle(int key) { return (key & 3) | ((key >> 1) & 4); }
 };
 
 __device__ __forceinline__ bf16x8 sh_zero8() {
@@ -41,148 +52,103 @@ struct SharedTile {
   int lo_page, hi_page;       // their places in the block table
 };
 
-// What a thread carries of every block: the same pieces of each of the block's four runs of sixteen keys (a run
-// lies inside one page), so that per block only four page numbers change, which are the same for the whole
-// workgroup, and a load is a scalar base plus an offset that the lane worked out once.
-template <int D, int THREADS>
+// What a wave brings of every block: one of its four runs of sixteen keys (a run lies inside one page), so
+// that per block a wave looks up one page number and every load is a scalar base plus an offset that the lane
+// worked out once.
+template <int D>
 struct Carrier {
-  static constexpr int RUN_PIECES = 2 * D;                  // 16 keys of D / 8 pieces; as many of the values
-  static constexpr int ROUNDS = (RUN_PIECES + THREADS - 1) / THREADS;
-  uint32_t k_from[ROUNDS], v_from[ROUNDS];                  // element offsets inside a run's part of its page
-  uint32_t k_to[ROUNDS], v_to[ROUNDS];                      // byte offsets inside a block in LDS (run 0)
-  bool mine[ROUNDS];
-  int v_first[ROUNDS];                                      // first key of the value piece, within its run
-  piece_t k[4][ROUNDS], v[4][ROUNDS];
-  int at_page, at_slot;                                     // where the next run to look up lies: index into the block table, slot in the page
-  int page[4], slot[4];                                     // of the runs of the block to fetch next (the same for all threads)
-  bool there[4];                                            // whether the run holds a key of lo..hi
+  typedef Staged<D> S;
+  int run;                                                  // which of a block's runs
+  uint32_t k_from[S::K_LOADS];                              // byte offsets of the lane's pieces inside the run's part of its page
+  uint32_t v_from;
+  int at_page, at_slot;                                     // where the run of the next block to look up lies: index into the block table, slot in the page
+  int step_pages, step_slots;                               // 64 keys on
+  int page, slot;                                           // of the run of the block to fetch next
   int page_size;
   uint32_t page_elements, first_element;                    // elements of a page (all kv heads); where this kv head's begin
 
   // first_key: the first key of the first block.
-  __device__ __forceinline__ void plan(int tid, const SharedTile& tile, int first_key) {
+  __device__ __forceinline__ void plan(int wave, int lane, const SharedTile& tile, int first_key) {
+    run = wave;
     page_size = tile.page_size;
     page_elements = (uint32_t)tile.n_kv * page_size * D;
     first_element = (uint32_t)tile.kvh * page_size * D;
-    at_page = first_key / page_size;
-    at_slot = first_key % page_size;
+    at_page = (first_key + 16 * run) / page_size;
+    at_slot = (first_key + 16 * run) % page_size;
+    step_pages = 64 / page_size;
+    step_slots = 64 % page_size;
 #pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-      const int piece = r * THREADS + tid;
-      mine[r] = RUN_PIECES % THREADS == 0 || piece < RUN_PIECES;
-      const int key = piece / (D / 8), part = piece % (D / 8);
-      k_from[r] = (uint32_t)(key * D + part * 8);
-      k_to[r] = (uint32_t)(key * Staged<D>::K_ROW + part * 16);
-      const int d = piece >> 1, half = piece & 1;
-      v_from[r] = (uint32_t)(d * page_size + half * 8);
-      v_to[r] = (uint32_t)(Staged<D>::K_BYTES + d * Staged<D>::V_ROW + half * 16);
-      v_first[r] = 8 * half;
+    for (int j = 0; j < S::K_LOADS; ++j) {
+      const int key = S::KEYS_A_LOAD * j + lane / S::PIECES;             // within the run; the run starts at a multiple of 16
+      const int part = (lane % S::PIECES) ^ S::swizzle(key);            // the piece that belongs at this lane's place
+      k_from[j] = (uint32_t)(key * D + part * 8) * 2;
     }
+    v_from = (uint32_t)((lane >> 1) * page_size + (lane & 1) * 8) * 2;
   }
 
-  // Where the four runs of block `kb` lie: their pages and slots, looked up a turn before the block is fetched,
-  // so that no wave waits for a page number.  Blocks are looked up in order.  `full`: every key of the block
-  // exists and is seen by every token.  Otherwise a run without a key of lo..hi (before `lo`: its page may have
-  // been given back; after `hi`: it may not exist yet) borrows the page of `lo` or `hi`, a valid address.
+  // Where the wave's run of block `kb` lies, looked up a turn before the block is fetched, so that no wave waits
+  // for a page number.  Blocks are looked up in order.  `full`: every key of the block exists and is seen by
+  // every token.  Otherwise a run without a key of lo..hi (before `lo`: its page may have been given back; after
+  // `hi`: it may not exist yet) borrows the page of `lo` or `hi`, a valid address; what lies there never counts
+  // (scores outside a token's range are masked by selection, values outside lo..hi are set to zero when read).
   __device__ __forceinline__ void look_up(const SharedTile& tile, int kb, bool full) {
-    if (full) {                                            // the usual block: nothing to decide per run
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        page[q] = tile.table[at_page];
-        slot[q] = at_slot;
-        there[q] = true;
-        step();
-      }
-      return;
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int key = kb + 16 * q;
-      int index = at_page;
-      there[q] = key + 15 >= tile.lo && key <= tile.hi;
+    int index = at_page;
+    if (!full) {
+      const int key = kb + 16 * run;
       if (key + 15 < tile.lo) index = tile.lo_page;
       if (key > tile.hi) index = tile.hi_page;
-      page[q] = tile.table[index];
-      slot[q] = at_slot;
-      step();
     }
-  }
-
-  // On to the next run: pages hold whole runs.
-  __device__ __forceinline__ void step() {
-    at_slot += 16;
+    page = tile.table[index];
+    slot = at_slot;
+    at_page += step_pages;
+    at_slot += step_slots;
     if (at_slot >= page_size) {
-      at_slot = 0;
+      at_slot -= page_size;
       ++at_page;
     }
   }
 
-  // The block that was looked up last, from the pages into registers.  Unless the block is `full`, the values
-  // of a borrowed run become zero, as do values past `hi` (slots never written): a probability of zero times
-  // whatever lies there must stay zero.  Keys need no such care, their scores are masked by selection.
-  __device__ __forceinline__ void fetch(const SharedTile& tile, int kb, bool full) {
+  // The run that was looked up last, from its page straight into `buf`.  The loads are under way when this
+  // returns; `landed` waits for them.
+  __device__ __forceinline__ void fetch(const SharedTile& tile, char* buf) const {
+    typedef const void __attribute__((address_space(1)))* from_t;
+    typedef void __attribute__((address_space(3)))* to_t;
+    const uint32_t head = (uint32_t)page * page_elements + first_element;
+    const char* k_run = reinterpret_cast<const char*>(tile.k_pages + (head + (uint32_t)slot * D));
+    const char* v_run = reinterpret_cast<const char*>(tile.vt_pages + (head + (uint32_t)slot));
+    char* k_to = buf + run * 16 * S::K_ROW;
+    char* v_to = buf + S::K_BYTES + run * S::V_RUN;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint32_t head = (uint32_t)page[q] * page_elements + first_element;
-      const bf16_t* k_run = tile.k_pages + (head + (uint32_t)slot[q] * D);
-      const bf16_t* v_run = tile.vt_pages + (head + (uint32_t)slot[q]);
+    for (int j = 0; j < S::K_LOADS; ++j)
+      __builtin_amdgcn_global_load_lds((from_t)(k_run + k_from[j]), (to_t)(k_to + j * 1024), 16, 0, 0);
 #pragma unroll
-      for (int r = 0; r < ROUNDS; ++r) {
-        if (!mine[r]) continue;
-        k[q][r] = *reinterpret_cast<const piece_t*>(k_run + k_from[r]);
-        v[q][r] = *reinterpret_cast<const piece_t*>(v_run + v_from[r]);
-      }
-    }
-    if (full) return;
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int r = 0; r < ROUNDS; ++r) {
-        if (!mine[r]) continue;
-        const int left = there[q] ? tile.hi - (kb + 16 * q + v_first[r]) : -1;     // keys of this piece that exist: 0..left
-        if (left < 7) {
-          piece_t x = v[q][r];
-          if (left < 0) x.x = 0; else if (left < 1) x.x &= 0xffffu;
-          if (left < 2) x.y = 0; else if (left < 3) x.y &= 0xffffu;
-          if (left < 4) x.z = 0; else if (left < 5) x.z &= 0xffffu;
-          if (left < 6) x.w = 0; else x.w &= 0xffffu;
-          v[q][r] = x;
-        }
-      }
+    for (int j = 0; j < S::V_LOADS; ++j)
+      __builtin_amdgcn_global_load_lds((from_t)(v_run + v_from + (uint32_t)j * 64 * page_size), (to_t)(v_to + j * 1024), 16, 0, 0);
   }
 
-  __device__ __forceinline__ void put(char* buf) const {
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int r = 0; r < ROUNDS; ++r) {
-        if (!mine[r]) continue;
-        *reinterpret_cast<piece_t*>(buf + k_to[r] + q * 16 * Staged<D>::K_ROW) = k[q][r];
-        *reinterpret_cast<piece_t*>(buf + v_to[r] + q * 32) = v[q][r];
-      }
-  }
+  // All that this wave fetched has arrived in LDS (vmcnt 0; the other counters stay as they are).
+  __device__ __forceinline__ static void landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 };
 
 // One step of the online softmax of a wave's HG heads over the block of 64 keys in `buf`.  Row r of the first
 // product's instruction t of a half of 32 keys is key 8 (r / 4) + 4 t + r % 4 of the half, whose score then lies
 // in the lane group that holds that key in the second product (lane group g: keys 8g .. 8g+7).
+// lo, hi: the first and last key that any token of the tile sees (unless FULL, values outside them may be anything).
 template <int D, int HG, bool FULL>
-__device__ __forceinline__ void shared_block(const char* buf, int kb, int col, int g, int my_pos, int my_lo, float c,
-                                             const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16],
+__device__ __forceinline__ void shared_block(const char* buf, int kb, int col, int g, int my_pos, int my_lo, int lo, int hi,
+                                             float c, const bf16x8 (&qf)[HG][D / 32], floatx4 (&acc)[HG][D / 16],
                                              float (&m)[HG], float (&l)[HG]) {
-  constexpr int KS = (D + 31) / 32;
+  constexpr int KS = D / 32;
   constexpr int DB = D / 16;
   float s[HG][16];
+  const int turned = (col & 3) | ((col >> 2) & 1) << 2;    // swizzle of the lane's keys: the same in every instruction
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     const int key = 32 * (t >> 1) + 8 * (col >> 2) + 4 * (t & 1) + (col & 3);
     bf16x8 kf[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      kf[ks] = sh_zero8();
-      if (ks * 32 + 8 * g < D)
-        kf[ks] = *reinterpret_cast<const bf16x8*>(buf + key * Staged<D>::K_ROW + (ks * 32 + 8 * g) * 2);
-    }
+    for (int ks = 0; ks < KS; ++ks)
+      kf[ks] = *reinterpret_cast<const bf16x8*>(buf + key * Staged<D>::K_ROW + ((ks * 4 + g) ^ turned) * 16);
 #pragma unroll
     for (int h = 0; h < HG; ++h) {
       floatx4 st = (floatx4){0.f, 0.f, 0.f, 0.f};
@@ -233,26 +199,34 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
   for (int u = 0; u < 2; ++u)
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      const bf16x8 vf = *reinterpret_cast<const bf16x8*>(buf + Staged<D>::K_BYTES + (db * 16 + col) * Staged<D>::V_ROW +
-                                                         (32 * u + 8 * g) * 2);
+      bf16x8 vf = *reinterpret_cast<const bf16x8*>(buf + Staged<D>::K_BYTES + (2 * u + (g >> 1)) * Staged<D>::V_RUN +
+                                                   (db * 16 + col) * 32 + (g & 1) * 16);
+      if (!FULL) {
+        // A probability of zero times whatever lies in a slot that was never written, or in a borrowed page,
+        // must stay zero.
+        const int first = kb + 32 * u + 8 * g;             // the lane's keys: first .. first + 7
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (first + i > hi || first + i < lo) vf[i] = (__bf16)0.0f;
+      }
 #pragma unroll
       for (int h = 0; h < HG; ++h) acc[h][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[h][u], acc[h][db], 0, 0, 0);
     }
 }
 
 // Arguments as in prefill_attention_kernel.  Dynamic LDS: two blocks (2 * Staged<D>::BYTES).
-template <int D, int HG, int NW>
-__global__ void __launch_bounds__(NW * WAVE, 1)
+template <int D, int HG>
+__global__ void __launch_bounds__(SHARED_WAVES * WAVE, 1)
 prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                 const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                                 const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
                                 const int* __restrict__ first_position, const int* __restrict__ block_table,
                                 int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
-  constexpr int KS = (D + 31) / 32;
+  constexpr int KS = D / 32;
   constexpr int DB = D / 16;
-  constexpr int THREADS = NW * WAVE;
+  constexpr int NW = SHARED_WAVES;
   extern __shared__ __attribute__((aligned(16))) char staged[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int group = n_q / n_kv;
   const int head_blocks = (group + HG * NW - 1) / (HG * NW);
@@ -261,7 +235,7 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   const int which = blockIdx.x % per_tile;
   const int kvh = which / head_blocks, hb = which % head_blocks;
   const int first_head = hb * HG * NW + wave * HG;            // among the heads of the kv head
-  const int heads_here = max(0, min(HG, group - first_head));  // a wave past the last head only carries blocks
+  const int heads_here = max(0, min(HG, group - first_head));  // a wave past the last head only brings blocks
   const int head0 = kvh * group + first_head;
   const int tile_index = n_tiles - 1 - blockIdx.x / per_tile;
   const int entry = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index]);
@@ -292,10 +266,9 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   for (int h = 0; h < HG; ++h)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int d0 = ks * 32 + 8 * g;
       qf[h][ks] = sh_zero8();
-      if (h < heads_here && d0 < D)
-        qf[h][ks] = *reinterpret_cast<const bf16x8*>(q + (size_t)my_row * q_stride + (size_t)(head0 + h) * D + d0);
+      if (h < heads_here)
+        qf[h][ks] = *reinterpret_cast<const bf16x8*>(q + (size_t)my_row * q_stride + (size_t)(head0 + h) * D + ks * 32 + 8 * g);
     }
   floatx4 acc[HG][DB];
   float m[HG], l[HG];
@@ -309,27 +282,28 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
 
   // Blocks come in three runs (the window's edge, those every token sees whole, the diagonal), each a loop of
   // its own over one variant of the block, so that the accumulators stay in the same registers within a loop.
-  // Every thread goes through every turn: the barrier at its end hands the buffer that was just filled to the
-  // next turn, and the buffer that was just read to the turn after it.
+  // A turn asks for the next block into the buffer that the turn before read, works on the current one, waits
+  // for what it asked for, and meets the other waves: after the barrier every wave's part of the next block
+  // has landed, and nobody reads the current one any more.
   int kb = (lo / 64) * 64;
   int cur = 0;
-  Carrier<D, THREADS> carrier;
-  carrier.plan(tid, tile, kb);
+  Carrier<D> carrier;
+  carrier.plan(wave, lane, tile, kb);
   const auto whole = [&](int block) { return block >= lo_all && block + 63 <= p0; };
   carrier.look_up(tile, kb, whole(kb));
-  carrier.fetch(tile, kb, whole(kb));
+  carrier.fetch(tile, staged);
   if (kb + 64 <= hi) carrier.look_up(tile, kb + 64, whole(kb + 64));
-  carrier.put(staged);
+  carrier.landed();
   __syncthreads();
 #define TURN(FULL)                                                                                            \
   {                                                                                                           \
     const int next = kb + 64;                                                                                 \
-    const bool more = next <= hi;                                                                             \
-    if (more) carrier.fetch(tile, next, whole(next));                                                         \
+    if (next <= hi) carrier.fetch(tile, staged + (cur ^ 1) * Staged<D>::BYTES);                               \
     if (next + 64 <= hi) carrier.look_up(tile, next + 64, whole(next + 64));                                  \
     if (heads_here > 0)                                                                                       \
-      shared_block<D, HG, FULL>(staged + cur * Staged<D>::BYTES, kb, col, g, my_pos, my_lo, scale_log2, qf, acc, m, l); \
-    if (more) carrier.put(staged + (cur ^ 1) * Staged<D>::BYTES);                                             \
+      shared_block<D, HG, FULL>(staged + cur * Staged<D>::BYTES, kb, col, g, my_pos, my_lo, lo, hi, scale_log2, \
+                                qf, acc, m, l);                                                               \
+    carrier.landed();                                                                                         \
     __syncthreads();                                                                                          \
     cur ^= 1;                                                                                                 \
   }
@@ -357,38 +331,42 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   }
 }
 
-template <int D, int HG, int NW>
+template <int D, int HG>
 static int launch_shared(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
                          const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
                          const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
                          float scale, hipStream_t stream) {
   const int group = n_q / n_kv;
-  const long workgroups = (long)n_tiles * n_kv * ((group + HG * NW - 1) / (HG * NW));
+  const long workgroups = (long)n_tiles * n_kv * ((group + HG * SHARED_WAVES - 1) / (HG * SHARED_WAVES));
   if (workgroups > 0x7fffffffL) return -1;
   constexpr int lds = 2 * Staged<D>::BYTES;
   static_assert(lds <= 160 * 1024, "two blocks must fit a compute unit's LDS");
   if (lds > 48 * 1024) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_shared_kernel<D, HG, NW>),
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_shared_kernel<D, HG>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (err != hipSuccess) return (int)err;
   }
-  prefill_attention_shared_kernel<D, HG, NW><<<(unsigned)workgroups, NW * WAVE, lds, stream>>>(
+  prefill_attention_shared_kernel<D, HG><<<(unsigned)workgroups, SHARED_WAVES * WAVE, lds, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
       n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
       window, scale * 1.4426950408889634f);
   return LAUNCH_STATUS();
 }
 
-// Where the workgroup-shared kernel is the faster one: five to eight query heads per kv head (or a multiple of
-// that many) fill its four waves, and the launch must have two workgroups or so for every compute unit, because a
-// workgroup walks all its keys alone (measured at head size 128 on 256 compute units: 0.5-0.95x with 64 to 256
-// workgroups, 1.4-1.9x from 512 on, for 5, 6, 7 and 8 heads per kv head; at head size 64 the two kernels are
-// level even at 32,768 tokens, so it has no instance there).
-extern "C" int ta_prefill_attention_shared_pays(int n_tiles, int n_q, int n_kv, int d) {
-  if (d != 96 && d != 128) return 0;
+// Where the workgroup-shared kernel is the faster one: five to eight query heads per kv head (or more) fill
+// its four waves, and the launch must fill the device although a workgroup walks all its keys alone: two
+// workgroups for every compute unit, or one where the walk is long.  reach: how far back the farthest-seeing
+// token looks, as the launcher plans it.  (Measured on 256 compute units, 7 heads per kv head, against the
+// per-wave kernel.  Head size 128: 0.75x with 128 workgroups; with 256: 0.84x at a reach of 2,048, 1.1-1.35x at
+// 4,096, 1.4x at 8,192; with 512 and more 1.5x at 2,048 tokens, 2.1x at 8,192, 2.2x at 32,768; 1.5x with 5 or 6
+// heads per kv head, where a wave only brings blocks.  Head size 64: 0.76-0.93x below 512 workgroups and a
+// reach of 4,096, 1.02-1.08x at these marks, 1.25x at 8,192 tokens, 1.35x at 32,768.)
+extern "C" int ta_prefill_attention_shared_pays(int n_tiles, int n_q, int n_kv, int d, int reach) {
+  if (d != 64 && d != 128) return 0;
   const int group = n_q / n_kv;
   if (group < 5) return 0;
-  return (long)n_tiles * n_kv * ((group + 7) / 8) >= 512;
+  const long workgroups = (long)n_tiles * n_kv * ((group + 7) / 8);
+  return workgroups >= 512 || (workgroups >= 256 && reach >= 4096);
 }
 
 // Returns -2 for a head size without an instance (the caller then uses the other kernel).
@@ -399,10 +377,10 @@ extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, voi
                                                 int page_size, int window, float scale, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
-#define SIZE(DD) case DD: return launch_shared<DD, 2, 4>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
+#define SIZE(DD) case DD: return launch_shared<DD, 2>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
   switch (d) {
-    SIZE(96) SIZE(128)
+    SIZE(64) SIZE(128)
     default: return -2;
   }
 #undef SIZE
