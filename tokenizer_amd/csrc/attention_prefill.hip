@@ -317,18 +317,21 @@ static int launch_prefill(const void* q, int q_stride, void* out, const void* k_
 }
 
 // The kernel whose waves share a block of keys through LDS (attention_prefill_shared.hip).
-extern "C" int ta_prefill_attention_shared_pays(int n_tiles, int n_q, int n_kv, int d, int reach);
+extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, int d, int reach);
 extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                                 const void* vt_pages, const void* tiles, int n_tiles,
                                                 const void* cu_q, const void* first_position,
                                                 const void* block_table, int table_stride, int n_q, int n_kv, int d,
-                                                int page_size, int window, float scale, hipStream_t stream);
+                                                int page_size, int window, float scale, int heads_per_wave,
+                                                hipStream_t stream);
 
 // Returns -2 for a head size without an instance (the caller then uses another kernel).
 // max_keys: the highest position of the batch + 1 (a hint for the number of waves per tile).
-// shared: 1 = the workgroup-shared kernel wherever it has an instance, -1 = never, 0 = where it is the faster one
-// (by the shape of the launch and the planned reach, so that a launch recorded for a range of contexts and a
-// launch for the exact context make the same choice).
+// shared: 1 = the workgroup-shared kernel wherever it has an instance (with heads_per_wave = 1 or 2 heads a wave,
+// 0 = its own choice), -1 = never, 0 = where it is the faster one (by the shape of the launch and the planned
+// reach, so that a launch recorded for a range of contexts and a launch for the exact context make the same
+// choice).  waves: waves that share a tile's keys in the per-wave kernel (1, 2, 4; 0 = by the reach); asking
+// for a number asks for that kernel.
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
@@ -337,29 +340,16 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
                                          hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
-  if (shared > 0 || (shared == 0 && heads_per_wave == 0 && waves == 0 &&
-                     ta_prefill_attention_shared_pays(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window)))) {
-    const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
-                                                        first_position, block_table, table_stride, n_q, n_kv, d,
-                                                        page_size, window, scale, stream);
-    if (status != -2) return status;
-  }
-  if (d == 64 && heads_per_wave == 0 && (n_q / n_kv) % 7 == 0 && planned_reach(max_keys, window) > 768) {
-    // Seven query heads per kv head (or fourteen) and enough tiles to fill the device with a quarter of the
-    // workgroups: a wave takes all seven heads, so that every key tile is read once instead of four times and no
-    // head slot of a wave stays empty (measured at 14 / 2 heads: level at 2,560 tokens, 1.13x at 3,072, 1.2x at
-    // 4,096, 1.3x from 8,192 on; with fewer tiles the device runs out of workgroups: 0.86x at 2,048).
-    const long workgroups = (long)n_tiles * n_kv * (n_q / n_kv / 7);
-    if (workgroups >= 384) {
-      heads_per_wave = 7;
-      if (waves == 0) waves = workgroups < 1024 ? 4 : 2;
+  if (shared >= 0 && waves == 0) {
+    int heads = ta_prefill_attention_shared_plan(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window));
+    if (shared > 0) heads = (heads_per_wave == 1 || heads_per_wave == 2) ? heads_per_wave : heads ? heads : 2;
+    if (heads) {
+      const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
+                                                          first_position, block_table, table_stride, n_q, n_kv, d,
+                                                          page_size, window, scale, heads, stream);
+      if (status != -2) return status;
     }
   }
-#define D64(HG) if (d == 64 && heads_per_wave == HG) \
-    return launch_prefill<64, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position, \
-                                  block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, stream);
-  D64(1) D64(7)
-#undef D64
 #define CASE(DD, HG) case DD: return launch_prefill<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, stream);
   switch (d) {

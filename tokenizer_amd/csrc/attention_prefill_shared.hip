@@ -353,35 +353,44 @@ static int launch_shared(const void* q, int q_stride, void* out, const void* k_p
   return LAUNCH_STATUS();
 }
 
-// Where the workgroup-shared kernel is the faster one: five to eight query heads per kv head (or more) fill
-// its four waves, and the launch must fill the device although a workgroup walks all its keys alone: two
-// workgroups for every compute unit, or one where the walk is long.  reach: how far back the farthest-seeing
-// token looks, as the launcher plans it.  (Measured on 256 compute units, 7 heads per kv head, against the
-// per-wave kernel.  Head size 128: 0.75x with 128 workgroups; with 256: 0.84x at a reach of 2,048, 1.1-1.35x at
-// 4,096, 1.4x at 8,192; with 512 and more 1.5x at 2,048 tokens, 2.1x at 8,192, 2.2x at 32,768; 1.5x with 5 or 6
-// heads per kv head, where a wave only brings blocks.  Head size 64: 0.76-0.93x below 512 workgroups and a
-// reach of 4,096, 1.02-1.08x at these marks, 1.25x at 8,192 tokens, 1.35x at 32,768.)
-extern "C" int ta_prefill_attention_shared_pays(int n_tiles, int n_q, int n_kv, int d, int reach) {
+// Whether the workgroup-shared kernel is the faster one, and with how many heads a wave: 0 = no, else 1 or 2.
+// Five to eight query heads per kv head (or more) fill its four waves at two heads a wave, and the launch must
+// fill the device although a workgroup walks all its keys alone: two or three workgroups for every compute unit,
+// or one where the walk is long.  With one head a wave there are twice the workgroups, each reading its blocks
+// for half the heads: the better cut while two heads a wave give fewer than 1,024 workgroups.
+// reach: how far back the farthest-seeing token looks, as the launcher plans it.
+// (Measured on 256 compute units, 7 heads per kv head, against the per-wave kernel.  Two heads a wave, head size
+// 128: 0.75x with 128 workgroups; with 256: 0.84x at a reach of 2,048, 1.1-1.35x at 4,096, 1.4x at 8,192; with 512
+// and more 1.5x at 2,048 tokens, 2.1x at 8,192, 2.2x at 32,768; 1.5x with 5 or 6 heads per kv head, where a wave
+// only brings blocks.  Head size 64: 0.76-0.93x below 512 workgroups, 1.25x at 8,192 tokens, 1.35x at 32,768.
+// One head a wave against two: head size 64 1.26x at 2,048 tokens (where it is level with the per-wave kernel),
+// 1.27x at 3,072, 1.23x at 4,096, 0.95x at 8,192; head size 128 1.05x at 2,048, 0.8x at 8,192.)
+extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, int d, int reach) {
   if (d != 64 && d != 128) return 0;
   const int group = n_q / n_kv;
   if (group < 5) return 0;
-  const long workgroups = (long)n_tiles * n_kv * ((group + 7) / 8);
-  return workgroups >= 512 || (workgroups >= 256 && reach >= 4096);
+  const long two = (long)n_tiles * n_kv * ((group + 7) / 8), one = (long)n_tiles * n_kv * ((group + 3) / 4);
+  if (one < 768 && !(two >= 256 && reach >= 4096)) return 0;
+  return (two >= 1024 || one < 768) ? 2 : 1;
 }
 
 // Returns -2 for a head size without an instance (the caller then uses the other kernel).
+// heads_per_wave: 1 or 2.
 extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                                 const void* vt_pages, const void* tiles, int n_tiles,
                                                 const void* cu_q, const void* first_position,
                                                 const void* block_table, int table_stride, int n_q, int n_kv, int d,
-                                                int page_size, int window, float scale, hipStream_t stream) {
+                                                int page_size, int window, float scale, int heads_per_wave,
+                                                hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
-#define SIZE(DD) case DD: return launch_shared<DD, 2>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
+  if (n_kv <= 0 || n_q % n_kv || page_size % 16 || heads_per_wave < 1 || heads_per_wave > 2) return -1;
+#define GO(DD, HG) return launch_shared<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
+#define SIZE(DD) case DD: if (heads_per_wave == 1) GO(DD, 1) GO(DD, 2)
   switch (d) {
     SIZE(64) SIZE(128)
     default: return -2;
   }
 #undef SIZE
+#undef GO
 }

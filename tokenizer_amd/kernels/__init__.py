@@ -82,7 +82,7 @@ class Ops:
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16",
-                     "ta_prefill_attention_shared_pays",
+                     "ta_prefill_attention_shared_plan",
                      "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16",
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
@@ -277,7 +277,7 @@ class Ops:
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
     use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
     prefill_waves = 0          # waves that share a tile's keys in the prompt kernel: 0 lets the launcher choose
-    prefill_heads_per_wave = 0    # 0: the kernel's own choice for the head size
+    prefill_heads_per_wave = 0    # heads a wave (1 or 2) of the workgroup-shared prompt kernel when it is asked for; 0: its choice
     prefill_shared = 0            # the prompt kernel whose waves share a block of keys through LDS: 1 = wherever it has
     #                               an instance, -1 = never, 0 = where the launcher expects it to be the faster one
     target_workgroups = 1024      # what the split of the key range aims at
