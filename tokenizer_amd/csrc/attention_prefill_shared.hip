@@ -3,8 +3,8 @@
 // same blocks of 64 keys.  A block's keys and values come from the pages once for the whole workgroup, by loads
 // that write straight into LDS (no register on the way), two buffers deep: the next block is on its way while
 // the matrix cores work on the current one, and every wave takes its fragments from LDS.  Against the kernel in
-// attention_prefill.hip (each wave fetches its own blocks for its own two heads) a key is read from the cache a
-// quarter as often and no wave waits for memory with nothing else to do; it pays where the pages' traffic or
+// attention_prefill.hip (each wave fetches its own blocks for its own two heads) a key is read from the cache half
+// or a quarter as often (one or two heads a wave) and no wave waits for memory with nothing else to do; it pays where the pages' traffic or
 // its latency bound that kernel: large heads, long prompts.  Same fragment layouts and key order as there:
 // S^T = K Q^T and O^T = V^T P^T with 16x16x32 MFMAs, token index in `lane % 16`, softmax online in float,
 // probabilities rounded to bfloat16 for the second product.
