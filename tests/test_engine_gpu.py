@@ -163,6 +163,49 @@ def test_thousands_of_tokens_of_context(tmp_path, dtype):
     eng.cache.check_invariants()
 
 
+def test_long_prompts_with_large_heads_through_the_engine(tmp_path):
+    """28 query heads of 128 over 4 kv heads (the head shape of the 7B model, one narrow layer) and prompts long
+    enough that the launcher gives their portions to the prompt kernel whose waves share each block of keys: a
+    prompt of 2,300 tokens in one step beside a short one, then a portion of 700 tokens that starts inside a page
+    after 1,650 cached ones (too few tiles: the other kernel), then single tokens; also under a window of 1,000
+    keys in the upper layer.  Logits against the plain implementation."""
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import StepEntry
+    from tokenizer_amd.kernels import get_ops
+    ops = get_ops()
+    assert ops.prefill_shared == 0
+    assert ops.lib.ta_prefill_attention_shared_plan(144 + 2, 28, 4, 128, 2560) == 1      # the first step below
+    raw = dict(TINY["A"][0], num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+               intermediate_size=256, vocab_size=300, max_position_embeddings=4096, rope_theta=1000000.0,
+               use_sliding_window=True, sliding_window=1000, max_window_layers=1)
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 17, str(tmp_path / "heads128"), norm_spread=0.3)
+    cfg, tensors = plain.load_folder(folder)
+    a_ids, b_ids, c_ids = random_ids(300, 2310, 41), random_ids(300, 30, 42), random_ids(300, 2360, 43)
+    want = {"a": plain.all_logits(cfg, tensors, a_ids), "b": plain.all_logits(cfg, tensors, b_ids),
+            "c": plain.all_logits(cfg, tensors, c_ids)}
+    eng = engine_for(folder, "bfloat16", max_tokens=2368 + 64 + 2368, max_requests=3)
+    eng.pools.poison()
+    for rid in "abc":
+        eng.add_request(rid)
+    rows = [0, 15, 16, 1000, 1001, 1650, 2299]
+    logits = eng.step([StepEntry("a", a_ids[:2300], rows), StepEntry("b", b_ids[:25], [0, 24])]).float().cpu()
+    close(logits[:len(rows)], want["a"][rows], "bfloat16")
+    close(logits[len(rows):], want["b"][[0, 24]], "bfloat16")
+    logits = eng.step([StepEntry("c", c_ids[:1650], [1649])]).float().cpu()
+    close(logits, want["c"][[1649]], "bfloat16")
+    logits = eng.step([StepEntry("c", c_ids[1650:2350], [0, 699]), StepEntry("a", a_ids[2300:2301], [0])]).float().cpu()
+    close(logits[:2], want["c"][[1650, 2349]], "bfloat16")
+    close(logits[2:], want["a"][[2300]], "bfloat16")
+    for i in range(2301, 2310):
+        logits = eng.step([StepEntry("a", a_ids[i:i + 1], [0]), StepEntry("c", c_ids[i + 49:i + 50], [0])]).float().cpu()
+        close(logits[:1], want["a"][[i]], "bfloat16")
+        close(logits[1:], want["c"][[i + 49]], "bfloat16")
+    for rid in "abc":
+        eng.end_request(rid)
+    eng.cache.check_invariants()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", list(TINY))
 def test_first_tokens_of_a_sequence(model_folders, oracle, name, dtype):
