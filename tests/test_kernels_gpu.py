@@ -285,6 +285,39 @@ def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref,
     torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_shared_block_prompt_attention_on_random_batches(ops, seed, monkeypatch):
+    # Random head counts, page sizes, windows and batches of portions (whole prompts, portions after cached tokens,
+    # two-token portions, single tokens beside them), unwritten slots holding NaN: the kernel whose waves share
+    # their blocks, with one and two heads a wave, against one masked matrix product per request.
+    import random
+    rng = random.Random(seed)
+    d = rng.choice([64, 128])
+    n_kv = rng.choice([1, 2, 3])
+    n_q = n_kv * rng.choice([5, 6, 7, 8, 12])
+    page_size = rng.choice([16, 32, 48, 64])
+    window = rng.choice([None, None, rng.randint(1, 40), rng.randint(41, 900)])
+    lengths, q_lens = [], []
+    for _ in range(rng.randint(1, 5)):
+        length = rng.choice([rng.randint(2, 70), rng.randint(71, 1500)])
+        lengths.append(length)
+        q_lens.append(rng.choice([length, rng.randint(1, length), min(length, 2), 1]))
+    if all(q == 1 for q in q_lens):
+        q_lens[0] = min(lengths[0], 17)
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=100 + seed)
+    scale = 1.0 / math.sqrt(d)
+    want = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
+    monkeypatch.setattr(ops, "prefill_shared", 1)
+    for heads in (1, 2):
+        monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
+        out = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+        ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                            max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+        torch.testing.assert_close(out.float(), want, **attention_tol(torch.bfloat16, True),
+                                   msg=lambda m: f"{m}\n{(n_q, n_kv, d, page_size, window, lengths, q_lens, heads)}")
+
+
 def test_where_the_workgroup_shared_kernel_is_planned(ops):
     plan = ops.lib.ta_prefill_attention_shared_plan
     # (tiles, query heads, kv heads, head size, reach) -> heads a wave, 0 = the per-wave kernel
