@@ -36,6 +36,12 @@ struct Staged {
   __device__ static constexpr int swizzle(int key) { return (key & 3) | ((key >> 1) & 4); }
 };
 
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 __device__ __forceinline__ bf16x8 sh_zero8() {
   bf16x8 z;
 #pragma unroll
@@ -137,7 +143,7 @@ struct Carrier {
 template <int D, int HG, bool FULL>
 __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, int g, int my_pos, int my_lo, int lo, int hi,
                                              float c, const bf16x8 (&qf)[HG][D / 32], floatx4 (&acc)[HG][D / 16],
-                                             float (&m)[HG], float (&l)[HG]) {
+                                             float (&m)[HG], floatx4 (&l)[HG]) {
   constexpr int KS = D / 32;
   constexpr int DB = D / 16;
   float s[HG][16];
@@ -170,8 +176,10 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     const float (&sh)[16] = s[h];
-    float mx = fmaxf(fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3])), fmaxf(fmaxf(sh[4], sh[5]), fmaxf(sh[6], sh[7])));
-    mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(sh[8], sh[9]), fmaxf(sh[10], sh[11])), fmaxf(fmaxf(sh[12], sh[13]), fmaxf(sh[14], sh[15]))));
+    // Sixteen scores, eight instructions: written out, because fmaxf first rewrites every input that might be a
+    // signalling NaN (one more instruction per score) before the compiler joins pairs of them into v_max3_f32.
+    float mx = max3(max3(max3(sh[0], sh[1], sh[2]), max3(sh[3], sh[4], sh[5]), max3(sh[6], sh[7], sh[8])),
+                    max3(sh[9], sh[10], sh[11]), max3(max3(sh[12], sh[13], sh[14]), sh[15], sh[15]));
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(m[h], mx);
@@ -179,22 +187,28 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
     const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
     if (__any(m_new > m[h])) {                          // rescale only when some token's maximum moved
       const float corr = __builtin_amdgcn_exp2f(m[h] * c - mc);   // m = -inf gives 0
-      l[h] *= corr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) l[h][r] *= corr;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[h][db][r] *= corr;
       m[h] = m_new;
     }
-    float psum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float p = __builtin_amdgcn_exp2f(fmaf(sh[i], c, -mc));   // masked keys: exp2(-inf) = 0
-      psum += p;
-      pf[h][i >> 3][i & 7] = (__bf16)p;
-    }
-    l[h] += psum;
+    for (int i = 0; i < 16; ++i)
+      pf[h][i >> 3][i & 7] = (__bf16)__builtin_amdgcn_exp2f(fmaf(sh[i], c, -mc));   // masked keys: exp2(-inf) = 0
   }
+  // The probabilities' sums come from the matrix cores as well, as one more row block of V^T that holds ones:
+  // every lane then has its token's sum over all 64 keys (of the rounded probabilities, the very weights of the
+  // second product), where sixteen additions a head and two exchanges between lanes at the end stood.
+  bf16x8 ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int h = 0; h < HG; ++h) l[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[h][u], l[h], 0, 0, 0);
 #pragma unroll
   for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -270,12 +284,12 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
       if (h < heads_here)
         qf[h][ks] = *reinterpret_cast<const bf16x8*>(q + (size_t)my_row * q_stride + (size_t)(head0 + h) * D + ks * 32 + 8 * g);
     }
-  floatx4 acc[HG][DB];
-  float m[HG], l[HG];
+  floatx4 acc[HG][DB], l[HG];                              // l: the sum of a token's probabilities, four times over
+  float m[HG];
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     m[h] = -INFINITY;
-    l[h] = 0.f;
+    l[h] = (floatx4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int db = 0; db < DB; ++db) acc[h][db] = (floatx4){0.f, 0.f, 0.f, 0.f};
   }
@@ -315,11 +329,8 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     if (h >= heads_here) break;
-    float total = l[h];
-    total += __shfl_xor(total, 16, WAVE);
-    total += __shfl_xor(total, 32, WAVE);
     if (col >= n_valid) continue;
-    const float inv = 1.0f / total;
+    const float inv = 1.0f / l[h][0];
     bf16_t* dst = out + (size_t)my_row * n_q * D + (size_t)(head0 + h) * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
