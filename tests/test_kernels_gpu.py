@@ -309,7 +309,7 @@ def test_shared_block_prompt_attention_on_random_batches(ops, seed, monkeypatch)
     scale = 1.0 / math.sqrt(d)
     want = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
     monkeypatch.setattr(ops, "prefill_shared", 1)
-    for heads in (1, 2):
+    for heads in (1, 2, 11, 12):
         monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
         out = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
         ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,

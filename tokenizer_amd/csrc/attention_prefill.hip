@@ -342,7 +342,7 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
   if (shared >= 0 && waves == 0) {
     int heads = ta_prefill_attention_shared_plan(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window));
-    if (shared > 0) heads = (heads_per_wave == 1 || heads_per_wave == 2) ? heads_per_wave : heads ? heads : 2;
+    if (shared > 0) heads = (heads_per_wave % 10 == 1 || heads_per_wave % 10 == 2) ? heads_per_wave : heads ? heads : 2;
     if (heads) {
       const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
                                                           first_position, block_table, table_stride, n_q, n_kv, d,

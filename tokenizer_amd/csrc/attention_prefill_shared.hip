@@ -36,12 +36,6 @@ struct Staged {
   __device__ static constexpr int swizzle(int key) { return (key & 3) | ((key >> 1) & 4); }
 };
 
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-
 __device__ __forceinline__ bf16x8 sh_zero8() {
   bf16x8 z;
 #pragma unroll
@@ -68,21 +62,22 @@ struct Carrier {
   uint32_t k_from[S::K_LOADS];                              // byte offsets of the lane's pieces inside the run's part of its page
   uint32_t v_from;
   int at_page, at_slot;                                     // where the run of the next block to look up lies: index into the block table, slot in the page
-  int step_pages, step_slots;                               // 64 keys on
+  int step_pages, step_slots;                               // from one of the wave's blocks to the next
   int page, slot;                                           // of the run of the block to fetch next
   int page_size;
   uint32_t page_elements, first_element;                    // elements of a page (all kv heads); where this kv head's begin
 
-  // first_key: the first key of the first block.
-  __device__ __forceinline__ void plan(int wave, int lane, const SharedTile& tile, int first_key) {
-    run = wave;
+  // run: which of a block's runs; first_key: the first key of the wave's first block; stride: keys from one of
+  // its blocks to the next (a multiple of 64).
+  __device__ __forceinline__ void plan(int which_run, int lane, const SharedTile& tile, int first_key, int stride) {
+    run = which_run;
     page_size = tile.page_size;
     page_elements = (uint32_t)tile.n_kv * page_size * D;
     first_element = (uint32_t)tile.kvh * page_size * D;
     at_page = (first_key + 16 * run) / page_size;
     at_slot = (first_key + 16 * run) % page_size;
-    step_pages = 64 / page_size;
-    step_slots = 64 % page_size;
+    step_pages = stride / page_size;
+    step_slots = stride % page_size;
 #pragma unroll
     for (int j = 0; j < S::K_LOADS; ++j) {
       const int key = S::KEYS_A_LOAD * j + lane / S::PIECES;             // within the run; the run starts at a multiple of 16
@@ -176,10 +171,11 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     const float (&sh)[16] = s[h];
-    // Sixteen scores, eight instructions: written out, because fmaxf first rewrites every input that might be a
-    // signalling NaN (one more instruction per score) before the compiler joins pairs of them into v_max3_f32.
-    float mx = max3(max3(max3(sh[0], sh[1], sh[2]), max3(sh[3], sh[4], sh[5]), max3(sh[6], sh[7], sh[8])),
-                    max3(sh[9], sh[10], sh[11]), max3(max3(sh[12], sh[13], sh[14]), sh[15], sh[15]));
+    // (Through fmaxf, which the compiler knows: the scores come straight from matrix instructions, whose results
+    // a vector instruction may only read after wait states that the compiler counts; it cannot count them for an
+    // instruction written in inline assembly, and a v_max3_f32 written that way read scores too early now and then.)
+    float mx = fmaxf(fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3])), fmaxf(fmaxf(sh[4], sh[5]), fmaxf(sh[6], sh[7])));
+    mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(sh[8], sh[9]), fmaxf(sh[10], sh[11])), fmaxf(fmaxf(sh[12], sh[13]), fmaxf(sh[14], sh[15]))));
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(m[h], mx);
@@ -228,9 +224,13 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
     }
 }
 
-// Arguments as in prefill_attention_kernel.  Dynamic LDS: two blocks (2 * Staged<D>::BYTES).
-template <int D, int HG>
-__global__ void __launch_bounds__(SHARED_WAVES * WAVE, 1)
+// Arguments as in prefill_attention_kernel.  Dynamic LDS: two blocks for each of the KG groups of four waves
+// (2 * KG * Staged<D>::BYTES).
+// KG = 2: two groups of four waves, each with the same heads, take the blocks in turn (group i the blocks i,
+// i + 2, ...) and merge their softmax states through LDS at the end: half as many turns for a long walk, for
+// launches that cannot fill the device with workgroups.
+template <int D, int HG, int KG>
+__global__ void __launch_bounds__(SHARED_WAVES * KG * WAVE, 1)
 prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                 const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                                 const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
@@ -239,8 +239,10 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   constexpr int KS = D / 32;
   constexpr int DB = D / 16;
   constexpr int NW = SHARED_WAVES;
+  constexpr int STRIDE = 64 * KG;                          // keys a turn of the whole workgroup covers
   extern __shared__ __attribute__((aligned(16))) char staged[];
   const int lane = threadIdx.x & 63, wave = wave_index();
+  const int head_wave = wave % NW, key_group = wave / NW;
   const int col = lane & 15, g = lane >> 4;
   const int group = n_q / n_kv;
   const int head_blocks = (group + HG * NW - 1) / (HG * NW);
@@ -248,7 +250,7 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   const int per_tile = n_kv * head_blocks;
   const int which = blockIdx.x % per_tile;
   const int kvh = which / head_blocks, hb = which % head_blocks;
-  const int first_head = hb * HG * NW + wave * HG;            // among the heads of the kv head
+  const int first_head = hb * HG * NW + head_wave * HG;       // among the heads of the kv head
   const int heads_here = max(0, min(HG, group - first_head));  // a wave past the last head only brings blocks
   const int head0 = kvh * group + first_head;
   const int tile_index = n_tiles - 1 - blockIdx.x / per_tile;
@@ -294,38 +296,85 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
     for (int db = 0; db < DB; ++db) acc[h][db] = (floatx4){0.f, 0.f, 0.f, 0.f};
   }
 
-  // Blocks come in three runs (the window's edge, those every token sees whole, the diagonal), each a loop of
-  // its own over one variant of the block, so that the accumulators stay in the same registers within a loop.
-  // A turn asks for the next block into the buffer that the turn before read, works on the current one, waits
-  // for what it asked for, and meets the other waves: after the barrier every wave's part of the next block
-  // has landed, and nobody reads the current one any more.
-  int kb = (lo / 64) * 64;
+  // A turn of the workgroup covers KG blocks, one for each group of waves.  Turns come in three runs (the
+  // window's edge, those whose blocks every token sees whole, the diagonal), each a loop of its own over one
+  // variant of the block, so that the accumulators stay in the same registers within a loop.  In a turn a wave
+  // asks for its group's next block into the buffer that the turn before read, works on the current one, waits
+  // for what it asked for, and meets the other waves: after the barrier every wave's part of the next blocks has
+  // landed, and nobody reads the current ones any more.  A group whose block of a turn lies past the last key
+  // leaves it out.
+  int kb = (lo / 64) * 64;                                 // the turn's first key
   int cur = 0;
+  char* buffers = staged + key_group * 2 * Staged<D>::BYTES;
+  const int ahead = 64 * key_group;                        // the group's block within a turn
   Carrier<D> carrier;
-  carrier.plan(wave, lane, tile, kb);
-  const auto whole = [&](int block) { return block >= lo_all && block + 63 <= p0; };
-  carrier.look_up(tile, kb, whole(kb));
-  carrier.fetch(tile, staged);
-  if (kb + 64 <= hi) carrier.look_up(tile, kb + 64, whole(kb + 64));
+  carrier.plan(head_wave, lane, tile, kb + ahead, STRIDE);
+  const auto whole = [&](int turn) { return turn >= lo_all && turn + STRIDE - 1 <= p0; };
+  carrier.look_up(tile, kb + ahead, whole(kb));
+  if (kb + ahead <= hi) carrier.fetch(tile, buffers);
+  if (kb + STRIDE + ahead <= hi) carrier.look_up(tile, kb + STRIDE + ahead, whole(kb + STRIDE));
   carrier.landed();
   __syncthreads();
 #define TURN(FULL)                                                                                            \
   {                                                                                                           \
-    const int next = kb + 64;                                                                                 \
-    if (next <= hi) carrier.fetch(tile, staged + (cur ^ 1) * Staged<D>::BYTES);                               \
-    if (next + 64 <= hi) carrier.look_up(tile, next + 64, whole(next + 64));                                  \
-    if (heads_here > 0)                                                                                       \
-      shared_block<D, HG, FULL>(staged + cur * Staged<D>::BYTES, kb, col, g, my_pos, my_lo, lo, hi, scale_log2, \
-                                qf, acc, m, l);                                                               \
+    const int next = kb + STRIDE;                                                                             \
+    if (next + ahead <= hi) carrier.fetch(tile, buffers + (cur ^ 1) * Staged<D>::BYTES);                      \
+    if (next + STRIDE + ahead <= hi) carrier.look_up(tile, next + STRIDE + ahead, whole(next + STRIDE));      \
+    if (heads_here > 0 && (FULL || kb + ahead <= hi))                                                         \
+      shared_block<D, HG, FULL>(buffers + cur * Staged<D>::BYTES, kb + ahead, col, g, my_pos, my_lo, lo, hi,  \
+                                scale_log2, qf, acc, m, l);                                                   \
     carrier.landed();                                                                                         \
     __syncthreads();                                                                                          \
     cur ^= 1;                                                                                                 \
   }
-  for (; kb <= hi && kb < lo_all; kb += 64) TURN(false)
-  for (; kb + 63 <= p0; kb += 64) TURN(true)
-  for (; kb <= hi; kb += 64) TURN(false)
+  for (; kb <= hi && kb < lo_all; kb += STRIDE) TURN(false)
+  for (; kb + STRIDE - 1 <= p0; kb += STRIDE) TURN(true)
+  for (; kb <= hi; kb += STRIDE) TURN(false)
 #undef TURN
 
+  if (KG > 1) {
+    // The later groups hand their state to the first (the last turn ended with a barrier: the buffers are free):
+    // maximum, sum and the output accumulators of each head.
+    float* handed = reinterpret_cast<float*>(staged);      // [KG - 1][NW][HG][DB * 4 + 2][WAVE]
+    const auto at = [&](int from_group, int h, int item) {
+      return handed + ((((from_group - 1) * NW + head_wave) * HG + h) * (DB * 4 + 2) + item) * WAVE + lane;
+    };
+    if (key_group > 0) {
+#pragma unroll
+      for (int h = 0; h < HG; ++h) {
+        *at(key_group, h, DB * 4) = m[h];
+        *at(key_group, h, DB * 4 + 1) = l[h][0];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) *at(key_group, h, db * 4 + r) = acc[h][db][r];
+      }
+    }
+    __syncthreads();
+    if (key_group > 0) return;
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+      float m_all = m[h];
+#pragma unroll
+      for (int k = 1; k < KG; ++k) m_all = fmaxf(m_all, *at(k, h, DB * 4));
+      const float mc = (m_all == -INFINITY) ? 0.f : m_all * scale_log2;
+      const float f0 = __builtin_amdgcn_exp2f(m[h] * scale_log2 - mc);       // a group without keys: exp2(-inf) = 0
+      l[h][0] *= f0;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[h][db][r] *= f0;
+#pragma unroll
+      for (int k = 1; k < KG; ++k) {
+        const float f = __builtin_amdgcn_exp2f(*at(k, h, DB * 4) * scale_log2 - mc);
+        l[h][0] += f * *at(k, h, DB * 4 + 1);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[h][db][r] += f * *at(k, h, db * 4 + r);
+      }
+    }
+  }
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     if (h >= heads_here) break;
@@ -342,7 +391,7 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   }
 }
 
-template <int D, int HG>
+template <int D, int HG, int KG>
 static int launch_shared(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
                          const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
                          const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
@@ -350,14 +399,15 @@ static int launch_shared(const void* q, int q_stride, void* out, const void* k_p
   const int group = n_q / n_kv;
   const long workgroups = (long)n_tiles * n_kv * ((group + HG * SHARED_WAVES - 1) / (HG * SHARED_WAVES));
   if (workgroups > 0x7fffffffL) return -1;
-  constexpr int lds = 2 * Staged<D>::BYTES;
-  static_assert(lds <= 160 * 1024, "two blocks must fit a compute unit's LDS");
+  constexpr int lds = 2 * KG * Staged<D>::BYTES;
+  static_assert(lds <= 160 * 1024, "the blocks must fit a compute unit's LDS");
+  static_assert((KG - 1) * SHARED_WAVES * HG * (D / 4 + 2) * WAVE * 4 <= lds, "the groups' states are handed over in the blocks' place");
   if (lds > 48 * 1024) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_shared_kernel<D, HG>),
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_shared_kernel<D, HG, KG>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (err != hipSuccess) return (int)err;
   }
-  prefill_attention_shared_kernel<D, HG><<<(unsigned)workgroups, SHARED_WAVES * WAVE, lds, stream>>>(
+  prefill_attention_shared_kernel<D, HG, KG><<<(unsigned)workgroups, SHARED_WAVES * KG * WAVE, lds, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
       n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
       window, scale * 1.4426950408889634f);
@@ -394,10 +444,13 @@ extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, voi
                                                 int page_size, int window, float scale, int heads_per_wave,
                                                 hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  const int key_groups = heads_per_wave > 10 ? 2 : 1;
+  heads_per_wave %= 10;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || heads_per_wave < 1 || heads_per_wave > 2) return -1;
-#define GO(DD, HG) return launch_shared<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
+#define GO(DD, HG, KG) return launch_shared<DD, HG, KG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
-#define SIZE(DD) case DD: if (heads_per_wave == 1) GO(DD, 1) GO(DD, 2)
+#define SIZE(DD) case DD: if (key_groups == 2) { if (heads_per_wave == 1) GO(DD, 1, 2) GO(DD, 2, 2) } \
+    if (heads_per_wave == 1) GO(DD, 1, 1) GO(DD, 2, 1)
   switch (d) {
     SIZE(64) SIZE(128)
     default: return -2;
