@@ -167,7 +167,7 @@ def test_long_prompts_with_large_heads_through_the_engine(tmp_path):
     """28 query heads of 128 over 4 kv heads (the head shape of the 7B model, one narrow layer) and prompts long
     enough that the launcher gives their portions to the prompt kernel whose waves share each block of keys: a
     prompt of 2,300 tokens in one step beside a short one, then a portion of 700 tokens that starts inside a page
-    after 1,650 cached ones (too few tiles: the other kernel), then single tokens; also under a window of 1,000
+    after 1,650 cached ones (fewer tiles: one head a wave), then single tokens; also under a window of 1,000
     keys in the upper layer.  Logits against the plain implementation."""
     import tokenizer_amd as ta
     from tokenizer_amd.config import Qwen2Config
@@ -175,7 +175,7 @@ def test_long_prompts_with_large_heads_through_the_engine(tmp_path):
     from tokenizer_amd.kernels import get_ops
     ops = get_ops()
     assert ops.prefill_shared == 0
-    assert ops.lib.ta_prefill_attention_shared_plan(144 + 2, 28, 4, 128, 2560) == 1      # the first step below
+    assert ops.lib.ta_prefill_attention_shared_plan(144 + 2, 28, 4, 128, 2560) == 12     # the first step below: two heads a wave, two key groups
     raw = dict(TINY["A"][0], num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
                intermediate_size=256, vocab_size=300, max_position_embeddings=4096, rope_theta=1000000.0,
                use_sliding_window=True, sliding_window=1000, max_window_layers=1)

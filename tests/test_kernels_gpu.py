@@ -254,15 +254,17 @@ def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, windo
     torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
 
 
-@pytest.mark.parametrize("geometry,lengths,q_lens,heads", [((14, 2, 64, 16), [4500, 333], [4400, 50], 1),
-                                                           ((28, 2, 64, 16), [2300, 40], [2200, 33], 1),
-                                                           ((28, 4, 128, 16), [2300, 40], [2200, 33], 1),
-                                                           ((28, 4, 128, 16), [4300, 40], [4200, 33], 2)])
+@pytest.mark.parametrize("geometry,lengths,q_lens,shape", [((14, 2, 64, 16), [4500, 333], [4400, 50], 11),
+                                                           ((28, 2, 64, 16), [2300, 40], [2200, 33], 11),
+                                                           ((28, 4, 128, 16), [2300, 40], [2200, 33], 12),
+                                                           ((28, 4, 128, 16), [4300, 40], [4200, 33], 2),
+                                                           ((14, 2, 64, 16), [1100, 40], [1000, 33], 11)])
 @pytest.mark.parametrize("window", [None, 1000])
-def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref, geometry, lengths, q_lens, heads, window):
-    # Seven (or twice seven) query heads per kv head and hundreds of tiles: the launcher's own choice is the kernel
-    # whose waves share their blocks of keys, with one head a wave or two by the number of workgroups.  Portions
-    # that start and end inside pages and tiles, beside a short one, with and without a window.
+def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref, geometry, lengths, q_lens, shape, window):
+    # Seven (or twice seven) query heads per kv head and dozens to hundreds of tiles: the launcher's own choice is
+    # the kernel whose waves share their blocks of keys, with one head a wave or two and one or two key groups by
+    # the number of workgroups (shape = heads a wave + 10 for two key groups).  Portions that start and end inside
+    # pages and tiles, beside a short one, with and without a window.
     n_q, n_kv, d, page_size = geometry
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=23)
@@ -270,7 +272,7 @@ def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref,
     assert ops.prefill_shared == 0 and ops.prefill_waves == 0 and ops.prefill_heads_per_wave == 0
     plan = ops.lib.ta_prefill_attention_shared_plan
     reach = -(-max(lengths) // 512) * 512 if window is None else window + 16
-    assert plan(batch.q_tiles.shape[0], n_q, n_kv, d, reach) == heads
+    assert plan(batch.q_tiles.shape[0], n_q, n_kv, d, reach) == shape
     scale = 1.0 / math.sqrt(d)
     out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
     ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
@@ -320,49 +322,15 @@ def test_shared_block_prompt_attention_on_random_batches(ops, seed, monkeypatch)
 
 def test_where_the_workgroup_shared_kernel_is_planned(ops):
     plan = ops.lib.ta_prefill_attention_shared_plan
-    # (tiles, query heads, kv heads, head size, reach) -> heads a wave, 0 = the per-wave kernel
-    assert plan(128, 14, 2, 64, 2048) == 0          # 2,048 tokens at 0.5B sizes: 512 workgroups even at one head a wave
-    assert plan(192, 14, 2, 64, 3072) == 1 and plan(256, 14, 2, 64, 4096) == 1 and plan(512, 14, 2, 64, 8192) == 2
-    assert plan(128, 28, 4, 128, 2048) == 1 and plan(256, 28, 4, 128, 4096) == 2
-    assert plan(64, 28, 4, 128, 2048) == 0 and plan(64, 28, 4, 128, 4096) == 2 and plan(63, 28, 4, 128, 4096) == 0
-    assert plan(128, 12, 2, 128, 2048) == 0 and plan(128, 12, 2, 128, 10240) == 2
+    # (tiles, query heads, kv heads, head size, reach) -> heads a wave + 10 for two key groups, 0 = the per-wave kernel
+    assert plan(32, 14, 2, 64, 512) == 0 and plan(64, 14, 2, 64, 1024) == 11       # 512 and 1,024 tokens at 0.5B sizes
+    assert plan(128, 14, 2, 64, 2048) == 11 and plan(256, 14, 2, 64, 4096) == 11 and plan(512, 14, 2, 64, 8192) == 2
+    assert plan(32, 28, 4, 128, 512) == 11 and plan(64, 28, 4, 128, 1024) == 11 and plan(64, 28, 4, 128, 8192) == 12
+    assert plan(128, 28, 4, 128, 2048) == 12 and plan(256, 28, 4, 128, 4096) == 2
+    assert plan(31, 28, 4, 128, 8192) == 0
+    assert plan(128, 12, 2, 128, 2048) == 11 and plan(128, 12, 2, 128, 10240) == 12
     assert plan(4096, 16, 4, 128, 8192) == 0        # four heads per kv head
     assert plan(4096, 28, 4, 96, 8192) == 0         # no instance
-
-
-@pytest.mark.parametrize("geometry", [(28, 4, 128, 16), (12, 2, 128, 32), (5, 1, 64, 48), (16, 2, 128, 16),
-                                      (24, 2, 128, 64), (3, 1, 128, 16), (14, 2, 64, 16)])
-@pytest.mark.parametrize("window", [None, 100])
-@pytest.mark.parametrize("heads", [1, 2])
-def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, geometry, window, heads, monkeypatch):
-    # The kernel whose four waves take one block of keys from LDS for up to eight query heads of a kv head: five,
-    # six, seven and eight heads (a wave with one head, a wave without any), twelve (two workgroups a tile) and
-    # three; portions that start in the middle of a page, end in the middle of a tile, lie under a window whose
-    # first pages hold nothing any more, and unwritten slots that hold NaN.  With two heads a wave and with one.
-    monkeypatch.setattr(ops, "prefill_shared", 1)
-    monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
-    n_q, n_kv, d, page_size = geometry
-    lengths, q_lens = [700, 333, 40, 16, 1000], [700, 50, 33, 16, 2]
-    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
-        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=29)
-    scale = 1.0 / math.sqrt(d)
-    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
-    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
-                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
-    out_b = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
-    torch.testing.assert_close(out_a.float(), out_b, **attention_tol(torch.bfloat16, True))
-    rows = torch.tensor([0, 17, 699, 700, 749, 750, qkv.shape[0] - 1]).cuda()
-    out_c = torch.empty((len(rows), n_q * d), dtype=torch.bfloat16).cuda()
-    ref.paged_attention(qkv[rows], out_c, k_pages, v_pages, positions[rows], entry_of_token[rows], table, n_q, n_kv, d,
-                        window, scale)
-    torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
-    # The other prompt kernel rounds at other places; both stay within the same distance of the float32 result.
-    monkeypatch.setattr(ops, "prefill_shared", -1)
-    monkeypatch.setattr(ops, "prefill_heads_per_wave", 0)
-    out_d = torch.full_like(out_a, float("nan"))
-    ops.paged_attention(qkv, out_d, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
-                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
-    torch.testing.assert_close(out_d.float(), out_b, **attention_tol(torch.bfloat16, True))
 
 
 @pytest.mark.parametrize("target", [1024, 16])

@@ -414,39 +414,44 @@ static int launch_shared(const void* q, int q_stride, void* out, const void* k_p
   return LAUNCH_STATUS();
 }
 
-// Whether the workgroup-shared kernel is the faster one, and with how many heads a wave: 0 = no, else 1 or 2.
-// Five to eight query heads per kv head (or more) fill its four waves at two heads a wave, and the launch must
-// fill the device although a workgroup walks all its keys alone: two or three workgroups for every compute unit,
-// or one where the walk is long.  With one head a wave there are twice the workgroups, each reading its blocks
-// for half the heads: the better cut while two heads a wave give fewer than 1,024 workgroups.
+// Whether the workgroup-shared kernel is the faster one, and in which shape: 0 = no, else heads a wave (1 or 2)
+// + 10 if two key groups share a workgroup.  Five to eight query heads per kv head (or more) fill its four waves
+// at two heads a wave.  A workgroup walks all its keys alone, so the launch must fill the device some other way:
+// with 1,024 workgroups and more, two heads a wave; below that two key groups halve the walk, and one head a
+// wave doubles the workgroups (each reading its blocks for half the heads); below 128 workgroups the per-wave
+// kernel, whose waves split the keys of a tile, is the faster one.
 // reach: how far back the farthest-seeing token looks, as the launcher plans it.
-// (Measured on 256 compute units, 7 heads per kv head, against the per-wave kernel.  Two heads a wave, head size
-// 128: 0.75x with 128 workgroups; with 256: 0.84x at a reach of 2,048, 1.1-1.35x at 4,096, 1.4x at 8,192; with 512
-// and more 1.5x at 2,048 tokens, 2.1x at 8,192, 2.2x at 32,768; 1.5x with 5 or 6 heads per kv head, where a wave
-// only brings blocks.  Head size 64: 0.76-0.93x below 512 workgroups, 1.25x at 8,192 tokens, 1.35x at 32,768.
-// One head a wave against two: head size 64 1.26x at 2,048 tokens (where it is level with the per-wave kernel),
-// 1.27x at 3,072, 1.23x at 4,096, 0.95x at 8,192; head size 128 1.05x at 2,048, 0.8x at 8,192.)
+// (Measured on 256 compute units against the per-wave kernel, times in us as per-wave | 1 head | 2 heads |
+// 1 head, 2 groups | 2 heads, 2 groups.  14 / 2 heads of 64: 1,024 tokens 14.3 | 17.4 | 23.6 | 13.6 | 18.6;
+// 2,048 tokens 31.5 | 31.1 | 42.1 | 24.9 | 31.6; 4,096 tokens 87 | 63 | 80 | 62 | 63; 8,192 tokens 298 | 201 |
+// 179 | 206 | 215; 2,048 tokens after 8,192 cached ones 174 | 138 | 178 | 121 | 126; 512 after 8,192: 59 | 100 | 151
+// | 69 | 105.  28 / 4 heads of 128: 512 tokens 18.5 | 16.4 | 20.0 | 14.0 | 18.3; 2,048 tokens 103 | 66 | 66 | 79 |
+// 58; 8,192 tokens 1,199 | 750 | 561 | 899 | 643; 2,048 after 8,192: 656 | 418 | 321 | 481 | 339.  12 / 2 heads of
+// 128: 2,048 tokens 44.4 | 48.3 | 56.0 | 40.5 | 44.1; 2,048 after 8,192: 316 | 221 | 250 | 256 | 184.)
 extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, int d, int reach) {
   if (d != 64 && d != 128) return 0;
   const int group = n_q / n_kv;
   if (group < 5) return 0;
-  const long two = (long)n_tiles * n_kv * ((group + 7) / 8), one = (long)n_tiles * n_kv * ((group + 3) / 4);
-  if (one < 768 && !(two >= 256 && reach >= 4096)) return 0;
-  return (two >= 1024 || one < 768) ? 2 : 1;
+  const long two = (long)n_tiles * n_kv * ((group + 7) / 8);      // workgroups at two heads a wave
+  if (two < 128) return 0;
+  if (two >= 1024) return 2;
+  if (d == 64) return 11;
+  if (two >= 512) return 12;
+  if (two >= 256) return reach >= 4096 ? 12 : 11;
+  return 11;
 }
 
 // Returns -2 for a head size without an instance (the caller then uses the other kernel).
-// heads_per_wave: 1 or 2.
+// shape: heads a wave (1 or 2), + 10 for two key groups in a workgroup.
 extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                                 const void* vt_pages, const void* tiles, int n_tiles,
                                                 const void* cu_q, const void* first_position,
                                                 const void* block_table, int table_stride, int n_q, int n_kv, int d,
-                                                int page_size, int window, float scale, int heads_per_wave,
+                                                int page_size, int window, float scale, int shape,
                                                 hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  const int key_groups = heads_per_wave > 10 ? 2 : 1;
-  heads_per_wave %= 10;
-  if (n_kv <= 0 || n_q % n_kv || page_size % 16 || heads_per_wave < 1 || heads_per_wave > 2) return -1;
+  const int heads_per_wave = shape % 10, key_groups = shape / 10 + 1;
+  if (n_kv <= 0 || n_q % n_kv || page_size % 16 || heads_per_wave < 1 || heads_per_wave > 2 || key_groups > 2) return -1;
 #define GO(DD, HG, KG) return launch_shared<DD, HG, KG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
 #define SIZE(DD) case DD: if (key_groups == 2) { if (heads_per_wave == 1) GO(DD, 1, 2) GO(DD, 2, 2) } \

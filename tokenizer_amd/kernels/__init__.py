@@ -277,7 +277,8 @@ class Ops:
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
     use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
     prefill_waves = 0          # waves that share a tile's keys in the prompt kernel: 0 lets the launcher choose
-    prefill_heads_per_wave = 0    # heads a wave (1 or 2) of the workgroup-shared prompt kernel when it is asked for; 0: its choice
+    prefill_heads_per_wave = 0    # shape of the workgroup-shared prompt kernel when it is asked for: heads a wave (1 or 2),
+    #                               + 10 for two key groups in a workgroup; 0: its own choice
     prefill_shared = 0            # the prompt kernel whose waves share a block of keys through LDS: 1 = wherever it has
     #                               an instance, -1 = never, 0 = where the launcher expects it to be the faster one
     target_workgroups = 1024      # what the split of the key range aims at
