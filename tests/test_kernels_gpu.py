@@ -291,7 +291,7 @@ def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref,
 def test_shared_block_prompt_attention_on_random_batches(ops, seed, monkeypatch):
     # Random head counts, page sizes, windows and batches of portions (whole prompts, portions after cached tokens,
     # two-token portions, single tokens beside them), unwritten slots holding NaN: the kernel whose waves share
-    # their blocks, with one and two heads a wave, against one masked matrix product per request.
+    # their blocks, in all its four shapes, against one masked matrix product per request.
     import random
     rng = random.Random(seed)
     d = rng.choice([64, 128])
@@ -331,6 +331,42 @@ def test_where_the_workgroup_shared_kernel_is_planned(ops):
     assert plan(128, 12, 2, 128, 2048) == 11 and plan(128, 12, 2, 128, 10240) == 12
     assert plan(4096, 16, 4, 128, 8192) == 0        # four heads per kv head
     assert plan(4096, 28, 4, 96, 8192) == 0         # no instance
+
+
+@pytest.mark.parametrize("geometry", [(28, 4, 128, 16), (12, 2, 128, 32), (5, 1, 64, 48), (16, 2, 128, 16),
+                                      (24, 2, 128, 64), (3, 1, 128, 16), (14, 2, 64, 16)])
+@pytest.mark.parametrize("window", [None, 100])
+@pytest.mark.parametrize("heads", [1, 2, 11, 12])
+def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, geometry, window, heads, monkeypatch):
+    # The kernel whose four waves take one block of keys from LDS for up to eight query heads of a kv head: five,
+    # six, seven and eight heads (a wave with one head, a wave without any), twelve (two workgroups a tile) and
+    # three; portions that start in the middle of a page, end in the middle of a tile, lie under a window whose
+    # first pages hold nothing any more, and unwritten slots that hold NaN.  With two heads a wave and with one, with
+    one group of waves and with two that take the blocks in turn (shape = heads a wave + 10 for two key groups).
+    monkeypatch.setattr(ops, "prefill_shared", 1)
+    monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
+    n_q, n_kv, d, page_size = geometry
+    lengths, q_lens = [700, 333, 40, 16, 1000], [700, 50, 33, 16, 2]
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=29)
+    scale = 1.0 / math.sqrt(d)
+    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    out_b = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
+    torch.testing.assert_close(out_a.float(), out_b, **attention_tol(torch.bfloat16, True))
+    rows = torch.tensor([0, 17, 699, 700, 749, 750, qkv.shape[0] - 1]).cuda()
+    out_c = torch.empty((len(rows), n_q * d), dtype=torch.bfloat16).cuda()
+    ref.paged_attention(qkv[rows], out_c, k_pages, v_pages, positions[rows], entry_of_token[rows], table, n_q, n_kv, d,
+                        window, scale)
+    torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
+    # The other prompt kernel rounds at other places; both stay within the same distance of the float32 result.
+    monkeypatch.setattr(ops, "prefill_shared", -1)
+    monkeypatch.setattr(ops, "prefill_heads_per_wave", 0)
+    out_d = torch.full_like(out_a, float("nan"))
+    ops.paged_attention(qkv, out_d, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    torch.testing.assert_close(out_d.float(), out_b, **attention_tol(torch.bfloat16, True))
 
 
 @pytest.mark.parametrize("target", [1024, 16])
