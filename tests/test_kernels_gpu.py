@@ -341,8 +341,8 @@ def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, 
     # The kernel whose four waves take one block of keys from LDS for up to eight query heads of a kv head: five,
     # six, seven and eight heads (a wave with one head, a wave without any), twelve (two workgroups a tile) and
     # three; portions that start in the middle of a page, end in the middle of a tile, lie under a window whose
-    # first pages hold nothing any more, and unwritten slots that hold NaN.  With two heads a wave and with one, with
-    one group of waves and with two that take the blocks in turn (shape = heads a wave + 10 for two key groups).
+    # first pages hold nothing any more, and unwritten slots that hold NaN.  With two heads a wave and with one,
+    # with one group of waves and with two that take the blocks in turn (shape = heads a wave + 10 for two groups).
     monkeypatch.setattr(ops, "prefill_shared", 1)
     monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
     n_q, n_kv, d, page_size = geometry
