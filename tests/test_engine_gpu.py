@@ -163,23 +163,25 @@ def test_thousands_of_tokens_of_context(tmp_path, dtype):
     eng.cache.check_invariants()
 
 
-def test_long_prompts_with_large_heads_through_the_engine(tmp_path):
-    """28 query heads of 128 over 4 kv heads (the head shape of the 7B model, one narrow layer) and prompts long
-    enough that the launcher gives their portions to the prompt kernel whose waves share each block of keys: a
-    prompt of 2,300 tokens in one step beside a short one, then a portion of 700 tokens that starts inside a page
-    after 1,650 cached ones (fewer tiles: one head a wave), then single tokens; also under a window of 1,000
-    keys in the upper layer.  Logits against the plain implementation."""
+@pytest.mark.parametrize("heads,shape", [((28, 4, 128), 12), ((14, 2, 64), 11)])
+def test_long_prompts_with_large_heads_through_the_engine(tmp_path, heads, shape):
+    """28 query heads of 128 over 4 kv heads, or 14 of 64 over 2 (the head shapes of the 7B and the 0.5B model, two
+    narrow layers), and prompts long enough that the launcher gives their portions to the prompt kernel whose waves
+    share each block of keys: a prompt of 2,300 tokens in one step beside a short one, then a portion of 700 tokens
+    that starts inside a page after 1,650 cached ones (fewer tiles: another shape of that kernel), then single
+    tokens; also under a window of 1,000 keys in the upper layer.  Logits against the plain implementation."""
     import tokenizer_amd as ta
     from tokenizer_amd.config import Qwen2Config
     from tokenizer_amd.engine import StepEntry
     from tokenizer_amd.kernels import get_ops
     ops = get_ops()
     assert ops.prefill_shared == 0
-    assert ops.lib.ta_prefill_attention_shared_plan(144 + 2, 28, 4, 128, 2560) == 12     # the first step below: two heads a wave, two key groups
-    raw = dict(TINY["A"][0], num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+    n_q, n_kv, d = heads
+    assert ops.lib.ta_prefill_attention_shared_plan(144 + 2, n_q, n_kv, d, 2560) == shape     # the first step below
+    raw = dict(TINY["A"][0], num_hidden_layers=2, hidden_size=n_q * d, num_attention_heads=n_q, num_key_value_heads=n_kv,
                intermediate_size=256, vocab_size=300, max_position_embeddings=4096, rope_theta=1000000.0,
                use_sliding_window=True, sliding_window=1000, max_window_layers=1)
-    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 17, str(tmp_path / "heads128"), norm_spread=0.3)
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 17, str(tmp_path / "heads"), norm_spread=0.3)
     cfg, tensors = plain.load_folder(folder)
     a_ids, b_ids, c_ids = random_ids(300, 2310, 41), random_ids(300, 30, 42), random_ids(300, 2360, 43)
     want = {"a": plain.all_logits(cfg, tensors, a_ids), "b": plain.all_logits(cfg, tensors, b_ids),
