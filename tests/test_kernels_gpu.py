@@ -258,7 +258,8 @@ def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, windo
                                                            ((28, 2, 64, 16), [2300, 40], [2200, 33], 11),
                                                            ((28, 4, 128, 16), [2300, 40], [2200, 33], 12),
                                                            ((28, 4, 128, 16), [4300, 40], [4200, 33], 2),
-                                                           ((14, 2, 64, 16), [1100, 40], [1000, 33], 11)])
+                                                           ((14, 2, 64, 16), [1100, 40], [1000, 33], 11),
+                                                           ((16, 4, 128, 16), [2300, 40], [2200, 33], 11)])
 @pytest.mark.parametrize("window", [None, 1000])
 def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref, geometry, lengths, q_lens, shape, window):
     # Seven (or twice seven) query heads per kv head and dozens to hundreds of tiles: the launcher's own choice is
@@ -296,7 +297,7 @@ def test_shared_block_prompt_attention_on_random_batches(ops, seed, monkeypatch)
     rng = random.Random(seed)
     d = rng.choice([64, 128])
     n_kv = rng.choice([1, 2, 3])
-    n_q = n_kv * rng.choice([5, 6, 7, 8, 12])
+    n_q = n_kv * rng.choice([3, 4, 5, 6, 7, 8, 12])
     page_size = rng.choice([16, 32, 48, 64])
     window = rng.choice([None, None, rng.randint(1, 40), rng.randint(41, 900)])
     lengths, q_lens = [], []
@@ -329,12 +330,14 @@ def test_where_the_workgroup_shared_kernel_is_planned(ops):
     assert plan(128, 28, 4, 128, 2048) == 12 and plan(256, 28, 4, 128, 4096) == 2
     assert plan(31, 28, 4, 128, 8192) == 0
     assert plan(128, 12, 2, 128, 2048) == 11 and plan(128, 12, 2, 128, 10240) == 12
-    assert plan(4096, 16, 4, 128, 8192) == 0        # four heads per kv head
+    assert plan(128, 32, 8, 128, 2048) == 1 and plan(64, 32, 8, 128, 1024) == 11 and plan(31, 32, 8, 128, 1024) == 0   # four heads per kv head: one a wave
+    assert plan(128, 16, 4, 64, 2048) == 11 and plan(512, 16, 4, 64, 8192) == 1 and plan(512, 24, 8, 128, 8192) == 1
+    assert plan(4096, 16, 8, 128, 8192) == 0        # two heads per kv head
     assert plan(4096, 28, 4, 96, 8192) == 0         # no instance
 
 
 @pytest.mark.parametrize("geometry", [(28, 4, 128, 16), (12, 2, 128, 32), (5, 1, 64, 48), (16, 2, 128, 16),
-                                      (24, 2, 128, 64), (3, 1, 128, 16), (14, 2, 64, 16)])
+                                      (24, 2, 128, 64), (3, 1, 128, 16), (14, 2, 64, 16), (8, 2, 64, 32)])
 @pytest.mark.parametrize("window", [None, 100])
 @pytest.mark.parametrize("heads", [1, 2, 11, 12])
 def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, geometry, window, heads, monkeypatch):

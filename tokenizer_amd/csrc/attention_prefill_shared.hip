@@ -416,7 +416,7 @@ static int launch_shared(const void* q, int q_stride, void* out, const void* k_p
 
 // Whether the workgroup-shared kernel is the faster one, and in which shape: 0 = no, else heads a wave (1 or 2)
 // + 10 if two key groups share a workgroup.  Five to eight query heads per kv head (or more) fill its four waves
-// at two heads a wave.  A workgroup walks all its keys alone, so the launch must fill the device some other way:
+// at two heads a wave, three or four at one.  A workgroup walks all its keys alone, so the launch must fill the device some other way:
 // with 1,024 workgroups and more, two heads a wave; below that two key groups halve the walk, and one head a
 // wave doubles the workgroups (each reading its blocks for half the heads); below 128 workgroups the per-wave
 // kernel, whose waves split the keys of a tile, is the faster one.
@@ -431,7 +431,15 @@ static int launch_shared(const void* q, int q_stride, void* out, const void* k_p
 extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, int d, int reach) {
   if (d != 64 && d != 128) return 0;
   const int group = n_q / n_kv;
-  if (group < 5) return 0;
+  if (group < 3) return 0;
+  if (group < 5) {
+    // Three or four heads per kv head fill the four waves at one head each (32 / 8 heads of 128, per-wave | 1 head
+    // | 1 head, 2 groups: 1,024 tokens 37 | 30 | 28; 2,048 tokens 106 | 69 | 81; 8,192 tokens 1,217 | 790 | 913;
+    // 16 / 4 heads of 64: 2,048 tokens 30.0 | 30.1 | 24.4; 8,192 tokens 307 | 213 | 221).
+    const long one = (long)n_tiles * n_kv;
+    if (one < 256) return 0;
+    return one < (d == 64 ? 2048 : 1024) ? 11 : 1;
+  }
   const long two = (long)n_tiles * n_kv * ((group + 7) / 8);      // workgroups at two heads a wave
   if (two < 128) return 0;
   if (two >= 1024) return 2;
