@@ -270,7 +270,7 @@ def test_the_launcher_takes_the_workgroup_shared_kernel_for_many_tiles(ops, ref,
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=23)
     batch = make_batch(lengths, q_lens)
-    assert ops.prefill_shared == 0 and ops.prefill_waves == 0 and ops.prefill_heads_per_wave == 0
+    assert ops.prefill_shared == 0 and ops.prefill_waves == 0 and ops.prefill_shape == 0
     plan = ops.lib.ta_prefill_attention_shared_plan
     reach = -(-max(lengths) // 512) * 512 if window is None else window + 16
     assert plan(batch.q_tiles.shape[0], n_q, n_kv, d, reach) == shape
@@ -313,7 +313,7 @@ def test_shared_block_prompt_attention_on_random_batches(ops, seed, monkeypatch)
     want = dense_attention(qkv, k_pages, v_pages, table, lengths, q_lens, n_q, n_kv, d, window, scale)
     monkeypatch.setattr(ops, "prefill_shared", 1)
     for heads in (1, 2, 11, 12):
-        monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
+        monkeypatch.setattr(ops, "prefill_shape", heads)
         out = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
         ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
                             max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
@@ -347,7 +347,7 @@ def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, 
     # first pages hold nothing any more, and unwritten slots that hold NaN.  With two heads a wave and with one,
     # with one group of waves and with two that take the blocks in turn (shape = heads a wave + 10 for two groups).
     monkeypatch.setattr(ops, "prefill_shared", 1)
-    monkeypatch.setattr(ops, "prefill_heads_per_wave", heads)
+    monkeypatch.setattr(ops, "prefill_shape", heads)
     n_q, n_kv, d, page_size = geometry
     lengths, q_lens = [700, 333, 40, 16, 1000], [700, 50, 33, 16, 2]
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
@@ -365,7 +365,7 @@ def test_prefill_attention_with_a_block_of_keys_shared_by_a_workgroup(ops, ref, 
     torch.testing.assert_close(out_c.float(), out_b[rows], **tol(torch.bfloat16))
     # The other prompt kernel rounds at other places; both stay within the same distance of the float32 result.
     monkeypatch.setattr(ops, "prefill_shared", -1)
-    monkeypatch.setattr(ops, "prefill_heads_per_wave", 0)
+    monkeypatch.setattr(ops, "prefill_shape", 0)
     out_d = torch.full_like(out_a, float("nan"))
     ops.paged_attention(qkv, out_d, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
                         max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))

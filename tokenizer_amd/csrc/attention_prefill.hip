@@ -327,7 +327,7 @@ extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, voi
 
 // Returns -2 for a head size without an instance (the caller then uses another kernel).
 // max_keys: the highest position of the batch + 1 (a hint for the number of waves per tile).
-// shared: 1 = the workgroup-shared kernel wherever it has an instance (in the shape heads_per_wave names: 1 or 2
+// shared: 1 = the workgroup-shared kernel wherever it has an instance (in the shape `shared_shape` names: 1 or 2
 // heads a wave, + 10 for two key groups; 0 = its own choice), -1 = never, 0 = where it is the faster one (by the shape of the launch and the planned
 // reach, so that a launch recorded for a range of contexts and a launch for the exact context make the same
 // choice).  waves: waves that share a tile's keys in the per-wave kernel (1, 2, 4; 0 = by the reach); asking
@@ -336,13 +336,13 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
                                          int n_q, int n_kv, int d, int page_size, int window, float scale,
-                                         int heads_per_wave, int max_keys, int waves, int shared,
+                                         int shared_shape, int max_keys, int waves, int shared,
                                          hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
   if (shared >= 0 && waves == 0) {
     int shape = ta_prefill_attention_shared_plan(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window));
-    if (shared > 0) shape = heads_per_wave > 0 ? heads_per_wave : shape ? shape : 2;
+    if (shared > 0) shape = shared_shape > 0 ? shared_shape : shape ? shape : 2;
     if (shape) {
       const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
                                                           first_position, block_table, table_stride, n_q, n_kv, d,

@@ -262,7 +262,7 @@ class Ops:
                 _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(batch.q_tiles),
                 batch.q_tiles.shape[0], _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
                 block_table.shape[1], n_q, n_kv, head_dim, page_size, -1 if window is None else int(window),
-                ctypes.c_float(scale), self.prefill_heads_per_wave, int(batch.max_position) + 1,
+                ctypes.c_float(scale), self.prefill_shape, int(batch.max_position) + 1,
                 self.prefill_waves, self.prefill_shared, self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
                 self._decode_attention(*args, rows=batch.decode_rows)
@@ -276,9 +276,10 @@ class Ops:
 
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
     use_fast_attention = True     # tests switch it off to reach the generic kernel in bfloat16
-    prefill_waves = 0          # waves that share a tile's keys in the prompt kernel: 0 lets the launcher choose
-    prefill_heads_per_wave = 0    # shape of the workgroup-shared prompt kernel when it is asked for: heads a wave (1 or 2),
-    #                               + 10 for two key groups in a workgroup; 0: its own choice
+    prefill_waves = 0             # waves that share a tile's keys in the per-wave prompt kernel: 0 lets the launcher choose;
+    #                               asking for a number asks for that kernel
+    prefill_shape = 0             # shape of the workgroup-shared prompt kernel when it is asked for: heads a wave
+    #                               (1 or 2), + 10 for two key groups in a workgroup; 0: its own choice
     prefill_shared = 0            # the prompt kernel whose waves share a block of keys through LDS: 1 = wherever it has
     #                               an instance, -1 = never, 0 = where the launcher expects it to be the faster one
     target_workgroups = 1024      # what the split of the key range aims at
