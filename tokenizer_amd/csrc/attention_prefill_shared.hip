@@ -131,6 +131,36 @@ struct Carrier {
   __device__ __forceinline__ static void landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 };
 
+// O^T += V^T P^T for one head over the block in `buf`, and the probabilities' sum by the same means: one more
+// row block of V^T that holds ones gives every lane its token's sum over all 64 keys (of the rounded
+// probabilities, the very weights of the product), where sixteen additions a head and two exchanges between
+// lanes at the end stood.
+template <int D, bool FULL>
+__device__ __forceinline__ void second_product(const char* buf, int kb, int col, int g, int lo, int hi,
+                                               const bf16x8 (&pf)[2], floatx4 (&acc)[D / 16], floatx4& l) {
+  bf16x8 ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    l = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[u], l, 0, 0, 0);
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      bf16x8 vf = *reinterpret_cast<const bf16x8*>(buf + Staged<D>::K_BYTES + (2 * u + (g >> 1)) * Staged<D>::V_RUN +
+                                                   (db * 16 + col) * 32 + (g & 1) * 16);
+      if (!FULL) {
+        // A probability of zero times whatever lies in a slot that was never written, or in a borrowed page,
+        // must stay zero.
+        const int first = kb + 32 * u + 8 * g;             // the lane's keys: first .. first + 7
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (first + i > hi || first + i < lo) vf[i] = (__bf16)0.0f;
+      }
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], acc[db], 0, 0, 0);
+    }
+  }
+}
+
 // One step of the online softmax of a wave's HG heads over the block of 64 keys in `buf`.  Row r of the first
 // product's instruction t of a half of 32 keys is key 8 (r / 4) + 4 t + r % 4 of the half, whose score then lies
 // in the lane group that holds that key in the second product (lane group g: keys 8g .. 8g+7).
@@ -194,34 +224,10 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
 #pragma unroll
     for (int i = 0; i < 16; ++i)
       pf[h][i >> 3][i & 7] = (__bf16)__builtin_amdgcn_exp2f(fmaf(sh[i], c, -mc));   // masked keys: exp2(-inf) = 0
+    // The head's second product follows at once, so that the matrix cores work on it while the vector unit
+    // works on the next head's probabilities (the values are read from LDS once per head for that).
+    second_product<D, FULL>(buf, kb, col, g, lo, hi, pf[h], acc[h], l[h]);
   }
-  // The probabilities' sums come from the matrix cores as well, as one more row block of V^T that holds ones:
-  // every lane then has its token's sum over all 64 keys (of the rounded probabilities, the very weights of the
-  // second product), where sixteen additions a head and two exchanges between lanes at the end stood.
-  bf16x8 ones;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
-#pragma unroll
-  for (int u = 0; u < 2; ++u)
-#pragma unroll
-    for (int h = 0; h < HG; ++h) l[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[h][u], l[h], 0, 0, 0);
-#pragma unroll
-  for (int u = 0; u < 2; ++u)
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      bf16x8 vf = *reinterpret_cast<const bf16x8*>(buf + Staged<D>::K_BYTES + (2 * u + (g >> 1)) * Staged<D>::V_RUN +
-                                                   (db * 16 + col) * 32 + (g & 1) * 16);
-      if (!FULL) {
-        // A probability of zero times whatever lies in a slot that was never written, or in a borrowed page,
-        // must stay zero.
-        const int first = kb + 32 * u + 8 * g;             // the lane's keys: first .. first + 7
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (first + i > hi || first + i < lo) vf[i] = (__bf16)0.0f;
-      }
-#pragma unroll
-      for (int h = 0; h < HG; ++h) acc[h][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[h][u], acc[h][db], 0, 0, 0);
-    }
 }
 
 // Arguments as in prefill_attention_kernel.  Dynamic LDS: two blocks for each of the KG groups of four waves
