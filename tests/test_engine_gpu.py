@@ -208,6 +208,40 @@ def test_long_prompts_with_large_heads_through_the_engine(tmp_path, heads, shape
     eng.cache.check_invariants()
 
 
+def test_recorded_steps_with_the_shared_block_prompt_attention(tmp_path):
+    """Five prompts of the same length, one after the other, at the 7B model's head shape: the step's shape recurs,
+    so the later ones replay a captured graph, in which the prompt attention is the kernel whose waves share their
+    blocks of keys (it asks the runtime for more LDS than the default at every launch, recorded or not).  Every
+    prompt's logits against the plain implementation and against an engine that records nothing."""
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import StepEntry
+    from tokenizer_amd.kernels import get_ops
+    assert get_ops().lib.ta_prefill_attention_shared_plan(69, 28, 4, 128, 1536) == 11
+    raw = dict(TINY["A"][0], num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+               intermediate_size=256, vocab_size=300, max_position_embeddings=2048, rope_theta=1000000.0)
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 19, str(tmp_path / "recorded"), norm_spread=0.3)
+    cfg, tensors = plain.load_folder(folder)
+    prompts = [random_ids(300, 1100, 60 + i) for i in range(5)]
+    rows = [0, 500, 1099]
+    got = {}
+    for use_graphs in (True, False):
+        eng = engine_for(folder, "bfloat16", max_tokens=1152, max_requests=1, use_graphs=use_graphs)
+        eng.pools.poison()
+        for i, ids in enumerate(prompts):
+            eng.add_request(i)
+            got[use_graphs, i] = eng.step([StepEntry(i, ids, rows)]).float().cpu()
+            eng.end_request(i)
+        if use_graphs:
+            assert any(not isinstance(key[0], int) for key in eng.graphs), "the recurring shape was not captured"
+    for i, ids in enumerate(prompts):
+        close(got[True, i], plain.all_logits(cfg, tensors, ids)[rows], "bfloat16")
+    # The first step ran eagerly in both engines; the last one replays a graph in the first (whose big library
+    # products were timed again before the capture, so their rounding may differ from the eager engine's).
+    assert torch.equal(got[True, 0], got[False, 0])
+    close(got[True, 4], got[False, 4], "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", list(TINY))
 def test_first_tokens_of_a_sequence(model_folders, oracle, name, dtype):
