@@ -1,13 +1,15 @@
-// Prompt attention for many query heads per kv head and long reaches: the workgroup of a tile of 16 tokens and one
-// kv head holds four waves, each with HG of the query heads that share the kv head, and all of them walk the
-// same blocks of 64 keys.  A block's keys and values come from the pages once for the whole workgroup, by loads
-// that write straight into LDS (no register on the way), two buffers deep: the next block is on its way while
-// the matrix cores work on the current one, and every wave takes its fragments from LDS.  Against the kernel in
-// attention_prefill.hip (each wave fetches its own blocks for its own two heads) a key is read from the cache half
-// or a quarter as often (one or two heads a wave) and no wave waits for memory with nothing else to do; it pays where the pages' traffic or
-// its latency bound that kernel: large heads, long prompts.  Same fragment layouts and key order as there:
-// S^T = K Q^T and O^T = V^T P^T with 16x16x32 MFMAs, token index in `lane % 16`, softmax online in float,
-// probabilities rounded to bfloat16 for the second product.
+// Prompt attention whose waves share their keys: the workgroup of a tile of 16 tokens and one kv head holds four
+// waves, each with HG (1 or 2) of the query heads that share the kv head, and all of them walk the same blocks of
+// 64 keys.  A block's keys and values come from the pages once for the whole workgroup, by loads that write
+// straight into LDS (no register on the way), two buffers deep: the next block is on its way while the matrix
+// cores work on the current one, and every wave takes its fragments from LDS.  With KG = 2 a second group of
+// four waves with the same heads takes every other block, and the groups merge their softmax states at the end.
+// Against the kernel in attention_prefill.hip (each wave fetches its own blocks for its own two heads) a key is
+// read from the cache half or a quarter as often, and no wave waits for memory with nothing else to do; which
+// of the two kernels, and which shape of this one, a launch gets is `ta_prefill_attention_shared_plan`'s
+// choice.  Same fragment layouts and key order as there: S^T = K Q^T and O^T = V^T P^T with 16x16x32 MFMAs,
+// token index in `lane % 16`, softmax online in float, probabilities rounded to bfloat16 for the second product
+// (whose row block of ones also yields their sums).
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
