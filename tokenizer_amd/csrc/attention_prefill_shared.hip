@@ -38,6 +38,13 @@ struct Staged {
   __device__ static constexpr int swizzle(int key) { return (key & 3) | ((key >> 1) & 4); }
 };
 
+__device__ __forceinline__ float max2(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float max16(const float (&v)[16]) {
+  const float a = max2(max2(v[0], v[1]), v[2]), b = max2(max2(v[3], v[4]), v[5]), c = max2(max2(v[6], v[7]), v[8]);
+  const float d = max2(max2(v[9], v[10]), v[11]), e = max2(max2(v[12], v[13]), v[14]);
+  return max2(max2(max2(a, b), c), max2(max2(d, e), v[15]));
+}
+
 __device__ __forceinline__ bf16x8 sh_zero8() {
   bf16x8 z;
 #pragma unroll
@@ -203,14 +210,15 @@ __device__ __forceinline__ void shared_block(const char* buf, int kb, int col, i
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     const float (&sh)[16] = s[h];
-    // (Through fmaxf, which the compiler knows: the scores come straight from matrix instructions, whose results
-    // a vector instruction may only read after wait states that the compiler counts; it cannot count them for an
-    // instruction written in inline assembly, and a v_max3_f32 written that way read scores too early now and then.)
-    float mx = fmaxf(fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3])), fmaxf(fmaxf(sh[4], sh[5]), fmaxf(sh[6], sh[7])));
-    mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(sh[8], sh[9]), fmaxf(sh[10], sh[11])), fmaxf(fmaxf(sh[12], sh[13]), fmaxf(sh[14], sh[15]))));
-    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(m[h], mx);
+    // The IEEE maximum (a NaN would spread, but masked scores are -inf and the others products of stored numbers)
+    // rather than fmaxf: the compiler joins it into v_maximum3_f32, eight instructions for sixteen scores, where
+    // fmaxf first rewrites every score that might be a signalling NaN.  (Not inline assembly: the scores come
+    // straight from matrix instructions, whose results a vector instruction may only read after wait states that
+    // the compiler counts for the instructions it knows; a v_max3_f32 written in assembly read them too early.)
+    float mx = max16(sh);
+    mx = max2(mx, __shfl_xor(mx, 16, WAVE));
+    mx = max2(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = max2(m[h], mx);
     // A token that has seen no key yet keeps m = -inf; exp2 of (-inf) - (-inf) would be NaN.
     const float mc = (m_new == -INFINITY) ? 0.f : m_new * c;
     if (__any(m_new > m[h])) {                          // rescale only when some token's maximum moved
