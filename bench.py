@@ -12,6 +12,10 @@ JSON line.
 runs a whole serving workload through the scheduler instead (64 requests at Qwen2.5-1.5B sizes
 with prompts of 128 to 2,048 ids and 256 new tokens each; 64 requests at Qwen2.5-7B sizes that
 share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for it.
+
+    python bench.py [--size 0.5b|1.5b|7b] --attention TOKENS [--cached C] [--attention-kernel auto|per-wave|shared]
+
+times the prompt attention kernel alone on a portion of TOKENS tokens after C cached ones.
 """
 from __future__ import annotations
 
@@ -240,6 +244,52 @@ def measure_peaks() -> dict:
     return out
 
 
+def run_attention(sizes: dict, tokens: int, cached: int, kernel: str, repeats: int = 20) -> dict:
+    """The prompt attention kernel alone at a size's head shape: a portion of `tokens` tokens after `cached` cached
+    ones, timed back to back on random keys and values (bfloat16, pages of 16).  kernel: "auto" (the launcher's
+    choice), "per-wave" or "shared" (with the launcher's shape where it plans one, else two heads a wave)."""
+    import types
+    import torch
+    from tokenizer_amd.kernels import get_ops
+    ops = get_ops()
+    n_q, n_kv = sizes["num_attention_heads"], sizes["num_key_value_heads"]
+    d = sizes["hidden_size"] // n_q
+    page, length = 16, cached + tokens
+    n_pages = length // page + 1
+    dev, bf = "cuda:0", torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    k_pages = torch.randn((n_pages, n_kv, page, d), generator=gen, device=dev).to(bf)
+    v_pages = torch.randn((n_pages, n_kv, d, page), generator=gen, device=dev).to(bf)
+    qkv = torch.randn((tokens, (n_q + 2 * n_kv) * d), generator=gen, device=dev).to(bf)
+    out = torch.empty((tokens, n_q * d), dtype=bf, device=dev)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device=dev)
+    table = torch.arange(n_pages, dtype=torch.int32, device=dev).reshape(1, n_pages)
+    positions = torch.arange(cached, length, dtype=torch.int32, device=dev)
+    entry_of_token = torch.zeros(tokens, dtype=torch.int32, device=dev)
+    batch = types.SimpleNamespace(n_tokens=tokens, cu_q=ints([0, tokens]), first_position=ints([cached]),
+                                  q_tiles=ints([[0, o] for o in range(0, tokens, 16)]), decode_rows=ints([]),
+                                  max_position=length - 1)
+    tiles = batch.q_tiles.shape[0]
+    plan = ops.lib.ta_prefill_attention_shared_plan(tiles, n_q, n_kv, d, -(-length // 512) * 512)
+    ops.prefill_shared = {"auto": 0, "per-wave": -1, "shared": 1}[kernel]
+
+    def run():
+        ops.paged_attention(qkv, out, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, None, d ** -0.5,
+                            max_position=length - 1, batch=batch)
+    run()
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(repeats):
+        run()
+    torch.cuda.synchronize()
+    seconds = (time.perf_counter() - started) / repeats
+    ops.prefill_shared = 0
+    flops = 4.0 * n_q * d * (tokens * cached + tokens * (tokens + 1) / 2)
+    return {"attention_us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1), "tokens": tokens,
+            "cached": cached, "q_heads": n_q, "kv_heads": n_kv, "head_dim": d, "kernel": kernel,
+            "planned_shape": plan}
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -257,6 +307,11 @@ def main() -> int:
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
+    parser.add_argument("--attention", type=int, default=None, metavar="TOKENS",
+                        help="time the prompt attention kernel alone on a portion of this many tokens at --size's head shape")
+    parser.add_argument("--cached", type=int, default=0, help="with --attention: tokens already in the cache")
+    parser.add_argument("--attention-kernel", default="auto", choices=["auto", "per-wave", "shared"],
+                        help="with --attention: the launcher's choice, or one of the two prompt kernels")
     parser.add_argument("--temperature", type=float, default=0.0,
                         help="with --workload: draw with this temperature and top_p 0.95 instead of greedy picks")
     parser.add_argument("--prompt-len", type=int, default=None,
@@ -282,6 +337,9 @@ def main() -> int:
         print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature)), flush=True)
         return 0
     sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
+    if args.attention:
+        print(json.dumps(run_attention(sizes, args.attention, args.cached, args.attention_kernel)), flush=True)
+        return 0
     full_layers = sizes["num_hidden_layers"]
     args.layers = args.layers or full_layers
 
