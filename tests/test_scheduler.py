@@ -103,6 +103,26 @@ def test_a_prompt_that_can_never_fit_fails_and_the_next_runs(model_folders):
     sched.assert_idle()
 
 
+def test_a_sequence_that_outgrows_the_pool_alone_in_the_batch_does_not_take_the_next_with_it(model_folders):
+    """Batches of one: the running sequence outgrows the whole pool and fails in an iteration that runs nothing.
+    Its pages are back then, and the queue's front, which needs exactly the whole pool, runs in the next one
+    (that nothing ran while nothing is running does not mean that the front can never be admitted)."""
+    folder = model_folders["A"]
+    config = SchedulerConfig(max_batch_size=1, num_blocks=5, prefix_cache=False, prefill_chunk=5,
+                             max_num_batched_tokens=16)
+    sched = Scheduler(cpu_engine(folder, num_pages=5, max_requests=1), config)
+    outgrows = sched.add_request(random_ids(256, 80, 1), GenerateParams.greedy(9))     # 89 tokens: six pages
+    fits_prompt = random_ids(256, 64, 2)
+    fits = sched.add_request(fits_prompt, GenerateParams.greedy(9))                    # 73 tokens: five pages
+    while sched.has_work():                      # one iteration a call, as a server's loop drives it
+        sched.run(max_steps=1)
+    results = sched.finished
+    assert isinstance(results[outgrows], Failure) and "needs 6" in results[outgrows].message
+    assert isinstance(results[fits], Generated), results[fits]
+    assert results[fits].tokens == solo(folder, fits_prompt, GenerateParams.greedy(9)).tokens
+    sched.assert_idle()
+
+
 def test_requests_that_cannot_be_accepted(model_folders):
     sched = Scheduler(cpu_engine(model_folders["A"]), SchedulerConfig(max_waiting=2))
     empty = sched.add_request([], GenerateParams.greedy(3))
@@ -185,7 +205,7 @@ def test_cancel(model_folders):
     sched.assert_idle()
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(12))
 def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed):
     """Random prompts, output lengths, pool sizes, batch caps, token budgets, portion sizes and arrival times
     (shared prefixes included): whatever the scheduler decides, every request gets the tokens it would get alone,
@@ -194,7 +214,7 @@ def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed
     rng = random.Random(seed)
     folder = model_folders["A"]
     page = 16
-    num_pages = rng.choice([4, 6, 9, 24])
+    num_pages = rng.choice([4, 5, 6, 9, 24])
     config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 3, 5]), num_blocks=num_pages,
                              prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 16, 40]),
                              prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64)
@@ -207,7 +227,7 @@ def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed
         prompt = random_ids(256, rng.choice([1, 2, 7, 16, 17, 33, 48]), 100 * seed + i)
         if rng.random() < 0.4:
             prompt = shared[:rng.choice([16, 32, 35])] + prompt
-        plan.append((rng.randint(0, 6), prompt, rng.randint(0, 7)))
+        plan.append((rng.randint(0, 6), prompt, rng.randint(0, 9)))
     ids, step = {}, 0
     pending = sorted(plan, key=lambda item: item[0])
     while pending or sched.has_work():

@@ -182,7 +182,9 @@ class Scheduler:
     # ----------------------------------------------------------------------- step
     def step(self) -> bool:
         """One iteration: the core admits, plans (pages reserved, the newest sequence preempted when they run
-        out) and requeues; the plan is then run as one batch.  Returns False when there was nothing to run."""
+        out) and requeues; the plan is then run as one batch.  Returns False when nothing changed: nothing ran,
+        nothing was preempted and nothing failed (a sequence that fails gives back its pages, so the queue's
+        front may well be admitted in the next iteration)."""
         room = max(1, len(self.sequences))
         planned = (ctypes.c_int64 * (4 * room))()
         preempted = (ctypes.c_int64 * room)()
@@ -204,7 +206,7 @@ class Scheduler:
             else:
                 self._run(plan)
         self._note_peaks()
-        return bool(plan) or n_preempted > 0
+        return bool(plan) or n_preempted > 0 or n_failed > 0
 
     def _tokens(self, seq_id: int, first: int, count: int) -> list[int]:
         out = (ctypes.c_int32 * max(1, count))()
