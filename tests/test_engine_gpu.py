@@ -679,8 +679,7 @@ def test_other_page_sizes(model_folders, oracle, dtype, page_size):
         reqs = requests_for(name)
         steps = tt.mixed(reqs, 7)
         live = tt.peak_tokens(steps)
-        eng = engine_for(model_folders[name], dtype, num_pages=-(-live // page_size) + 4, page_size=page_size,
-                         max_requests=4)
+        eng = engine_for(model_folders[name], dtype, max_tokens=live, page_size=page_size, max_requests=4)
         eng.pools.poison()
         got = tt.run_in_process(eng, steps)
         for rid, ids in reqs.items():

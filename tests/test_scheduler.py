@@ -262,3 +262,19 @@ def test_a_step_that_may_not_reserve_refuses_an_entry_without_pages(model_folder
     assert engine.step([StepEntry("a", [1, 2, 3], [2])], reserve=False).shape == (1, 256)
     assert engine.cache.seq_len("a") == 3 and engine.cache.groups[0].allocator.live_count() == 1
     engine.end_request("a")
+
+
+@pytest.mark.parametrize("page_size", [16, 48, 128])
+def test_a_pool_made_for_so_many_tokens_holds_them_at_any_page_size(model_folders, page_size):
+    """`Engine(max_tokens=N)`: N counts each live request's tokens rounded up to a multiple of 64.  Pages that do
+    not divide 64 round each request up on their own; four requests of 64 tokens still find their pages."""
+    from kernel_refs import PlainOps
+    from tokenizer_amd.engine import Engine, load_model
+    engine = Engine(load_model(model_folders["A"], "float32", "cpu", ops=PlainOps()), max_tokens=4 * 64,
+                    page_size=page_size, max_requests=4)
+    for rid in range(4):
+        engine.add_request(rid)
+        assert engine.cache.reserve(rid, 64), (rid, engine.cache.num_pages)
+    for rid in range(4):
+        engine.end_request(rid)
+    engine.cache.check_invariants()

@@ -170,7 +170,9 @@ class Engine:
                  num_blocks: int | None = None, max_batch_size: int | None = None,
                  max_num_batched_tokens: int = 2048):
         """`num_blocks` and `max_batch_size` are the reference's names (qwen-server/src/lib.rs:33-56) for
-        `num_pages` and `max_requests`; `max_num_batched_tokens` is the token budget of `run()`."""
+        `num_pages` and `max_requests`; `max_num_batched_tokens` is the token budget of `run()`.  Without
+        `num_pages` the pool is made for `max_tokens`: the most tokens that live requests hold at any time, each
+        request's count rounded up to a multiple of 64."""
         num_pages = num_blocks if num_pages is None else num_pages
         max_requests = max_batch_size if max_batch_size is not None else max_requests
         self.max_num_batched_tokens = max_num_batched_tokens
@@ -178,7 +180,9 @@ class Engine:
         if num_pages is None:
             if max_tokens is None:
                 raise ValueError("give num_pages or max_tokens")
-            num_pages = -(-max_tokens // page_size)
+            # `max_tokens` counts every live request's tokens rounded up to a multiple of 64.  Pages whose size
+            # does not divide 64 round each request up on their own: at worst one page more per further request.
+            num_pages = -(-max_tokens // page_size) + (max_requests - 1 if 64 % page_size else 0)
         self.model = model
         self.cache = CacheManager(model.cache_needs, num_pages, page_size, max_requests, prefix_cache)
         self.pools = CachePools(self.cache, model.cache_needs, model.dtype, model.device)
