@@ -282,14 +282,17 @@ def test_trace_run_program(model_folders, oracle, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_captured_decode_steps_equal_eager_ones(model_folders, dtype):
+@pytest.mark.parametrize("page_size", [16, 48])
+def test_captured_decode_steps_equal_eager_ones(model_folders, dtype, page_size):
     # The same trace with and without graph replay: decode steps of changing batch size, with a mixed step
-    # (captured from its third appearance) between them, each replay checked against the eager engine.
+    # (captured from its third appearance) between them, each replay checked against the eager engine.  Pages of
+    # 48 tokens: a graph's context range is no whole number of pages, and still it plans its launches for the
+    # range an eager step plans for.
     from tokenizer_amd.engine import StepEntry
     name = "B"
     vocab = TINY[name][0]["vocab_size"]
-    engines = [engine_for(model_folders[name], dtype, max_tokens=1024, max_requests=4, use_graphs=flag)
-               for flag in (True, False)]
+    engines = [engine_for(model_folders[name], dtype, max_tokens=1024, max_requests=4, use_graphs=flag,
+                          page_size=page_size) for flag in (True, False)]
     assert engines[0].use_graphs and not engines[1].use_graphs
     prompts = {rid: random_ids(vocab, n, 50 + rid) for rid, n in enumerate([37, 5, 64])}
     for eng in engines:

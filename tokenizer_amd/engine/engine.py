@@ -72,7 +72,7 @@ class StepGraph:
 
     def __init__(self, engine: "Engine", entries: list[StepEntry], bucket: int):
         self.bucket = bucket
-        self.width = bucket // engine.cache.page_size
+        self.width = -(-bucket // engine.cache.page_size)
         device = engine.model.device
         probe = build_context(entries, engine.cache, device, table_width=self.width)
         size = sum(t.numel() for t in (probe.token_ids, probe.positions, probe.entry_of_token, probe.cu_q,
@@ -302,8 +302,9 @@ class Engine:
 
     def _graph_key(self, entries: list[StepEntry]) -> tuple:
         longest = max(self.cache.seq_len(e.rid) + len(e.tokens) for e in entries)
+        # (The bucket is what the kernels' launch shapes are planned for, with any page size: an eager step plans
+        # for its context rounded up in the same way, so both cut their sums alike.)
         bucket = -(-longest // self.GRAPH_BUCKET) * self.GRAPH_BUCKET
-        bucket = -(-bucket // self.cache.page_size) * self.cache.page_size
         return (self._shape_of(entries), bucket)
 
     def _graph_for(self, entries: list[StepEntry]) -> "StepGraph":
