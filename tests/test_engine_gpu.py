@@ -651,6 +651,66 @@ def test_sizes_away_from_every_tile(tmp_path, size):
                 close(got[rid], want[rid], dtype)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_configurations_pages_and_traces(tmp_path, seed):
+    """Configurations drawn at random (head sizes in steps of 16, any number of heads and groups, inner widths and
+    vocabularies that are no power of two, windows on some layers, one to three layers), pages of 16, 32 or 48
+    tokens, one of the ways to cut requests into steps, 32-bit or bfloat16: every logit against the plain model,
+    nothing left over.  With every step recorded and replayed at its first sight (odd seeds), the replays also equal
+    an engine that records nothing, bit for bit."""
+    import random
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import Engine
+    from tokenizer_amd.kernels import get_ops
+    rng = random.Random(5000 + seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    n_kv = rng.choice([1, 2, 3, 5])
+    n_q = n_kv * rng.choice([1, 2, 3, 4, 7, 8] if d <= 64 else [1, 2, 4])
+    layers = rng.choice([1, 2, 3])
+    window = rng.random() < 0.4
+    max_pos = rng.choice([160, 300, 520])
+    raw = dict(TINY["A"][0], num_hidden_layers=layers, hidden_size=n_q * d, num_attention_heads=n_q,
+               num_key_value_heads=n_kv, intermediate_size=rng.choice([40, 100, 136, 272, 500]),
+               vocab_size=rng.choice([97, 256, 333, 1000]), rope_theta=rng.choice([10000.0, 1e6]),
+               rms_norm_eps=rng.choice([1e-6, 1e-5]), tie_word_embeddings=rng.random() < 0.5,
+               max_position_embeddings=max_pos, use_sliding_window=window,
+               sliding_window=rng.choice([5, 21, 64, 100]) if window else max_pos,
+               max_window_layers=rng.randrange(0, layers + 1) if window else layers)
+    page_size = rng.choice([16, 16, 32, 48])
+    dtype = rng.choice(["float32", "bfloat16"])
+    kind = rng.choice(["mixed", "portions", "tail"])
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), seed, str(tmp_path / "drawn"), norm_spread=0.3)
+    cfg, tensors = plain.load_folder(folder)
+    lens = [min(n, max_pos) for n in rng.sample([1, 2, 9, 17, 40, 64, 65, 100, 130, 150, 257, 400], 5)]
+    reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 10 * seed + i) for i, n in enumerate(lens)}
+    steps = {"mixed": lambda: tt.mixed(reqs, seed), "portions": lambda: tt.portions(reqs, seed),
+             "tail": lambda: tt.decode_tail(reqs)}[kind]()
+    recorded = seed % 2 == 1
+    before = (Engine.GRAPH_AFTER, Engine.STEP_GRAPHS, get_ops().EAGER_LIBRARY_WORK)
+    try:
+        if recorded:
+            Engine.GRAPH_AFTER, Engine.STEP_GRAPHS = 1, 10 ** 6
+            get_ops().EAGER_LIBRARY_WORK = 0          # eager steps choose their products as recorded ones do
+        eng = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=4, page_size=page_size)
+        eng.pools.poison()
+        got = tt.run_in_process(eng, steps)
+        for rid, ids in reqs.items():
+            close(got[rid], plain.all_logits(cfg, tensors, ids), dtype)
+        eng.cache.check_invariants()
+        assert not eng.cache.requests
+        if recorded:
+            assert eng.graphs
+            eager = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=4, page_size=page_size,
+                               use_graphs=False)
+            eager.pools.poison()
+            again = tt.run_in_process(eager, steps)
+            for rid in reqs:
+                assert torch.equal(got[rid], again[rid]), rid
+    finally:
+        Engine.GRAPH_AFTER, Engine.STEP_GRAPHS, get_ops().EAGER_LIBRARY_WORK = before
+
+
 def test_the_whole_model_at_half_a_billion_parameters(tmp_path):
     # All 24 layers and the vocabulary of 151,936 at Qwen2.5-0.5B sizes, random weights: prompts in portions beside
     # decoded tokens and with their last tokens one by one, in 32-bit and in bfloat16, against the plain implementation.

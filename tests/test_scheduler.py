@@ -250,6 +250,73 @@ def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed
     sched.assert_idle()
 
 
+def requests_of_every_kind(rng, vocab, seed):
+    """Prompts (some with a shared beginning) with greedy or warm sampling, nucleus cuts, end-of-sequence ids, stop
+    strings and budgets down to zero, and the steps at which they arrive."""
+    shared = random_ids(vocab, 40, 7000 + seed)
+    plan = []
+    for i in range(rng.randint(3, 8)):
+        prompt = random_ids(vocab, rng.choice([1, 3, 15, 16, 17, 31, 40]), 50 * seed + i)
+        if rng.random() < 0.4:
+            prompt = shared[:rng.choice([16, 32, 40])] + prompt
+        warm = rng.random() < 0.5
+        params = GenerateParams(max_tokens=rng.choice([0, 1, 2, 5, 9, 14]),
+                                temperature=rng.choice([0.7, 1.0, 1.5]) if warm else 0.0,
+                                top_p=rng.choice([1.0, 0.9, 0.5]) if warm else 1.0, seed=rng.randint(0, 99),
+                                eos=[rng.randrange(vocab) for _ in range(rng.choice([0, 0, 3, 40]))],
+                                stop=rng.choice([[], [], ["ab"], ["cc", "gfe"], ["a"]]))
+        plan.append((rng.randint(0, 5), prompt, params))
+    return sorted(plan, key=lambda item: item[0])
+
+
+def run_requests_of_every_kind(make_engine, folder, vocab, seed):
+    """Drive a scheduler over `make_engine(...)` with random limits through such requests; every result must be
+    what the same request gives when it is generated alone."""
+    import random
+    rng = random.Random(1000 + seed)
+    num_pages = rng.choice([5, 6, 8, 12, 30])
+    config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 4, 6]), num_blocks=num_pages,
+                             prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 24, 64]),
+                             prefill_chunk=rng.choice([None, 7, 16]), max_waiting=64,
+                             decode_burst=rng.choice([1, 4, 16]))
+    engine = make_engine(folder, num_pages=num_pages, max_requests=config.max_batch_size,
+                         prefix_cache=config.prefix_cache)
+    alone = make_engine(folder, num_pages=40, max_requests=1, prefix_cache=False)
+    sched = Scheduler(engine, config)
+    token_bytes = lambda token: bytes([97 + token % 7])
+    pending = requests_of_every_kind(rng, vocab, seed)
+    ids, step = {}, 0
+    while pending or sched.has_work():
+        while pending and pending[0][0] <= step:
+            _, prompt, params = pending.pop(0)
+            ids[sched.add_request(prompt, params, token_bytes=token_bytes)] = (prompt, params)
+        if sched.has_work():
+            sched.run(max_steps=1)
+        step += 1
+        assert step < 3000
+        engine.cache.check_invariants()
+    for rid, (prompt, params) in ids.items():
+        got = sched.finished[rid]
+        if isinstance(got, Failure):
+            assert "kv pool has" in got.message and -(-(len(prompt) + params.max_tokens) // 16) > num_pages
+            continue
+        want = generate(alone, prompt, params, token_bytes=token_bytes)
+        assert (got.tokens, got.text, got.reason, got.completion_tokens, "".join(got.chunks)) == \
+               (want.tokens, want.text, want.reason, want.completion_tokens, "".join(want.chunks)), (rid, params)
+    sched.assert_idle()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_requests_of_every_kind_get_what_they_get_alone(model_folders, seed):
+    """Greedy and warm requests, nucleus cuts, end-of-sequence ids, stop strings and zero budgets side by side, under
+    random pools, batch caps, token budgets and portion sizes: tokens, text, chunks, reason and counts of every
+    request equal those of the request generated alone (qwen-server/src/engine.rs:1328-1420 widened)."""
+    name = "ABC"[seed % 3]
+    vocab = {"A": 256, "B": 384, "C": 320}[name]
+    run_requests_of_every_kind(lambda folder, **kw: cpu_engine(folder, counting=False, **kw), model_folders[name],
+                               vocab, seed)
+
+
 def test_a_step_that_may_not_reserve_refuses_an_entry_without_pages(model_folders):
     """The scheduler reserves while it plans; the step it then runs takes nothing from the pool."""
     from tokenizer_amd.engine import StepEntry
