@@ -205,6 +205,60 @@ def test_cancel(model_folders):
     sched.assert_idle()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_requests_cancelled_at_random_keep_what_they_sampled(model_folders, seed):
+    """Requests cancelled from outside at random iterations (waiting, in the middle of their prompt, decoding) or by
+    their own chunk callback after so many chunks, among requests that run to their end, under small pools: a
+    cancelled request holds a beginning of what it would have got alone, the others all of it, nothing is left."""
+    import random
+    from tokenizer_amd.engine.generate import Control
+    rng = random.Random(3000 + seed)
+    folder = model_folders["A"]
+    num_pages = rng.choice([5, 8, 12, 30])
+    config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 4]), num_blocks=num_pages, prefix_cache=rng.random() < 0.5,
+                             max_num_batched_tokens=rng.choice([8, 24, 64]), prefill_chunk=rng.choice([None, 7, 16]))
+    engine = cpu_engine(folder, num_pages=num_pages, max_requests=config.max_batch_size,
+                        prefix_cache=config.prefix_cache, counting=False)
+    sched = Scheduler(engine, config)
+    token_bytes = lambda token: bytes([97 + token % 7])
+    shared = random_ids(256, 40, 7000 + seed)
+    ids = {}
+    for i in range(rng.randint(4, 7)):
+        prompt = random_ids(256, rng.choice([1, 3, 15, 16, 17, 31, 40]), 50 * seed + i)
+        if rng.random() < 0.4:
+            prompt = shared[:rng.choice([16, 32, 40])] + prompt
+        params = GenerateParams(max_tokens=rng.choice([1, 5, 9, 14]), temperature=rng.choice([0.0, 1.0]), seed=i)
+        limit = rng.choice([None, None, 0, 1, 3])          # the callback says Stop after so many chunks
+
+        def on_chunk(text, limit=limit, seen=[0]):
+            if limit is None or (text == "" and limit > 0):
+                return Control.Continue
+            seen[0] += 1
+            return Control.Stop if seen[0] > limit else Control.Continue
+
+        ids[sched.add_request(prompt, params, token_bytes=token_bytes, on_chunk=on_chunk)] = (prompt, params, limit)
+    from_outside = {rid: rng.randint(0, 12) for rid in ids if rng.random() < 0.3}
+    step = 0
+    while sched.has_work():
+        for rid, when in from_outside.items():
+            if when == step:
+                sched.cancel(rid)
+        sched.run(max_steps=1)
+        step += 1
+        assert step < 3000
+        engine.cache.check_invariants()
+    for rid, (prompt, params, limit) in ids.items():
+        got = sched.finished[rid]
+        assert isinstance(got, Generated), got
+        want = generate(cpu_engine(folder), prompt, params, token_bytes=token_bytes)
+        assert got.tokens == want.tokens[:len(got.tokens)]
+        if got.reason == StopReason.Cancelled:
+            assert rid in from_outside or limit is not None
+        else:
+            assert (got.tokens, got.text, got.reason) == (want.tokens, want.text, want.reason)
+    sched.assert_idle()
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed):
     """Random prompts, output lengths, pool sizes, batch caps, token budgets, portion sizes and arrival times
