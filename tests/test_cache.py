@@ -333,3 +333,15 @@ def test_random_orders_lose_nothing(seed):
         assert group.allocator.free_count() == group.allocator.capacity()
     with pytest.raises(KeyError):
         manager.release(0)
+
+
+def test_a_pool_the_kernels_cannot_address_is_refused_when_it_is_made():
+    """The attention kernels count a layer's key elements with 32 bits: a pool beyond that is refused with the
+    number of pages that would fit, before anything is allocated."""
+    import torch
+    from tokenizer_amd.cache.pools import CachePools
+    need = CacheNeed("full", 2, 64)                      # 2 kv heads of 64: 2,048 elements a page of 16
+    fits = 2 ** 31 // 2048 - 1
+    CachePools(CacheManager([need], num_pages=fits, page_size=P, max_requests=1), [need], torch.bfloat16, "meta")
+    with pytest.raises(ValueError, match=f"at most {fits} pages"):
+        CachePools(CacheManager([need], num_pages=fits + 1, page_size=P, max_requests=1), [need], torch.bfloat16, "meta")

@@ -19,6 +19,12 @@ class CachePools:
         self.pages = []
         for group in manager.groups:
             need = group.need
+            per_layer = manager.num_pages * need.n_kv_heads * manager.page_size * need.head_dim
+            if per_layer >= 2 ** 31:
+                # The attention kernels count a layer's keys (and its values) with 32 bits.
+                raise ValueError(f"{manager.num_pages} pages of {manager.page_size} tokens are {per_layer} key elements "
+                                 f"a layer; the kernels address fewer than 2^31 (at most "
+                                 f"{(2 ** 31 - 1) // (need.n_kv_heads * manager.page_size * need.head_dim)} pages here)")
             self.pages.append(torch.zeros((len(group.layers), 2, manager.num_pages, need.n_kv_heads,
                                            manager.page_size * need.head_dim), dtype=dtype, device=device))
         self.states = {}
