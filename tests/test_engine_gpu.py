@@ -651,6 +651,70 @@ def test_sizes_away_from_every_tile(tmp_path, size):
                 close(got[rid], want[rid], dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_like_layers_make_the_recorded_calls_of_the_first_again(model_folders, name, dtype):
+    """Eager steps record the library calls of one layer and make them again for the like layers after it, with
+    their weights' and pages' addresses put in place.  The logits equal, bit for bit, those of an engine whose
+    layers all run their own Python: mixed batches with reused pages, and decode steps (whose fused layers hand
+    nothing on, so the first layer already serves the rest).  Configuration C has a full layer and three with a
+    window: the second layer is the one that is recorded for the two after it."""
+    reqs = requests_for(name)
+    n_layers = TINY[name][0]["num_hidden_layers"]
+    for steps in (tt.mixed(reqs, 9), tt.decode_tail(reqs, 12)):
+        logits, repeated = [], []
+        for repeat in (True, False):
+            eng = engine_for(model_folders[name], dtype, max_tokens=tt.peak_tokens(steps), max_requests=4,
+                             use_graphs=False)
+            eng.model.decoder.repeat_layers = repeat
+            eng.pools.poison()
+            logits.append(tt.run_in_process(eng, steps))
+            repeated.append(eng.model.decoder.layers_repeated)
+        for rid in reqs:
+            assert torch.equal(logits[0][rid], logits[1][rid]), rid
+        assert repeated[1] == 0
+        # Every step repeats the layers behind the recorded one of each make: all but two (the first hands on what
+        # it was not handed), or all but one where a layer hands nothing on.
+        assert repeated[0] >= len(steps) * (n_layers - 2)
+
+
+def test_a_layer_named_twice_and_a_layer_on_anothers_pages_are_repeated_rightly(tmp_path):
+    """The order of layers is data: a schedule that runs a layer twice and lets a layer read another layer's pages
+    (without writing) gives the same logits whether the like layers repeat recorded calls or run on their own."""
+    import dataclasses
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config, register_architecture, registered_architectures
+    from tokenizer_amd.models.qwen2 import qwen2_spec
+    from tokenizer_amd.parts.spec import ScheduleEntry
+
+    class TwiceConfig(Qwen2Config):
+        pass
+
+    def twice_spec(cfg):
+        spec = qwen2_spec(cfg)
+        order = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2), ScheduleEntry(1), ScheduleEntry(3),
+                 ScheduleEntry(2, cache_of=3), ScheduleEntry(3, cache_of=3), ScheduleEntry(1))
+        return dataclasses.replace(spec, architecture="TwiceQwen2ForCausalLM", schedule=order)
+
+    if "TwiceQwen2ForCausalLM" not in registered_architectures():
+        register_architecture("TwiceQwen2ForCausalLM", TwiceConfig, twice_spec)
+    raw = dict(TINY["B"][0], architectures=["TwiceQwen2ForCausalLM"], num_hidden_layers=4, max_window_layers=4)
+    folder = ta.write_random_model(TwiceConfig.from_dict(raw), 3, str(tmp_path / "twice"), norm_spread=0.3)
+    reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 70 + i) for i, n in enumerate([40, 7, 90, 33])}
+    for dtype in ("float32", "bfloat16"):
+        steps = tt.mixed(reqs, 2)
+        got = []
+        for repeat in (True, False):
+            eng = engine_for(folder, dtype, max_tokens=tt.peak_tokens(steps), max_requests=4, use_graphs=False)
+            eng.model.decoder.repeat_layers = repeat
+            eng.pools.poison()
+            got.append(tt.run_in_process(eng, steps))
+            assert (eng.model.decoder.layers_repeated > 0) == repeat
+        for rid in reqs:
+            assert torch.equal(got[0][rid], got[1][rid]), rid
+            assert torch.isfinite(got[0][rid]).all()
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_random_configurations_pages_and_traces(tmp_path, seed):
     """Configurations drawn at random (head sizes in steps of 16, any number of heads and groups, inner widths and

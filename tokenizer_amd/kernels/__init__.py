@@ -6,6 +6,7 @@ layout its kernel and grid assume, and launches on torch's current stream.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import math
 import threading
@@ -33,7 +34,12 @@ def _raw_stream(device_index: int) -> int:
     return torch._C._cuda_getCurrentRawStream(device_index)
 
 
+_KEEP: list | None = None      # while a layer's calls are recorded: every tensor whose address went into one
+
+
 def _ptr(tensor: torch.Tensor | None) -> ctypes.c_void_p:
+    if _KEEP is not None and tensor is not None:
+        _KEEP.append(tensor)
     return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
 
 
@@ -72,6 +78,52 @@ class PendingSum:
         self.ops._check(self.ops.lib.ta_splitk_reduce(_ptr(self.partial), _ptr(self.bias), _ptr(out), m, n, n, parts,
                                                       _code(self.dtype), self.ops._stream()), "splitk_reduce")
         return out
+
+
+class LaunchTape:
+    """The library calls that one layer made, in order, each with its arguments and the status it returned.
+
+    Layers of the same make (the same parts with the same sizes and constants) make the same calls on a step's
+    batch; only the addresses of their own tensors differ.  `replay(put)` makes the calls again with every
+    address found in `put` replaced: the Python between the calls (checks, choices of kernel and split, buffers)
+    ran once, for the recorded layer.  The tape keeps every tensor whose address it holds, so the recorded
+    layer's buffers are there for the layers that use them again (all on one stream, one after another).
+    """
+
+    def __init__(self):
+        self.calls: list[tuple] = []          # (function, arguments, status, ((index, address), ...))
+        self.keep: list[torch.Tensor] = []
+
+    def replay(self, put: dict[int, int]) -> None:
+        for function, args, status, addresses in self.calls:
+            changed = None
+            for index, address in addresses:
+                to = put.get(address)
+                if to is not None:
+                    if changed is None:
+                        changed = list(args)
+                    changed[index] = ctypes.c_void_p(to)
+            got = function(*args) if changed is None else function(*changed)
+            if got != status:
+                raise KernelError(f"a recorded call returned {got} where it had returned {status}")
+
+
+class _RecordingLibrary:
+    """Stands in for the loaded library while a tape is recorded: every call goes through and onto the tape."""
+
+    def __init__(self, lib, tape: LaunchTape):
+        self._lib, self._tape = lib, tape
+
+    def __getattr__(self, name):
+        function = getattr(self._lib, name)
+        calls = self._tape.calls
+
+        def call(*args):
+            status = function(*args)
+            calls.append((function, args, status,
+                          tuple((i, a.value) for i, a in enumerate(args) if isinstance(a, ctypes.c_void_p) and a.value)))
+            return status
+        return call
 
 
 class Ops:
@@ -114,6 +166,18 @@ class Ops:
         if status != 0:
             raise KernelError(f"{what} failed with status {status}"
                               + (" (sizes the kernel does not take)" if status < 0 else " (HIP error)"))
+
+    @contextlib.contextmanager
+    def record_launches(self):
+        """Record every library call made inside the block on a `LaunchTape` (which the block receives)."""
+        global _KEEP
+        tape = LaunchTape()
+        library, keep = self.lib, _KEEP
+        self.lib, _KEEP = _RecordingLibrary(library, tape), tape.keep
+        try:
+            yield tape
+        finally:
+            self.lib, _KEEP = library, keep
 
     # ------------------------------------------------------------------ embedding
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

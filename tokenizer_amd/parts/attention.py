@@ -6,7 +6,7 @@ import math
 import torch
 
 from .base import can_fuse_decode as _can_fuse
-from .base import MIXERS, POSITIONS, Mixer, Runtime
+from .base import MIXERS, POSITIONS, Mixer, Repeatable, Runtime, repeatable_of
 from .spec import CacheNeed, MixerSpec, PositionSpec, TensorSpec
 
 
@@ -58,6 +58,13 @@ class GQAttention(Mixer):
     def cache_need(spec: MixerSpec) -> CacheNeed:
         kind = "full" if spec.window is None else "window"
         return CacheNeed(kind=kind, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window)
+
+    def repeatable(self):
+        position = repeatable_of(self.position)
+        if position is None:
+            return None
+        return Repeatable(("gqa_attention", self.n_q, self.n_kv, self.d, self.scale, self.window, position.constants),
+                          (self.w_qkv, self.b_qkv, self.w_o, self.b_o) + position.tensors)
 
     def forward_normed(self, residual, delta, norm, ctx, cache):
         """Decode batches of few bfloat16 rows: norm + q/k/v product + bias + rotation + cache write in one

@@ -27,6 +27,12 @@ FeedForward     tensor_specs(spec); forward(x [T, H], ctx) -> [T, H]; optional f
 Block           arranges two norms, a mixer and a feed-forward around the residual stream (either sub-layer may
                 be absent: None for the part and its norm):
                 forward(residual, delta, ctx, cache) -> delta still to be added.
+
+Every part may also say `repeatable() -> Repeatable` (a block: `repeatable(cache)`): that on the device its forward
+does nothing but call the kernel library, and that those calls depend on the part only through the constants and the
+tensors it lists.  The model then records the calls of one such layer on a step's batch and makes them again for
+the like layers after it, with their tensors' addresses put in place (`kernels.LaunchTape`), instead of running
+their Python.  The promise is the class's own: a subclass does not inherit it and has to give it again.
 """
 from __future__ import annotations
 
@@ -105,6 +111,24 @@ class StoreEpilogue:
     `cos_sin` None meaning no rotation, and write keys and values into their pages.  A position encoding that is
     of that form says so through `PositionEncoding.epilogue()`."""
     cos_sin: torch.Tensor | None
+
+
+@dataclasses.dataclass(frozen=True)
+class Repeatable:
+    """What a part's library calls depend on: `constants` (hashable; parts whose constants are equal make the same
+    calls) and `tensors` (their addresses are what differs from one such part to the next; None where a part has
+    none, the same places in every like part)."""
+    constants: tuple
+    tensors: tuple
+
+
+def repeatable_of(part, *args) -> Repeatable | None:
+    """The part's `repeatable(*args)` if its own class gives that promise, else None."""
+    if part is None:
+        return Repeatable(("absent",), ())
+    if "repeatable" not in vars(type(part)):
+        return None
+    return part.repeatable(*args)
 
 
 class Norm(Part):

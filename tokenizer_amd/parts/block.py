@@ -1,7 +1,7 @@
 """Arrangements of norms, mixer and feed-forward around the residual stream."""
 from __future__ import annotations
 
-from .base import BLOCKS, Block
+from .base import BLOCKS, Block, Repeatable, repeatable_of
 
 
 @BLOCKS.register("pre_norm")
@@ -18,6 +18,14 @@ class PreNormBlock(Block):
     def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
         self.mixer_norm, self.mixer = mixer_norm, mixer
         self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+
+    def repeatable(self, cache):
+        """The layer's library calls depend on its four parts and on which pages it reads and writes."""
+        parts = [repeatable_of(part) for part in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)]
+        if any(part is None for part in parts) or cache.state is not None:
+            return None
+        return Repeatable(("pre_norm", cache.group, cache.writes) + tuple(part.constants for part in parts),
+                          sum((part.tensors for part in parts), ()) + (cache.k_pages, cache.v_pages))
 
     def forward(self, residual, delta, ctx, cache):
         if self.mixer is not None:

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from .base import can_fuse_decode as _can_fuse
-from .base import FEED_FORWARDS, FeedForward, Runtime
+from .base import FEED_FORWARDS, FeedForward, Repeatable, Runtime
 from .spec import FeedForwardSpec, TensorSpec
 
 
@@ -39,6 +39,9 @@ class GatedDense(FeedForward):
         return {"gate_proj.weight": TensorSpec((spec.intermediate_size, spec.hidden_size)),
                 "up_proj.weight": TensorSpec((spec.intermediate_size, spec.hidden_size)),
                 "down_proj.weight": TensorSpec((spec.hidden_size, spec.intermediate_size))}
+
+    def repeatable(self):
+        return Repeatable(("gated_dense",), (self.w_gate_up, self.w_down))
 
     def forward_normed(self, residual, delta, norm, ctx):
         """Decode batches of few bfloat16 rows: norm + gate/up product + activation in one kernel, then the

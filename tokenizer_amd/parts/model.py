@@ -5,7 +5,7 @@ import dataclasses
 
 import torch
 
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Runtime
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Runtime, repeatable_of
 from .spec import CacheNeed, ModelSpec, TensorSpec
 
 
@@ -52,6 +52,42 @@ class LayerCache:
     writes: bool = True                     # False when the layer reads another layer's cache
 
 
+class _Make:
+    """What one scheduled layer's library calls depend on: `key` (layers with equal keys make the same calls) and the
+    addresses of its tensors, in the order in which every layer of that key lists them."""
+
+    def __init__(self, constants: tuple, tensors: tuple):
+        # (Strides and alignment too: the recorded layer's tensors passed the wrappers' checks, a like layer's must
+        # be laid out the same way to pass them unseen.)
+        self.key = (constants, tuple(None if t is None else (tuple(t.shape), t.dtype, t.stride(), t.data_ptr() % 16)
+                                     for t in tensors))
+        self.addresses = tuple(0 if t is None else t.data_ptr() for t in tensors)
+        self.tensors = tensors                 # kept, so the addresses stay theirs
+
+
+def _coming(delta):
+    """What a layer is handed besides the stream: (a word for its form, the addresses a library call would be given).
+    Forms this module does not know make the layer run on its own."""
+    if delta is None:
+        return "none", ()
+    if isinstance(delta, torch.Tensor):
+        return ("tensor", tuple(delta.shape), delta.dtype, delta.is_contiguous()), (delta.data_ptr(),)
+    partial, bias = getattr(delta, "partial", None), getattr(delta, "bias", None)
+    if isinstance(partial, torch.Tensor) and bias is None:
+        return ("parts", tuple(partial.shape), getattr(delta, "dtype", None)), (partial.data_ptr(),)
+    return None, ()
+
+
+def _addresses_put(recorded: tuple, wanted: tuple):
+    """The map from the recorded layer's addresses to another layer's, or False if one address would have to stand
+    for two."""
+    put: dict[int, int] = {}
+    for a, b in zip(recorded, wanted):
+        if put.setdefault(a, b) != b:
+            return False
+    return {a: b for a, b in put.items() if a != b}
+
+
 class DecoderModel:
     """Weights and parts of one model.  It owns no cache: `forward` is handed the step's context
     (token ids, positions, block tables) and one `LayerCache` per schedule entry."""
@@ -78,6 +114,18 @@ class DecoderModel:
                                      if p is not None]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in parts) and \
             all(hasattr(b, "mixer") for b in self.blocks)
+        self.repeat_layers = True      # record one layer's library calls and make them again for the like ones
+        self.layers_repeated = 0       # how many scheduled layers have run that way so far
+        self._put: dict[tuple[int, int], dict[int, int]] = {}
+
+    def _make_of(self, block, layer: int, cache: "LayerCache"):
+        """The make of a scheduled layer on this cache, or None if the block does not promise to be repeatable.
+        Worked out once and kept on the cache entry."""
+        makes = cache.__dict__.setdefault("_makes", {})
+        if layer not in makes:
+            said = repeatable_of(block, cache)
+            makes[layer] = None if said is None else _Make(said.constants, said.tensors)
+        return makes[layer]
 
     def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
         """Run the tokens of `ctx` through the schedule; float32 logits [len(want_rows), vocab]."""
@@ -85,8 +133,40 @@ class DecoderModel:
         residual = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.runtime.device)
         ops.embedding(ctx.token_ids, self.embedding, residual)
         delta = None
+        # Like layers make the same library calls on a batch: the calls of the first are recorded and made again
+        # for the others with their tensors' addresses put in place, which spares those layers' Python (about
+        # two thirds of an eager step's host time; a step of a small model is bound by it).  Not while a graph
+        # is recorded or warmed up: that happens once, and the library times its products there.
+        record = getattr(ops, "record_launches", None) if self.repeat_layers and not getattr(ops, "capturing", False) else None
+        tapes: dict = {}
         for entry, cache in zip(self.spec.schedule, layer_caches):
-            delta = self.blocks[entry.layer].forward(residual, delta, ctx, cache)
+            block = self.blocks[entry.layer]
+            make = self._make_of(block, entry.layer, cache) if record is not None else None
+            form, addresses = _coming(delta) if make is not None else (None, ())
+            if form is None:
+                delta = block.forward(residual, delta, ctx, cache)
+                continue
+            tape = tapes.get((make.key, form))
+            if tape is None:
+                with record() as tape:
+                    out = block.forward(residual, delta, ctx, cache)
+                if _coming(out)[0] == form:       # what it hands on looks like what it was handed: it can follow itself
+                    tape.make, tape.coming, tape.result = make, addresses, out
+                    tapes[(make.key, form)] = tape
+                delta = out
+                continue
+            put = self._put.get((id(tape.make), id(make)))
+            if put is None:
+                put = self._put[(id(tape.make), id(make))] = _addresses_put(tape.make.addresses, make.addresses)
+            if put is False:                      # one tensor in two places there, two tensors here: no single map
+                delta = block.forward(residual, delta, ctx, cache)
+                continue
+            if addresses != tape.coming:
+                put = dict(put)
+                put.update(zip(tape.coming, addresses))
+            tape.replay(put)
+            self.layers_repeated += 1
+            delta = tape.result                   # the recorded layer's buffers hold this layer's output now
         if ctx.want_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.runtime.device)
         # Only the wanted rows are normalised and multiplied with the head (the reference keeps

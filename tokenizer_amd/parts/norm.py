@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import NORMS, Norm, NormFold, Runtime
+from .base import NORMS, Norm, NormFold, Repeatable, Runtime
 from .spec import NormSpec, TensorSpec
 
 
@@ -24,6 +24,9 @@ class RMSNorm(Norm):
 
     def fold(self):
         return NormFold(self.weight, self.eps)
+
+    def repeatable(self):
+        return Repeatable(("rmsnorm", self.size, self.eps), (self.weight,))
 
     def apply(self, residual, delta, rows=None):
         n_rows = residual.shape[0] if rows is None else rows.numel()

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import POSITIONS, PositionEncoding, Runtime, StoreEpilogue
+from .base import POSITIONS, PositionEncoding, Repeatable, Runtime, StoreEpilogue
 from .spec import PositionSpec
 
 
@@ -18,6 +18,9 @@ class NoPosition(PositionEncoding):
 
     def table(self):
         return None
+
+    def repeatable(self):
+        return Repeatable(("none",), ())
 
     def epilogue(self):
         # A subclass that encodes in its own way inherits this method but not the promise: it has to offer an
@@ -61,3 +64,6 @@ class RotaryHalfSplit(NoPosition):
 
     def table(self):
         return self.cos_sin
+
+    def repeatable(self):
+        return Repeatable(("rope_half_split", self.max_positions), (self.cos_sin,))
