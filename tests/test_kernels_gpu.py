@@ -4,6 +4,8 @@ import math
 import pytest
 import torch
 
+from tokenizer_amd.kernels import PendingSum
+
 from kernel_refs import PlainOps
 
 pytestmark = pytest.mark.gpu
@@ -479,6 +481,42 @@ def test_linear_with_k_cut_over_workgroups(ops, ref, shape, monkeypatch):
             torch.testing.assert_close(got.double(), want, **linear_tol(out_dtype, x, w))
             again = ops.linear(x, w, bias if use_bias else None, out_dtype=out_dtype)
             assert torch.equal(got, again)
+
+
+@pytest.mark.parametrize("shape", [(137, 896, 4864), (65, 100, 2056), (256, 1536, 8960), (100, 896, 896), (200, 60, 776)])
+def test_linear_of_a_few_hundred_rows_with_k_cut(ops, ref, shape, monkeypatch):
+    """65 to 256 rows (a portion of a prompt beside decoded tokens) and few output tiles: K is cut where the parts
+    may stay for the next norm (long K: recorded or not; shorter K: when launched eagerly, where small products
+    do not go to the library), or into four parts that the kernel adds itself.  The same product either way, the
+    same on every run; the parts, added, are the product too."""
+    m, n, k = shape
+    x = rand((m, k), torch.bfloat16, 34)
+    w = rand((n, k), torch.bfloat16, 35, 0.1)
+    bias = rand((n,), torch.float32, 36)
+    want = ref.linear(x, w, bias, out_dtype=torch.float64)
+    for capturing in (False, True):
+        monkeypatch.setattr(ops, "capturing", capturing)
+        expect_parts = k >= 2048 or (not capturing and k >= 768)
+        assert (ops._k_splits(m, n, k, True) > 1) == expect_parts
+        assert (ops._k_splits(m, n, k, False) > 1) == (not capturing and k >= 2048 and m * n * k < ops.EAGER_LIBRARY_WORK)
+        left = ops.linear(x, w, bias, pending=True)
+        assert isinstance(left, PendingSum) == expect_parts
+        got = left.resolve() if expect_parts else left
+        torch.testing.assert_close(got.double(), want, **linear_tol(torch.bfloat16, x, w))
+        added = ops.linear(x, w, bias)
+        torch.testing.assert_close(added.double(), want, **linear_tol(torch.bfloat16, x, w))
+        assert torch.equal(added, ops.linear(x, w, bias))
+        if expect_parts:
+            # The parts go into the norm that follows as they are: sum + bias + residual, then the norm.
+            residual = rand((m, n), torch.float32, 37)
+            weight = rand((n,), torch.float32, 38).abs() + 0.5
+            out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+            stream = residual.clone()
+            ops.add_rmsnorm(stream, left, weight, 1e-6, out)
+            total = residual.double() + want
+            torch.testing.assert_close(stream.double(), total, rtol=1e-5, atol=linear_tol(torch.float32, x, w)["atol"])
+            normed = total / (total.pow(2).mean(dim=1, keepdim=True) + 1e-6).sqrt() * weight.double()
+            torch.testing.assert_close(out.double(), normed, rtol=1e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("shape", [(40, 200, 2304), (64, 96, 4864), (17, 1028, 2048), (33, 64, 2056), (20, 52, 4104)])

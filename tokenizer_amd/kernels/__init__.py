@@ -428,7 +428,7 @@ class Ops:
                     _ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(None if leave else out), n, _ptr(partial), m, n, k,
                     _code(out_dtype), streaming_splits, self.skinny_column_blocks, self._stream()), "linear")
                 return PendingSum(self, partial, bias, out_dtype) if leave else out
-            splits = self._k_splits(m, n, k)
+            splits = self._k_splits(m, n, k, pending)
             if splits > 1:
                 # The same with the tiled kernel.
                 parts = _parts_of_k(k, splits, 64)
@@ -479,12 +479,31 @@ class Ops:
     use_split_k = True
     skinny_column_blocks = 0   # blocks of sixteen output columns per workgroup of the weight-streaming kernel: 0 = its choice
 
-    def _k_splits(self, m: int, n: int, k: int) -> int:
-        """Into how many parts the tiled kernel cuts K: more than one for 17 to 64 rows with a K so long, and so
-        few output tiles of 64 x 64, that the library (which cuts K as well) falls behind."""
-        if not self.use_split_k or not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or k < self.SPLIT_K_FROM or n % 4:
+    def _k_splits(self, m: int, n: int, k: int, pending: bool = False) -> int:
+        """Into how many parts the tiled kernel cuts K.  17 to 64 rows: more than one with a K so long, and so few
+        output tiles of 64 x 64, that the library (which cuts K as well) falls behind.  65 to 256 rows (portions of
+        prompts beside decoded tokens): few tiles again, far fewer than compute units, and a whole K for each is
+        a long walk (137 rows x 896 columns over a K of 4,864: 32 us in one piece).  Where the parts may be left
+        for the norm that follows (`pending`) and K is 2,048 or more, eight parts beat the library as well (the same
+        product: 10 us against 10 us; 137 x 1,536 over 8,960: 17 us against 23 us).  Launched eagerly, small
+        products do not go to the library at all (its launch costs the host more than they take): those are cut
+        whenever K allows, into parts for the next norm or, with a long K, into four that the kernel adds itself
+        (14 us)."""
+        if not self.use_split_k or n % 4:
             return 1
         tiles = -(-m // 64) * -(-n // 64)
+        if self.SKINNY_ROWS < m <= 256:
+            if tiles >= 128:
+                return 1
+            if pending and k >= 2048:
+                return min(8, k // 512)
+            if self.capturing or m * n * k >= self.EAGER_LIBRARY_WORK:
+                return 1                   # the library's
+            if pending and k >= 768:
+                return min(8, k // 384)
+            return 4 if k >= 2048 else 1
+        if not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or k < self.SPLIT_K_FROM:
+            return 1
         if tiles >= 256:
             return 1
         return max(1, min(-(-512 // tiles), k // 256))
