@@ -7,9 +7,9 @@ random ids and decodes every request on to 4,096 tokens (8 warm-up steps, 2,040 
 also times a prefill of 2,048 tokens and the same decoding at batch 1 and 64, and prints one
 JSON line.
 
-    python bench.py --workload mixed-1.5b | prefix-7b
+    python bench.py --workload mixed-1.5b | mixed-0.5b | prefix-7b [--token-budget N]
 
-runs a whole serving workload through the scheduler instead (64 requests at Qwen2.5-1.5B sizes
+runs a whole serving workload through the scheduler instead (64 requests at Qwen2.5-1.5B or 0.5B sizes
 with prompts of 128 to 2,048 ids and 256 new tokens each; 64 requests at Qwen2.5-7B sizes that
 share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for it.
 
@@ -155,7 +155,7 @@ def run_prefill(model, repeats: int = 7):
     return best
 
 
-def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0) -> dict:
+def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0, token_budget: int = 2048) -> dict:
     """A serving workload through the scheduler: every request is admitted, its prompt cut into portions under
     the token budget beside the others' decode tokens, decoded greedily to its length, and freed."""
     import numpy as np
@@ -164,8 +164,8 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
     from tokenizer_amd.engine import Engine, GenerateParams, Generated, Scheduler, SchedulerConfig, random_model
 
     rng = np.random.default_rng(7)
-    if name == "mixed-1.5b":
-        raw, new_tokens, prefix_cache = QWEN2_1_5B, 256, False
+    if name in ("mixed-1.5b", "mixed-0.5b"):
+        raw, new_tokens, prefix_cache = (QWEN2_1_5B if name == "mixed-1.5b" else QWEN2_0_5B), 256, False
         lengths = [int(n) for n in rng.integers(128, 2049, size=64)]
         prompts = [[int(t) for t in rng.integers(0, raw["vocab_size"], size=n)] for n in lengths]
     elif name == "prefix-7b":
@@ -183,7 +183,7 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
     log(f"{name}: {len(prompts)} requests, {sum(len(p) for p in prompts)} prompt tokens, {new_tokens} new tokens each")
     for attempt in ("warm-up", "timed"):        # the first pass captures the decode graphs and warms the library
         sched = Scheduler(engine, SchedulerConfig(max_batch_size=64, max_waiting=64, num_blocks=pages,
-                                                  prefix_cache=prefix_cache, max_num_batched_tokens=2048))
+                                                  prefix_cache=prefix_cache, max_num_batched_tokens=token_budget))
         torch.cuda.synchronize()
         started = time.perf_counter()
         params = lambda i: (GenerateParams.greedy(new_tokens) if temperature == 0 else
@@ -208,7 +208,7 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
                        "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                        "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                        "requests": len(prompts), "prompt_tokens": sum(len(p) for p in prompts),
-                       "new_tokens_each": new_tokens, "token_budget": 2048, "prefix_cache": prefix_cache,
+                       "new_tokens_each": new_tokens, "token_budget": token_budget, "prefix_cache": prefix_cache,
                        "pages": pages, "page_size": 16, "temperature": temperature},
             "scheduler": {"steps": stats.steps, "tokens_forwarded": stats.tokens_forwarded, "max_running": stats.max_running,
                           "preemptions": stats.preemptions, "peak_pages": stats.peak_blocks,
@@ -303,7 +303,7 @@ def main() -> int:
     parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
                         help="layer sizes of the decode benchmark (the default is the one the record is for)")
     parser.add_argument("--peaks", action="store_true", help="measure what the device reaches in HBM reads and bf16 products")
-    parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "prefix-7b"],
+    parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "mixed-0.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
@@ -312,6 +312,8 @@ def main() -> int:
     parser.add_argument("--cached", type=int, default=0, help="with --attention: tokens already in the cache")
     parser.add_argument("--attention-kernel", default="auto", choices=["auto", "per-wave", "shared"],
                         help="with --attention: the launcher's choice, or one of the two prompt kernels")
+    parser.add_argument("--token-budget", type=int, default=2048,
+                        help="with --workload: the most tokens a step of the scheduler may hold")
     parser.add_argument("--temperature", type=float, default=0.0,
                         help="with --workload: draw with this temperature and top_p 0.95 instead of greedy picks")
     parser.add_argument("--prompt-len", type=int, default=None,
@@ -334,7 +336,7 @@ def main() -> int:
         print(json.dumps(measure_peaks()), flush=True)
         return 0
     if args.workload:
-        print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature)), flush=True)
+        print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature, args.token_budget)), flush=True)
         return 0
     sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
     if args.attention:
