@@ -295,7 +295,8 @@ static int planned_reach(int max_keys, int window) {
   return (window >= 0 && window + 16 < planned) ? window + 16 : planned;
 }
 
-// waves: waves per tile (1, 2 or 4); 0 = by the longest reach of a token: one wave per 256 keys or so.
+// waves: waves per tile (1, 2, 4, or 8 at head sizes 48 and 64); 0 = by the longest reach of a token: one wave per
+// 256 keys or so, eight for few tiles with a long reach.
 template <int D, int HG>
 static int launch_prefill(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
                           const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
@@ -304,12 +305,21 @@ static int launch_prefill(const void* q, int q_stride, void* out, const void* k_
   if (waves == 0) {
     const int reach = planned_reach(max_keys, window);
     waves = reach > 768 ? 4 : reach > 256 ? 2 : 1;
+    // A short portion behind a long cached context: a handful of tiles, each with thousands of keys to walk and a
+    // SIMD to itself, so that nothing hides a block's trip to memory.  Eight waves halve each wave's walk (512
+    // tokens of 14 / 2 heads of 64 behind 8,192: 64 -> 56 us; behind 30,000: 240 -> 161 us; 256 behind 8,192:
+    // 58 -> 49 us); from 1,024 tokens on, where the waves crowd the compute units, they are slower (89 -> 109 us).
+    const long workgroups = (long)n_tiles * n_kv * ((n_q / n_kv + HG - 1) / HG);
+    if ((D == 48 || D == 64) && reach >= 4096 && workgroups <= 256) waves = 8;
     // Head sizes above 64 need so many registers that a SIMD holds one wave: two workgroups of two waves fill a
     // compute unit better than one of four (measured at head sizes 96, 128 and 256, 512 to 8,192 tokens).
     if (D > 64 && waves > 2) waves = 2;
   }
 #define GO(NWV) launch_prefill_waves<D, HG, NWV>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream)
+  if constexpr (D == 48 || D == 64) {          // (the eight waves' states fit the static LDS at these sizes)
+    if (waves >= 8) return GO(8);
+  }
   if (waves >= 4) return GO(4);
   if (waves >= 2) return GO(2);
   return GO(1);
@@ -330,7 +340,7 @@ extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, voi
 // shared: 1 = the workgroup-shared kernel wherever it has an instance (in the shape `shared_shape` names: 1 or 2
 // heads a wave, + 10 for two key groups; 0 = its own choice), -1 = never, 0 = where it is the faster one (by the shape of the launch and the planned
 // reach, so that a launch recorded for a range of contexts and a launch for the exact context make the same
-// choice).  waves: waves that share a tile's keys in the per-wave kernel (1, 2, 4; 0 = by the reach); asking
+// choice).  waves: waves that share a tile's keys in the per-wave kernel (1, 2, 4, 8; 0 = by the reach); asking
 // for a number asks for that kernel.
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
