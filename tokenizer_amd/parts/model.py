@@ -50,6 +50,7 @@ class LayerCache:
     v_pages: torch.Tensor | None = None
     state: torch.Tensor | None = None       # [n_slots, *state_shape]
     writes: bool = True                     # False when the layer reads another layer's cache
+    makes: dict = dataclasses.field(default_factory=dict, repr=False, compare=False)   # what the layers run on it depend on
 
 
 class _Make:
@@ -63,6 +64,15 @@ class _Make:
                                      for t in tensors))
         self.addresses = tuple(0 if t is None else t.data_ptr() for t in tensors)
         self.tensors = tensors                 # kept, so the addresses stay theirs
+
+
+@dataclasses.dataclass
+class _Recorded:
+    """One layer's library calls on this step's batch, with what they were recorded for."""
+    tape: object                  # kernels.LaunchTape
+    make: _Make
+    coming: tuple                 # the addresses of what the layer was handed
+    result: object                # what it handed on (its buffers serve every layer that repeats the calls)
 
 
 def _coming(delta):
@@ -121,11 +131,10 @@ class DecoderModel:
     def _make_of(self, block, layer: int, cache: "LayerCache"):
         """The make of a scheduled layer on this cache, or None if the block does not promise to be repeatable.
         Worked out once and kept on the cache entry."""
-        makes = cache.__dict__.setdefault("_makes", {})
-        if layer not in makes:
+        if layer not in cache.makes:
             said = repeatable_of(block, cache)
-            makes[layer] = None if said is None else _Make(said.constants, said.tensors)
-        return makes[layer]
+            cache.makes[layer] = None if said is None else _Make(said.constants, said.tensors)
+        return cache.makes[layer]
 
     def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
         """Run the tokens of `ctx` through the schedule; float32 logits [len(want_rows), vocab]."""
@@ -146,27 +155,26 @@ class DecoderModel:
             if form is None:
                 delta = block.forward(residual, delta, ctx, cache)
                 continue
-            tape = tapes.get((make.key, form))
-            if tape is None:
+            recorded = tapes.get((make.key, form))
+            if recorded is None:
                 with record() as tape:
                     out = block.forward(residual, delta, ctx, cache)
                 if _coming(out)[0] == form:       # what it hands on looks like what it was handed: it can follow itself
-                    tape.make, tape.coming, tape.result = make, addresses, out
-                    tapes[(make.key, form)] = tape
+                    tapes[(make.key, form)] = _Recorded(tape, make, addresses, out)
                 delta = out
                 continue
-            put = self._put.get((id(tape.make), id(make)))
+            put = self._put.get((id(recorded.make), id(make)))
             if put is None:
-                put = self._put[(id(tape.make), id(make))] = _addresses_put(tape.make.addresses, make.addresses)
+                put = self._put[(id(recorded.make), id(make))] = _addresses_put(recorded.make.addresses, make.addresses)
             if put is False:                      # one tensor in two places there, two tensors here: no single map
                 delta = block.forward(residual, delta, ctx, cache)
                 continue
-            if addresses != tape.coming:
+            if addresses != recorded.coming:
                 put = dict(put)
-                put.update(zip(tape.coming, addresses))
-            tape.replay(put)
+                put.update(zip(recorded.coming, addresses))
+            recorded.tape.replay(put)
             self.layers_repeated += 1
-            delta = tape.result                   # the recorded layer's buffers hold this layer's output now
+            delta = recorded.result               # the recorded layer's buffers hold this layer's output now
         if ctx.want_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.runtime.device)
         # Only the wanted rows are normalised and multiplied with the head (the reference keeps
