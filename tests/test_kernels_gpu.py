@@ -257,19 +257,19 @@ def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, windo
     torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
 
 
-@pytest.mark.parametrize("window", [None, 5000, 600])
+@pytest.mark.parametrize("window", [None, 600])
 def test_a_short_portion_behind_a_long_context_takes_eight_waves_a_tile(ops, ref, window):
-    """A portion of 200 tokens behind 4,400 cached ones (and a second request's 40 behind 300): few tiles with a
+    """A portion of 70 tokens behind 4,150 cached ones (and a second request's 20 behind 320): few tiles with a
     long walk each, for which the launcher gives a tile eight waves at head size 64 (with a window of 600 nobody
     looks that far back and it stays at fewer).  Keys the waves share out unevenly, waves without a key of their
     own at the short request, unwritten slots holding NaN."""
     n_q, n_kv, d, page_size = 14, 2, 64, 16
-    lengths, q_lens = [4600, 340], [200, 40]
+    lengths, q_lens = [4220, 340], [70, 20]
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=23)
     assert ops.prefill_waves == 0 and ops.prefill_shared == 0
     tiles = sum(-(-n // 16) for n in q_lens)
-    assert ops.lib.ta_prefill_attention_shared_plan(tiles, n_q, n_kv, d, 5120) == 0      # the per-wave kernel's
+    assert ops.lib.ta_prefill_attention_shared_plan(tiles, n_q, n_kv, d, 4608) == 0      # the per-wave kernel's
     out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
     out_b = torch.empty_like(out_a)
     scale = 1.0 / math.sqrt(d)
