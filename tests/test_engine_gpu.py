@@ -208,6 +208,46 @@ def test_long_prompts_with_large_heads_through_the_engine(tmp_path, heads, shape
     eng.cache.check_invariants()
 
 
+@pytest.mark.parametrize("heads", [(28, 4, 128), (14, 2, 64)])
+def test_short_portions_behind_a_long_context_through_the_engine(tmp_path, heads):
+    """A prompt of 3,400 tokens: 3,000 in one step, then equal portions of 64 beside a decoded token of another
+    request.  The portions are a handful of tiles with thousands of keys behind them, whose keys the prompt kernel
+    cuts over workgroups (a second kernel merges the parts); their shape recurs, so the later ones replay a graph
+    with those two kernels in it.  Every portion against the plain implementation, recorded and not."""
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import StepEntry
+    from tokenizer_amd.kernels import get_ops
+    n_q, n_kv, d = heads
+    ops = get_ops()
+    assert ops.lib.ta_prefill_attention_key_splits(4, n_q, n_kv, d, -1, 0, 3100, 0, 0) > 1       # the portions below
+    raw = dict(TINY["A"][0], num_hidden_layers=2, hidden_size=n_q * d, num_attention_heads=n_q, num_key_value_heads=n_kv,
+               intermediate_size=256, vocab_size=300, max_position_embeddings=4096, rope_theta=1000000.0)
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 23, str(tmp_path / "far"), norm_spread=0.3)
+    cfg, tensors = plain.load_folder(folder)
+    a_ids, b_ids = random_ids(300, 3400, 81), random_ids(300, 40, 82)
+    want_a, want_b = plain.all_logits(cfg, tensors, a_ids), plain.all_logits(cfg, tensors, b_ids)
+    got = {}
+    for use_graphs in (True, False):
+        eng = engine_for(folder, "bfloat16", max_tokens=3456 + 64, max_requests=2, use_graphs=use_graphs)
+        eng.pools.poison()
+        eng.add_request("a")
+        eng.add_request("b")
+        eng.step([StepEntry("a", a_ids[:3000], []), StepEntry("b", b_ids[:30], [])])
+        for k in range(6):
+            at = 3000 + 64 * k
+            logits = eng.step([StepEntry("a", a_ids[at:at + 64], [0, 17, 63]), StepEntry("b", b_ids[30 + k:31 + k], [0])])
+            got[use_graphs, k] = logits.float().cpu()
+        if use_graphs:
+            assert any(not isinstance(key[0], int) for key in eng.graphs), "the recurring shape was not captured"
+    for k in range(6):
+        at = 3000 + 64 * k
+        for use_graphs in (True, False):
+            close(got[use_graphs, k][:3], want_a[[at, at + 17, at + 63]], "bfloat16")
+            close(got[use_graphs, k][3:], want_b[[30 + k]], "bfloat16")
+    assert torch.equal(got[True, 0], got[False, 0])          # both eager
+
+
 def test_recorded_steps_with_the_shared_block_prompt_attention(tmp_path):
     """Five prompts of the same length, one after the other, at the 7B model's head shape: the step's shape recurs,
     so the later ones replay a captured graph, in which the prompt attention is the kernel whose waves share their

@@ -257,19 +257,54 @@ def test_prefill_attention_on_long_and_ragged_portions(ops, ref, geometry, windo
     torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
 
 
+@pytest.mark.parametrize("geometry,shape,window", [
+    ((28, 4, 128, 16), 0, None), ((12, 2, 128, 32), 0, None), ((28, 4, 128, 16), 2, None), ((12, 2, 128, 16), 12, None),
+    ((14, 2, 64, 16), 11, None), ((6, 2, 64, 48), 1, None), ((28, 4, 128, 16), 0, 4150), ((14, 2, 64, 16), 11, 4150),
+    ((12, 2, 128, 32), 0, 600), ((6, 2, 64, 48), 1, 600)])
+def test_few_tiles_behind_a_long_context_cut_their_keys_over_workgroups(ops, ref, geometry, shape, window, monkeypatch):
+    """A portion of 70 tokens behind 4,150 cached ones and a second request's 20 behind 320: fewer workgroups than
+    compute units, thousands of keys each.  The workgroup-shared kernel then cuts every tile's keys over several
+    workgroups (whole turns each; the short request's later parts are empty) and a second kernel merges their
+    states.  Every shape of the kernel, a window that reaches nearly as far and one that does not (no cut then);
+    unwritten slots hold NaN."""
+    n_q, n_kv, d, page_size = geometry
+    lengths, q_lens = [4220, 340], [70, 20]
+    qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
+        torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=29)
+    if shape:
+        monkeypatch.setattr(ops, "prefill_shared", 1)
+        monkeypatch.setattr(ops, "prefill_shape", shape)
+    tiles = sum(-(-n // 16) for n in q_lens)
+    parts = ops.lib.ta_prefill_attention_key_splits(tiles, n_q, n_kv, d, -1 if window is None else window,
+                                                    ops.prefill_shape, max(lengths), ops.prefill_waves, ops.prefill_shared)
+    assert (parts > 1) == (window != 600), parts
+    out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
+    out_b = torch.empty_like(out_a)
+    scale = 1.0 / math.sqrt(d)
+    ops.paged_attention(qkv, out_a, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    ref.paged_attention(qkv, out_b, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale)
+    torch.testing.assert_close(out_a.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
+    # The same launch with the keys in one piece: the same attention, up to the order of the sums.
+    monkeypatch.setattr(ops, "prefill_key_splits", False)
+    out_c = torch.full_like(out_a, float("nan"))
+    ops.paged_attention(qkv, out_c, k_pages, v_pages, positions, entry_of_token, table, n_q, n_kv, d, window, scale,
+                        max_position=max(lengths) - 1, batch=make_batch(lengths, q_lens))
+    torch.testing.assert_close(out_c.float(), out_b.float(), **attention_tol(torch.bfloat16, True))
+
+
 @pytest.mark.parametrize("window", [None, 600])
-def test_a_short_portion_behind_a_long_context_takes_eight_waves_a_tile(ops, ref, window):
+def test_a_short_portion_behind_a_long_context_takes_eight_waves_a_tile(ops, ref, window, monkeypatch):
     """A portion of 70 tokens behind 4,150 cached ones (and a second request's 20 behind 320): few tiles with a
-    long walk each, for which the launcher gives a tile eight waves at head size 64 (with a window of 600 nobody
-    looks that far back and it stays at fewer).  Keys the waves share out unevenly, waves without a key of their
+    long walk each, for which the per-wave kernel's launcher gives a tile eight waves at head size 64 (with a window
+    of 600 nobody looks that far back and it stays at fewer).  Keys the waves share out unevenly, waves without a key of their
     own at the short request, unwritten slots holding NaN."""
     n_q, n_kv, d, page_size = 14, 2, 64, 16
     lengths, q_lens = [4220, 340], [70, 20]
     qkv, k_pages, v_pages, positions, entry_of_token, table = make_paged_case(
         torch.bfloat16, n_q, n_kv, d, page_size, lengths=lengths, q_lens=q_lens, seed=23)
-    assert ops.prefill_waves == 0 and ops.prefill_shared == 0
-    tiles = sum(-(-n // 16) for n in q_lens)
-    assert ops.lib.ta_prefill_attention_shared_plan(tiles, n_q, n_kv, d, 4608) == 0      # the per-wave kernel's
+    assert ops.prefill_waves == 0
+    monkeypatch.setattr(ops, "prefill_shared", -1)        # the per-wave kernel (where it has the launch to itself)
     out_a = torch.full((qkv.shape[0], n_q * d), float("nan"), dtype=torch.bfloat16).cuda()
     out_b = torch.empty_like(out_a)
     scale = 1.0 / math.sqrt(d)
@@ -353,9 +388,17 @@ def test_where_the_workgroup_shared_kernel_is_planned(ops):
     assert plan(128, 14, 2, 64, 2048) == 11 and plan(256, 14, 2, 64, 4096) == 11 and plan(512, 14, 2, 64, 8192) == 2
     assert plan(32, 28, 4, 128, 512) == 11 and plan(64, 28, 4, 128, 1024) == 11 and plan(64, 28, 4, 128, 8192) == 12
     assert plan(128, 28, 4, 128, 2048) == 12 and plan(256, 28, 4, 128, 4096) == 2
-    assert plan(31, 28, 4, 128, 8192) == 0
+    assert plan(31, 28, 4, 128, 512) == 0 and plan(31, 28, 4, 128, 1024) == 11      # few tiles: only behind some context ...
+    assert plan(1, 12, 2, 128, 4096) == 11 and plan(8, 32, 8, 128, 8192) == 11 and plan(31, 14, 2, 64, 2560) == 0   # ... at head size 128,
+    assert plan(31, 14, 2, 64, 3072) == 11 and plan(2, 16, 4, 64, 8192) == 11           # behind 3,072 keys and more at head size 64
+    splits = ops.lib.ta_prefill_attention_shared_key_splits
+    # (tiles, query heads, kv heads, reach, shape) -> parts of a tile's keys: fewer workgroups than compute units and a long reach
+    assert splits(8, 28, 4, 8704, 11) == 4 and splits(1, 28, 4, 8704, 11) == 8 and splits(32, 12, 2, 8704, 11) == 2
+    assert splits(32, 28, 4, 8704, 11) == 1 and splits(8, 28, 4, 3584, 11) == 3 and splits(8, 28, 4, 4096, 11) == 4
+    assert splits(8, 28, 4, 2048, 11) == 2 and splits(8, 28, 4, 1536, 11) == 1 and splits(1, 28, 4, 2048, 1) == 4
+    assert splits(2, 28, 4, 30720, 2) == 16 and splits(8, 28, 4, 8704, 0) == 1
     assert plan(128, 12, 2, 128, 2048) == 11 and plan(128, 12, 2, 128, 10240) == 12
-    assert plan(128, 32, 8, 128, 2048) == 1 and plan(64, 32, 8, 128, 1024) == 11 and plan(31, 32, 8, 128, 1024) == 0   # four heads per kv head: one a wave
+    assert plan(128, 32, 8, 128, 2048) == 1 and plan(64, 32, 8, 128, 1024) == 11 and plan(31, 32, 8, 128, 512) == 0   # four heads per kv head: one a wave
     assert plan(128, 16, 4, 64, 2048) == 11 and plan(512, 16, 4, 64, 8192) == 1 and plan(512, 24, 8, 128, 8192) == 1
     assert plan(4096, 16, 8, 128, 8192) == 0        # two heads per kv head
     assert plan(4096, 28, 4, 96, 8192) == 0         # no instance

@@ -241,9 +241,18 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
 // which flush the L2 of every XCD and cost more than this launch.
 __global__ void __launch_bounds__(WAVE)
 decode_attention_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                       const int* __restrict__ rows, bf16_t* __restrict__ out, int n_q, int d, int splits) {
+                       const int* __restrict__ rows, bf16_t* __restrict__ out, int n_q, int d, int splits,
+                       const int* __restrict__ tiles, const int* __restrict__ cu_q) {
   const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
-  const int t = rows ? rows[item] : item;
+  int t = rows ? rows[item] : item;
+  if (tiles) {
+    // Items are (tile, token of the tile): the output row is the tile's first row + the token; a tile's padding
+    // has no row.
+    const int tile = item >> 4, token = item & 15;
+    const int entry = tiles[2 * tile], row0 = cu_q[entry] + tiles[2 * tile + 1];
+    if (token >= cu_q[entry + 1] - row0) return;
+    t = row0 + token;
+  }
   const size_t base = ((size_t)item * n_q + head) * splits;
   const int lane = threadIdx.x, part = lane & 15, grp = lane >> 4;
   const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
@@ -320,10 +329,23 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
   int status = LAUNCH_STATUS();
   if (status == 0 && splits > 1) {
     decode_attention_merge<<<n_items * n_q, 64, 0, stream>>>((const float*)part_o, (const float*)part_ml,
-                                                             (const int*)rows, (bf16_t*)out, n_q, D, splits);
+                                                             (const int*)rows, (bf16_t*)out, n_q, D, splits,
+                                                             nullptr, nullptr);
     status = LAUNCH_STATUS();
   }
   return status;
+}
+
+// The same merge for the prompt kernel whose tiles' keys were cut over workgroups: items are (tile, token of the
+// tile), part_o float [n_tiles * 16, n_q, splits, d], part_ml float [n_tiles * 16, n_q, splits, 2].
+extern "C" int ta_attention_merge_tiles(const void* part_o, const void* part_ml, const void* tiles, int n_tiles,
+                                        const void* cu_q, void* out, int n_q, int d, int splits, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if ((long)n_tiles * 16 * n_q > 0x7fffffffL || d % 4 || splits < 1) return -1;
+  decode_attention_merge<<<n_tiles * 16 * n_q, 64, 0, stream>>>((const float*)part_o, (const float*)part_ml, nullptr,
+                                                                (bf16_t*)out, n_q, d, splits, (const int*)tiles,
+                                                                (const int*)cu_q);
+  return LAUNCH_STATUS();
 }
 
 // Returns -2 for a head size this kernel has no instance for (the caller then uses the generic kernel).

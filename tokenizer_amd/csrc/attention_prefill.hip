@@ -328,12 +328,32 @@ static int launch_prefill(const void* q, int q_stride, void* out, const void* k_
 
 // The kernel whose waves share a block of keys through LDS (attention_prefill_shared.hip).
 extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, int d, int reach);
+extern "C" int ta_prefill_attention_shared_key_splits(int n_tiles, int n_q, int n_kv, int reach, int shape);
 extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                                 const void* vt_pages, const void* tiles, int n_tiles,
                                                 const void* cu_q, const void* first_position,
                                                 const void* block_table, int table_stride, int n_q, int n_kv, int d,
                                                 int page_size, int window, float scale, int shape,
-                                                hipStream_t stream);
+                                                int key_splits, void* part_o, void* part_ml, hipStream_t stream);
+
+// The shape in which the workgroup-shared kernel takes a launch (0: the per-wave kernel takes it), by what the
+// caller asked for and the launch's own plan.
+static int shared_shape_for(int n_tiles, int n_q, int n_kv, int d, int window, int shared_shape, int max_keys,
+                            int waves, int shared) {
+  if (shared < 0 || waves != 0 || (d != 64 && d != 128)) return 0;
+  int shape = ta_prefill_attention_shared_plan(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window));
+  if (shared > 0) shape = shared_shape > 0 ? shared_shape : shape ? shape : 2;
+  return shape;
+}
+
+// Into how many parts the launch below cuts the keys of a tile over workgroups (1: it does not).  More than one
+// needs the buffers `part_o` float [n_tiles * 16, n_q, parts, d] and `part_ml` float [n_tiles * 16, n_q, parts, 2].
+extern "C" int ta_prefill_attention_key_splits(int n_tiles, int n_q, int n_kv, int d, int window, int shared_shape,
+                                               int max_keys, int waves, int shared) {
+  if (n_tiles <= 0 || n_kv <= 0 || n_q % n_kv) return 1;
+  const int shape = shared_shape_for(n_tiles, n_q, n_kv, d, window, shared_shape, max_keys, waves, shared);
+  return ta_prefill_attention_shared_key_splits(n_tiles, n_q, n_kv, planned_reach(max_keys, window), shape);
+}
 
 // Returns -2 for a head size without an instance (the caller then uses another kernel).
 // max_keys: the highest position of the batch + 1 (a hint for the number of waves per tile).
@@ -341,24 +361,24 @@ extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, voi
 // heads a wave, + 10 for two key groups; 0 = its own choice), -1 = never, 0 = where it is the faster one (by the shape of the launch and the planned
 // reach, so that a launch recorded for a range of contexts and a launch for the exact context make the same
 // choice).  waves: waves that share a tile's keys in the per-wave kernel (1, 2, 4, 8; 0 = by the reach); asking
-// for a number asks for that kernel.
+// for a number asks for that kernel.  part_o, part_ml: buffers for `ta_prefill_attention_key_splits(...)` parts of
+// a tile's keys (null: the keys are not cut).
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
                                          int n_q, int n_kv, int d, int page_size, int window, float scale,
                                          int shared_shape, int max_keys, int waves, int shared,
-                                         hipStream_t stream) {
+                                         void* part_o, void* part_ml, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
-  if (shared >= 0 && waves == 0) {
-    int shape = ta_prefill_attention_shared_plan(n_tiles, n_q, n_kv, d, planned_reach(max_keys, window));
-    if (shared > 0) shape = shared_shape > 0 ? shared_shape : shape ? shape : 2;
-    if (shape) {
-      const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
-                                                          first_position, block_table, table_stride, n_q, n_kv, d,
-                                                          page_size, window, scale, shape, stream);
-      if (status != -2) return status;
-    }
+  const int shape = shared_shape_for(n_tiles, n_q, n_kv, d, window, shared_shape, max_keys, waves, shared);
+  if (shape) {
+    const int parts = (part_o && part_ml)
+        ? ta_prefill_attention_shared_key_splits(n_tiles, n_q, n_kv, planned_reach(max_keys, window), shape) : 1;
+    const int status = ta_prefill_attention_shared_bf16(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q,
+                                                        first_position, block_table, table_stride, n_q, n_kv, d,
+                                                        page_size, window, scale, shape, parts, part_o, part_ml, stream);
+    if (status != -2) return status;
   }
 #define CASE(DD, HG) case DD: return launch_prefill<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
     first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, stream);

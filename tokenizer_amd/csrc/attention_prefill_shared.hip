@@ -23,6 +23,10 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // Keys: 64 rows of D / 8 pieces, no padding; the piece that holds elements 8 p .. 8 p + 7 of key k stands at
 // place p ^ swizzle(k), so that the eight rows which neighbouring lanes read at once lie in different banks.
 // Values: run by run, D rows of the run's sixteen keys (32 bytes), which neighbouring lanes read 32 bytes apart.
+// attention_decode.hip: the parts of a tile's keys, merged into the output rows of the tile's tokens.
+extern "C" int ta_attention_merge_tiles(const void* part_o, const void* part_ml, const void* tiles, int n_tiles,
+                                        const void* cu_q, void* out, int n_q, int d, int splits, hipStream_t stream);
+
 template <int D>
 struct Staged {
   static_assert(D == 64 || D == 128, "a key row must be a power of two of pieces for the swizzle");
@@ -251,7 +255,8 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
                                 const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                                 const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
                                 const int* __restrict__ first_position, const int* __restrict__ block_table,
-                                int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
+                                int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2,
+                                int key_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int KS = D / 32;
   constexpr int DB = D / 16;
   constexpr int NW = SHARED_WAVES;
@@ -264,12 +269,14 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   const int head_blocks = (group + HG * NW - 1) / (HG * NW);
   // Late tiles first, as in the other prompt kernel: they see the most keys.
   const int per_tile = n_kv * head_blocks;
-  const int which = blockIdx.x % per_tile;
+  const int split = blockIdx.x % key_splits;               // which part of the tile's keys (of key_splits)
+  const int block = blockIdx.x / key_splits;
+  const int which = block % per_tile;
   const int kvh = which / head_blocks, hb = which % head_blocks;
   const int first_head = hb * HG * NW + head_wave * HG;       // among the heads of the kv head
   const int heads_here = max(0, min(HG, group - first_head));  // a wave past the last head only brings blocks
   const int head0 = kvh * group + first_head;
-  const int tile_index = n_tiles - 1 - blockIdx.x / per_tile;
+  const int tile_index = n_tiles - 1 - block / per_tile;
   const int entry = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index]);
   const int offset = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index + 1]);
   const int row0 = __builtin_amdgcn_readfirstlane(cu_q[entry]) + offset;
@@ -319,7 +326,13 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   // for what it asked for, and meets the other waves: after the barrier every wave's part of the next blocks has
   // landed, and nobody reads the current ones any more.  A group whose block of a turn lies past the last key
   // leaves it out.
-  int kb = (lo / 64) * 64;                                 // the turn's first key
+  // With the keys cut over workgroups (key_splits > 1: few tiles behind a long context), this one takes a run of
+  // whole turns of the tile's walk, `kb` .. `end`; a workgroup past the last turn walks nothing and hands on an
+  // empty state.
+  const int first_turn = (lo / 64) * 64;
+  const int turns_each = ((hi - first_turn) / STRIDE + key_splits) / key_splits;
+  int kb = first_turn + split * turns_each * STRIDE;       // the turn's first key
+  const int end = min(hi, kb + turns_each * STRIDE - 1);   // the last key of this workgroup's turns
   int cur = 0;
   char* buffers = staged + key_group * 2 * Staged<D>::BYTES;
   const int ahead = 64 * key_group;                        // the group's block within a turn
@@ -327,25 +340,25 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   carrier.plan(head_wave, lane, tile, kb + ahead, STRIDE);
   const auto whole = [&](int turn) { return turn >= lo_all && turn + STRIDE - 1 <= p0; };
   carrier.look_up(tile, kb + ahead, whole(kb));
-  if (kb + ahead <= hi) carrier.fetch(tile, buffers);
-  if (kb + STRIDE + ahead <= hi) carrier.look_up(tile, kb + STRIDE + ahead, whole(kb + STRIDE));
+  if (kb + ahead <= end) carrier.fetch(tile, buffers);
+  if (kb + STRIDE + ahead <= end) carrier.look_up(tile, kb + STRIDE + ahead, whole(kb + STRIDE));
   carrier.landed();
   __syncthreads();
 #define TURN(FULL)                                                                                            \
   {                                                                                                           \
     const int next = kb + STRIDE;                                                                             \
-    if (next + ahead <= hi) carrier.fetch(tile, buffers + (cur ^ 1) * Staged<D>::BYTES);                      \
-    if (next + STRIDE + ahead <= hi) carrier.look_up(tile, next + STRIDE + ahead, whole(next + STRIDE));      \
-    if (heads_here > 0 && (FULL || kb + ahead <= hi))                                                         \
+    if (next + ahead <= end) carrier.fetch(tile, buffers + (cur ^ 1) * Staged<D>::BYTES);                     \
+    if (next + STRIDE + ahead <= end) carrier.look_up(tile, next + STRIDE + ahead, whole(next + STRIDE));     \
+    if (heads_here > 0 && (FULL || kb + ahead <= end))                                                        \
       shared_block<D, HG, FULL>(buffers + cur * Staged<D>::BYTES, kb + ahead, col, g, my_pos, my_lo, lo, hi,  \
                                 scale_log2, qf, acc, m, l);                                                   \
     carrier.landed();                                                                                         \
     __syncthreads();                                                                                          \
     cur ^= 1;                                                                                                 \
   }
-  for (; kb <= hi && kb < lo_all; kb += STRIDE) TURN(false)
-  for (; kb + STRIDE - 1 <= p0; kb += STRIDE) TURN(true)
-  for (; kb <= hi; kb += STRIDE) TURN(false)
+  for (; kb <= end && kb < lo_all; kb += STRIDE) TURN(false)
+  for (; kb <= end && kb + STRIDE - 1 <= p0; kb += STRIDE) TURN(true)
+  for (; kb <= end; kb += STRIDE) TURN(false)
 #undef TURN
 
   if (KG > 1) {
@@ -389,7 +402,27 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc[h][db][r] += f * *at(k, h, db * 4 + r);
       }
+      m[h] = m_all;                                        // what the sums now stand under (a part hands it on)
     }
+  }
+  if (key_splits > 1) {
+    // This workgroup's part of the keys: the state goes out as it is, item (tile, token) x head x part, for the
+    // kernel that merges the parts (maximum in natural units of the scaled scores, sum, unnormalised output).
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+      if (h >= heads_here) break;
+      if (col >= n_valid) continue;
+      const size_t at = (((size_t)tile_index * 16 + col) * n_q + head0 + h) * key_splits + split;
+      if (g == 0) {
+        part_ml[2 * at] = (m[h] == -INFINITY) ? -INFINITY : m[h] * scale_log2 * 0.6931471805599453f;
+        part_ml[2 * at + 1] = l[h][0];
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        *reinterpret_cast<float4*>(part_o + at * D + db * 16 + 4 * g) =
+            make_float4(acc[h][db][0], acc[h][db][1], acc[h][db][2], acc[h][db][3]);
+    }
+    return;
   }
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
@@ -411,9 +444,9 @@ template <int D, int HG, int KG>
 static int launch_shared(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
                          const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
                          const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
-                         float scale, hipStream_t stream) {
+                         float scale, int key_splits, void* part_o, void* part_ml, hipStream_t stream) {
   const int group = n_q / n_kv;
-  const long workgroups = (long)n_tiles * n_kv * ((group + HG * SHARED_WAVES - 1) / (HG * SHARED_WAVES));
+  const long workgroups = (long)n_tiles * n_kv * ((group + HG * SHARED_WAVES - 1) / (HG * SHARED_WAVES)) * key_splits;
   if (workgroups > 0x7fffffffL) return -1;
   constexpr int lds = 2 * KG * Staged<D>::BYTES;
   static_assert(lds <= 160 * 1024, "the blocks must fit a compute unit's LDS");
@@ -426,8 +459,29 @@ static int launch_shared(const void* q, int q_stride, void* out, const void* k_p
   prefill_attention_shared_kernel<D, HG, KG><<<(unsigned)workgroups, SHARED_WAVES * KG * WAVE, lds, stream>>>(
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
       n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
-      window, scale * 1.4426950408889634f);
-  return LAUNCH_STATUS();
+      window, scale * 1.4426950408889634f, key_splits, (float*)part_o, (float*)part_ml);
+  int status = LAUNCH_STATUS();
+  if (status == 0 && key_splits > 1)
+    status = ta_attention_merge_tiles(part_o, part_ml, tiles, n_tiles, cu_q, out, n_q, D, key_splits, stream);
+  return status;
+}
+
+// Into how many parts the keys of a tile are cut over workgroups when the kernel runs in `shape`: one, unless the
+// launch has fewer workgroups than the device has compute units and the tokens look back over sixteen turns or
+// more.  Then a workgroup walks its keys while most of the device idles, and parts of at least eight turns each,
+// up to sixteen of them, fill it (28 / 4 heads of 128 behind 8,192 cached tokens, uncut | cut: 256 tokens 117 | 78
+// us, 128 tokens 110 | 45, 16 tokens 109 | 25; 12 / 2 heads: 512 tokens 122 | 79, 128 tokens 114 | 29).
+extern "C" int ta_prefill_attention_shared_key_splits(int n_tiles, int n_q, int n_kv, int reach, int shape) {
+  if (shape <= 0 || n_kv <= 0) return 1;
+  const int heads = shape % 10, key_groups = shape / 10 + 1;
+  const int group = n_q / n_kv;
+  const long workgroups = (long)n_tiles * n_kv * ((group + heads * SHARED_WAVES - 1) / (heads * SHARED_WAVES));
+  if (workgroups >= 256 || workgroups <= 0) return 1;
+  const int turns = reach / (64 * key_groups);
+  long parts = (256 + workgroups - 1) / workgroups;
+  if (parts > turns / 8) parts = turns / 8;
+  if (parts > 16) parts = 16;
+  return parts < 1 ? 1 : (int)parts;
 }
 
 // Whether the workgroup-shared kernel is the faster one, and in which shape: 0 = no, else heads a wave (1 or 2)
@@ -448,16 +502,25 @@ extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, 
   if (d != 64 && d != 128) return 0;
   const int group = n_q / n_kv;
   if (group < 3) return 0;
+  // A short portion behind a cached context at head size 128: however few the workgroups, the per-wave kernel's
+  // waves (two a tile there) each walk their keys with nothing to hide a block's trip to memory, and one head a
+  // wave with two key groups is ahead (12 / 2 heads: 512 tokens behind 8,192: 147 | 121 us, behind 30,000: 504 |
+  // 395; 128 behind 8,192: 151 | 114; 64 behind 2,000: 36 | 32; behind 1,000: 22 | 21.  28 / 4 heads: 256 behind
+  // 8,192: 130 | 116), the more so as its tiles' keys can be cut over workgroups (below).  At head size 64 the
+  // per-wave kernel (which gives such tiles eight waves) stays ahead up to some 3,000 keys (14 / 2 heads, 64 tokens
+  // behind 2,000: 19 | 20 us) and falls behind the cut tiles beyond (16 behind 3,500: 27 | 20; 256 behind 8,192: 50 |
+  // 30; 512 behind 30,000: 162 | 136).
+  const bool far = reach >= (d == 128 ? 1024 : 3072);
   if (group < 5) {
     // Three or four heads per kv head fill the four waves at one head each (32 / 8 heads of 128, per-wave | 1 head
     // | 1 head, 2 groups: 1,024 tokens 37 | 30 | 28; 2,048 tokens 106 | 69 | 81; 8,192 tokens 1,217 | 790 | 913;
     // 16 / 4 heads of 64: 2,048 tokens 30.0 | 30.1 | 24.4; 8,192 tokens 307 | 213 | 221).
     const long one = (long)n_tiles * n_kv;
-    if (one < 256) return 0;
+    if (one < 256) return far ? 11 : 0;
     return one < (d == 64 ? 2048 : 1024) ? 11 : 1;
   }
   const long two = (long)n_tiles * n_kv * ((group + 7) / 8);      // workgroups at two heads a wave
-  if (two < 128) return 0;
+  if (two < 128) return far ? 11 : 0;
   if (two >= 1024) return 2;
   if (d == 64) return 11;
   if (two >= 512) return 12;
@@ -466,18 +529,20 @@ extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, 
 }
 
 // Returns -2 for a head size without an instance (the caller then uses the other kernel).
-// shape: heads a wave (1 or 2), + 10 for two key groups in a workgroup.
+// shape: heads a wave (1 or 2), + 10 for two key groups in a workgroup.  key_splits: parts of a tile's keys, each
+// a workgroup's; more than one needs part_o float [n_tiles * 16, n_q, key_splits, d] and part_ml float [.., 2].
 extern "C" int ta_prefill_attention_shared_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                                 const void* vt_pages, const void* tiles, int n_tiles,
                                                 const void* cu_q, const void* first_position,
                                                 const void* block_table, int table_stride, int n_q, int n_kv, int d,
                                                 int page_size, int window, float scale, int shape,
-                                                hipStream_t stream) {
+                                                int key_splits, void* part_o, void* part_ml, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   const int heads_per_wave = shape % 10, key_groups = shape / 10 + 1;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || heads_per_wave < 1 || heads_per_wave > 2 || key_groups > 2) return -1;
+  if (key_splits < 1 || key_splits > 64 || (key_splits > 1 && (!part_o || !part_ml))) return -1;
 #define GO(DD, HG, KG) return launch_shared<DD, HG, KG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
-    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream);
+    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, key_splits, part_o, part_ml, stream);
 #define SIZE(DD) case DD: if (key_groups == 2) { if (heads_per_wave == 1) GO(DD, 1, 2) GO(DD, 2, 2) } \
     if (heads_per_wave == 1) GO(DD, 1, 1) GO(DD, 2, 1)
   switch (d) {

@@ -134,7 +134,7 @@ class Ops:
         self.lib = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16",
-                     "ta_prefill_attention_shared_plan",
+                     "ta_prefill_attention_shared_plan", "ta_prefill_attention_key_splits",
                      "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16",
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
@@ -322,12 +322,21 @@ class Ops:
                 return self._decode_attention(*args, identity_entries=batch.n_tokens == block_table.shape[0])
             _need(batch.n_tokens == n_tokens and batch.cu_q.numel() == block_table.shape[0] + 1,
                   "the batch description does not belong to these tokens")
+            n_tiles, choice = batch.q_tiles.shape[0], (
+                -1 if window is None else int(window), self.prefill_shape, int(batch.max_position) + 1,
+                self.prefill_waves, self.prefill_shared)
+            # A few tiles behind a long context: the launcher cuts each tile's keys over workgroups, whose states
+            # a second kernel merges; it says into how many parts, and gets the buffers for them.
+            parts = self.lib.ta_prefill_attention_key_splits(n_tiles, n_q, n_kv, head_dim, *choice) if self.prefill_key_splits else 1
+            part_o = part_ml = None
+            if parts > 1:
+                part_o = torch.empty((n_tiles * 16, n_q, parts, head_dim), dtype=torch.float32, device=qkv.device)
+                part_ml = torch.empty((n_tiles * 16, n_q, parts, 2), dtype=torch.float32, device=qkv.device)
             self._check(self.lib.ta_prefill_attention_bf16(
                 _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(batch.q_tiles),
-                batch.q_tiles.shape[0], _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
-                block_table.shape[1], n_q, n_kv, head_dim, page_size, -1 if window is None else int(window),
-                ctypes.c_float(scale), self.prefill_shape, int(batch.max_position) + 1,
-                self.prefill_waves, self.prefill_shared, self._stream()), "prefill_attention")
+                n_tiles, _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
+                block_table.shape[1], n_q, n_kv, head_dim, page_size, choice[0], ctypes.c_float(scale), *choice[1:],
+                _ptr(part_o), _ptr(part_ml), self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
                 self._decode_attention(*args, rows=batch.decode_rows)
             return out
@@ -346,6 +355,7 @@ class Ops:
     #                               (1 or 2), + 10 for two key groups in a workgroup; 0: its own choice
     prefill_shared = 0            # the prompt kernel whose waves share a block of keys through LDS: 1 = wherever it has
     #                               an instance, -1 = never, 0 = where the launcher expects it to be the faster one
+    prefill_key_splits = True     # whether the prompt kernel may cut a tile's keys over workgroups (tests switch it off)
     target_workgroups = 1024      # what the split of the key range aims at
     PLAN_KEYS = 512               # launch shapes depend on the context only through its multiple of this
 
