@@ -136,17 +136,21 @@ def run_decode(model, batch: int, steps: int, warmup: int):
     return elapsed, kv_mean
 
 
-def run_prefill(model, repeats: int = 7):
+def run_prefill(model, repeats: int = 7, portion: int | None = None):
+    """The prompt in one step, or cut into portions of `portion` tokens, one step each (the best of the repeats)."""
     import torch
     from tokenizer_amd.engine import Engine, StepEntry
     engine = Engine(model, num_pages=PROMPT_LEN // 16 + 8, page_size=16, max_requests=1)
     prompt = make_prompts(1, model.vocab_size, seed=2)[0]
+    portion = portion or PROMPT_LEN
     best = None
     for _ in range(repeats + 1):
         engine.add_request("p")
         torch.cuda.synchronize()
         started = time.perf_counter()
-        logits = engine.step([StepEntry("p", prompt, [PROMPT_LEN - 1])])
+        for at in range(0, PROMPT_LEN, portion):
+            tokens = prompt[at:at + portion]
+            logits = engine.step([StepEntry("p", tokens, [len(tokens) - 1] if at + portion >= PROMPT_LEN else [])])
         engine.argmax(logits)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
@@ -307,6 +311,8 @@ def main() -> int:
                         help="run a serving workload through the scheduler instead of the decode benchmark")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     parser.add_argument("--only-prefill", action="store_true", help="time the prefill alone (for profiling)")
+    parser.add_argument("--portion", type=int, default=None,
+                        help="with --only-prefill: cut the prompt into portions of this many tokens, one step each")
     parser.add_argument("--attention", type=int, default=None, metavar="TOKENS",
                         help="time the prompt attention kernel alone on a portion of this many tokens at --size's head shape")
     parser.add_argument("--cached", type=int, default=0, help="with --attention: tokens already in the cache")
@@ -357,8 +363,9 @@ def main() -> int:
     kv_token = kv_bytes_per_token(cfg, itemsize)
 
     if args.only_prefill:
-        seconds = run_prefill(model)
-        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PROMPT_LEN}), flush=True)
+        seconds = run_prefill(model, repeats=3 if args.portion else 7, portion=args.portion)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PROMPT_LEN, "portion": args.portion or PROMPT_LEN,
+                          "tokens_per_s": round(PROMPT_LEN / seconds, 1)}), flush=True)
         return 0
     log(f"decode at batch {args.batch}: {args.warmup} warmup + {args.steps} timed steps")
     elapsed, kv_mean = run_decode(model, args.batch, args.steps, args.warmup)
