@@ -391,6 +391,10 @@ def test_where_the_workgroup_shared_kernel_is_planned(ops):
     assert plan(31, 28, 4, 128, 512) == 0 and plan(31, 28, 4, 128, 1024) == 11      # few tiles: only behind some context ...
     assert plan(1, 12, 2, 128, 4096) == 11 and plan(8, 32, 8, 128, 8192) == 11 and plan(31, 14, 2, 64, 2560) == 0   # ... at head size 128,
     assert plan(31, 14, 2, 64, 3072) == 11 and plan(2, 16, 4, 64, 8192) == 11           # behind 3,072 keys and more at head size 64
+    # behind 6,144 keys and more two heads a wave read each block half as often; the shortest portions stay at one
+    assert plan(16, 28, 4, 128, 8704) == 12 and plan(4, 28, 4, 128, 8704) == 11 and plan(16, 28, 4, 128, 5632) == 11
+    assert plan(32, 28, 4, 128, 8704) == 12 and plan(64, 12, 2, 128, 9216) == 12 and plan(64, 14, 2, 64, 9216) == 12
+    assert plan(128, 14, 2, 64, 10240) == 11 and plan(32, 14, 2, 64, 8704) == 12 and plan(8, 14, 2, 64, 8704) == 11
     splits = ops.lib.ta_prefill_attention_shared_key_splits
     # (tiles, query heads, kv heads, reach, shape) -> parts of a tile's keys: fewer workgroups than compute units and a long reach
     assert splits(8, 28, 4, 8704, 11) == 4 and splits(1, 28, 4, 8704, 11) == 8 and splits(32, 12, 2, 8704, 11) == 2

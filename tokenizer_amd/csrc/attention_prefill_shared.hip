@@ -520,12 +520,18 @@ extern "C" int ta_prefill_attention_shared_plan(int n_tiles, int n_q, int n_kv, 
     return one < (d == 64 ? 2048 : 1024) ? 11 : 1;
   }
   const long two = (long)n_tiles * n_kv * ((group + 7) / 8);      // workgroups at two heads a wave
-  if (two < 128) return far ? 11 : 0;
+  // Behind 6,144 keys and more, with the keys cut over workgroups where those are few, what a launch pulls through
+  // the fabric counts: two heads a wave read every block half as often (28 / 4 heads of 128, one | two heads a wave,
+  // 256 tokens behind 8,192: 78 | 62 us, 512 tokens: 120 | 102, 256 behind 16,000: 121 | 93; 12 / 2 heads: 512 behind
+  // 8,192: 73 | 58, 1,024: 128 | 101; 14 / 2 heads of 64: 512 behind 8,192: 47 | 41), but for the shortest portions
+  // one head a wave stays ahead (64 tokens of 28 / 4 heads: 29 | 34; 128 of 12 / 2: 27 | 33).
+  const bool very_far = far && reach >= 6144;
+  if (two < 128) return !far ? 0 : (very_far && two >= 32) ? 12 : 11;
   if (two >= 1024) return 2;
-  if (d == 64) return 11;
+  if (d == 64) return (very_far && two < 256) ? 12 : 11;
   if (two >= 512) return 12;
   if (two >= 256) return reach >= 4096 ? 12 : 11;
-  return 11;
+  return very_far ? 12 : 11;
 }
 
 // Returns -2 for a head size without an instance (the caller then uses the other kernel).
