@@ -718,6 +718,35 @@ def test_like_layers_make_the_recorded_calls_of_the_first_again(model_folders, n
         assert repeated[0] >= len(steps) * (n_layers - 2)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_model_under_one_engine_after_another(model_folders, oracle, dtype):
+    """A model outlives its engines (a benchmark makes one engine per batch size over one model): the second and
+    third engines have pools of other sizes at other addresses, and the first is gone (collected) when they run.
+    Their eager mixed steps repeat recorded layers and still equal, bit for bit, an engine whose layers all run
+    their own Python, and the plain model."""
+    import gc
+    from tokenizer_amd.engine import Engine, load_model
+    name = "C"
+    reqs = requests_for(name)
+    steps = tt.mixed(reqs, 21)
+    model = load_model(model_folders[name], dtype)
+    plain_engine = engine_for(model_folders[name], dtype, max_tokens=tt.peak_tokens(steps), max_requests=4, use_graphs=False)
+    plain_engine.model.decoder.repeat_layers = False
+    want = tt.run_in_process(plain_engine, steps)
+    for extra_pages in (0, 7, 3, 11, 0, 5):
+        eng = Engine(model, num_pages=-(-tt.peak_tokens(steps) // 16) + extra_pages, max_requests=4, use_graphs=False)
+        eng.pools.poison()
+        before = model.decoder.layers_repeated
+        got = tt.run_in_process(eng, steps)
+        assert model.decoder.layers_repeated > before
+        for rid, ids in reqs.items():
+            assert torch.equal(got[rid], want[rid]), (rid, extra_pages)
+            close(got[rid], oracle(name, ids), dtype)
+        del eng
+        gc.collect()
+        torch.cuda.empty_cache()
+
+
 def test_a_layer_named_twice_and_a_layer_on_anothers_pages_are_repeated_rightly(tmp_path):
     """The order of layers is data: a schedule that runs a layer twice and lets a layer read another layer's pages
     (without writing) gives the same logits whether the like layers repeat recorded calls or run on their own."""

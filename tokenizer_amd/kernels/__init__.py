@@ -34,13 +34,22 @@ def _raw_stream(device_index: int) -> int:
     return torch._C._cuda_getCurrentRawStream(device_index)
 
 
-_KEEP: list | None = None      # while a layer's calls are recorded: every tensor whose address went into one
+class _Recording(threading.local):
+    """What the thread that records a layer's calls is recording into (nothing, for every other thread)."""
+    library = None        # the `_RecordingLibrary` that stands in for the loaded one
+    keep: list | None = None      # every tensor whose address went into a recorded call
+
+
+_RECORDING = _Recording()
 
 
 def _ptr(tensor: torch.Tensor | None) -> ctypes.c_void_p:
-    if _KEEP is not None and tensor is not None:
-        _KEEP.append(tensor)
-    return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+    if tensor is None:
+        return ctypes.c_void_p(0)
+    keep = _RECORDING.keep
+    if keep is not None:
+        keep.append(tensor)
+    return ctypes.c_void_p(tensor.data_ptr())
 
 
 def _need(cond: bool, message: str) -> None:
@@ -107,6 +116,10 @@ class LaunchTape:
             if got != status:
                 raise KernelError(f"a recorded call returned {got} where it had returned {status}")
 
+    def addresses(self) -> set:
+        """Every address that went into a recorded call."""
+        return {address for _, _, _, addresses in self.calls for _, address in addresses}
+
 
 class _RecordingLibrary:
     """Stands in for the loaded library while a tape is recorded: every call goes through and onto the tape."""
@@ -131,7 +144,7 @@ class Ops:
 
     def __init__(self, path: str):
         self.path = path
-        self.lib = ctypes.CDLL(path)
+        self._loaded = ctypes.CDLL(path)
         for name in ("ta_embedding", "ta_add_rmsnorm", "ta_silu_gate", "ta_rope_store",
                      "ta_paged_attention_generic", "ta_decode_attention_bf16", "ta_prefill_attention_bf16",
                      "ta_prefill_attention_shared_plan", "ta_prefill_attention_key_splits",
@@ -167,17 +180,22 @@ class Ops:
             raise KernelError(f"{what} failed with status {status}"
                               + (" (sizes the kernel does not take)" if status < 0 else " (HIP error)"))
 
+    @property
+    def lib(self):
+        """The loaded library, or, on a thread that is recording a layer's calls, the recorder in front of it."""
+        return _RECORDING.library or self._loaded
+
     @contextlib.contextmanager
     def record_launches(self):
-        """Record every library call made inside the block on a `LaunchTape` (which the block receives)."""
-        global _KEEP
+        """Record every library call this thread makes inside the block on a `LaunchTape` (which the block
+        receives).  Other threads' calls are not touched; a recording inside a recording takes over until it ends."""
         tape = LaunchTape()
-        library, keep = self.lib, _KEEP
-        self.lib, _KEEP = _RecordingLibrary(library, tape), tape.keep
+        before = _RECORDING.library, _RECORDING.keep
+        _RECORDING.library, _RECORDING.keep = _RecordingLibrary(self._loaded, tape), tape.keep
         try:
             yield tape
         finally:
-            self.lib, _KEEP = library, keep
+            _RECORDING.library, _RECORDING.keep = before
 
     # ------------------------------------------------------------------ embedding
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -64,6 +64,11 @@ class _Make:
                                      for t in tensors))
         self.addresses = tuple(0 if t is None else t.data_ptr() for t in tensors)
         self.tensors = tensors                 # kept, so the addresses stay theirs
+        # The address maps from recorded layers of the same key to this one, by the recorded layer's make itself
+        # (never by its id, which another object may get once that make is gone): they live and die with the
+        # makes, which belong to one engine's cache entries.
+        self.puts: dict["_Make", object] = {}
+        self.held: frozenset = frozenset()     # addresses of every tensor the layer's parts hold, listed or not
 
 
 @dataclasses.dataclass
@@ -73,6 +78,26 @@ class _Recorded:
     make: _Make
     coming: tuple                 # the addresses of what the layer was handed
     result: object                # what it handed on (its buffers serve every layer that repeats the calls)
+    unlisted: frozenset = frozenset()   # addresses on the tape of tensors the layer holds without having listed them
+
+
+def _tensor_addresses(part, seen=None) -> set:
+    """The addresses of every tensor that a part holds as an attribute, itself or through the parts it holds (a
+    block's norms, a mixer's position encoding), lists and tuples included."""
+    seen = set() if seen is None else seen
+    found: set[int] = set()
+    if part is None or id(part) in seen or not hasattr(part, "__dict__"):
+        return found
+    seen.add(id(part))
+    for value in vars(part).values():
+        for item in (value if isinstance(value, (list, tuple)) else (value,)):
+            if isinstance(item, torch.Tensor):
+                if item.numel():
+                    found.add(item.data_ptr())
+            elif hasattr(item, "__dict__") and not isinstance(item, (type, Runtime)) \
+                    and type(item).__module__.split(".")[0] not in ("torch", "ctypes", "threading", "builtins"):
+                found |= _tensor_addresses(item, seen)
+    return found
 
 
 def _coming(delta):
@@ -126,14 +151,17 @@ class DecoderModel:
             all(hasattr(b, "mixer") for b in self.blocks)
         self.repeat_layers = True      # record one layer's library calls and make them again for the like ones
         self.layers_repeated = 0       # how many scheduled layers have run that way so far
-        self._put: dict[tuple[int, int], dict[int, int]] = {}
+        self.promises_broken = 0       # recordings thrown away because a call took a tensor the parts had not listed
 
     def _make_of(self, block, layer: int, cache: "LayerCache"):
         """The make of a scheduled layer on this cache, or None if the block does not promise to be repeatable.
         Worked out once and kept on the cache entry."""
         if layer not in cache.makes:
             said = repeatable_of(block, cache)
-            cache.makes[layer] = None if said is None else _Make(said.constants, said.tensors)
+            make = None if said is None else _Make(said.constants, said.tensors)
+            if make is not None:
+                make.held = frozenset(_tensor_addresses(block))
+            cache.makes[layer] = make
         return cache.makes[layer]
 
     def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
@@ -160,13 +188,20 @@ class DecoderModel:
                 with record() as tape:
                     out = block.forward(residual, delta, ctx, cache)
                 if _coming(out)[0] == form:       # what it hands on looks like what it was handed: it can follow itself
-                    tapes[(make.key, form)] = _Recorded(tape, make, addresses, out)
+                    # The promise is checked as far as the host can see: a call that took a tensor which the
+                    # layer's parts hold but did not list depends on the layer through more than the list.
+                    unlisted = (make.held - set(make.addresses)) & tape.addresses()
+                    tapes[(make.key, form)] = _Recorded(tape, make, addresses, out, frozenset(unlisted))
                 delta = out
                 continue
-            put = self._put.get((id(recorded.make), id(make)))
+            put = make.puts.get(recorded.make)
             if put is None:
-                put = self._put[(id(recorded.make), id(make))] = _addresses_put(recorded.make.addresses, make.addresses)
-            if put is False:                      # one tensor in two places there, two tensors here: no single map
+                if recorded.unlisted <= make.held:     # (a tensor that both layers hold, a shared table, is the same one)
+                    put = _addresses_put(recorded.make.addresses, make.addresses)
+                else:
+                    put, self.promises_broken = False, self.promises_broken + 1
+                make.puts[recorded.make] = put
+            if put is False:                      # no single map (one tensor in two places there, two here), or a broken promise
                 delta = block.forward(residual, delta, ctx, cache)
                 continue
             if addresses != recorded.coming:
