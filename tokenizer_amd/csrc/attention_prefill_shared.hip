@@ -476,9 +476,10 @@ extern "C" int ta_prefill_attention_shared_key_splits(int n_tiles, int n_q, int 
   const int heads = shape % 10, key_groups = shape / 10 + 1;
   const int group = n_q / n_kv;
   const long workgroups = (long)n_tiles * n_kv * ((group + heads * SHARED_WAVES - 1) / (heads * SHARED_WAVES));
-  if (workgroups >= 256 || workgroups <= 0) return 1;
+  const long units = compute_units();
+  if (workgroups >= units || workgroups <= 0) return 1;
   const int turns = reach / (64 * key_groups);
-  long parts = (256 + workgroups - 1) / workgroups;
+  long parts = (units + workgroups - 1) / workgroups;
   if (parts > turns / 8) parts = turns / 8;
   if (parts > 16) parts = 16;
   return parts < 1 ? 1 : (int)parts;

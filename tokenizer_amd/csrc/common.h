@@ -53,6 +53,21 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// The compute units of the device, asked of the runtime once (the same on every device of a machine); launchers
+// that weigh a launch's workgroups against the device use this, never a number of their own.
+static inline int compute_units() {
+  static int count = 0;
+  if (count == 0) {
+    int device = 0, value = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0)
+      count = value;
+    else
+      count = 256;
+  }
+  return count;
+}
+
 // Every launcher returns 0, or the HIP error code of its launch.
 #define LAUNCH_STATUS() ((int)hipGetLastError())
 

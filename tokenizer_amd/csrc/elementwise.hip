@@ -247,3 +247,6 @@ extern "C" int ta_silu_gate(const void* in, void* out, int n_tokens, int inner, 
     silu_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner, total);
   return LAUNCH_STATUS();
 }
+
+// The number of compute units that the launchers plan for (the current device's).
+extern "C" int ta_compute_units() { return compute_units(); }

@@ -388,19 +388,6 @@ static int launch_rows(const FusedArgs& args, int tiles, int waves, hipStream_t 
   return -1;
 }
 
-static int compute_units() {
-  static int count = 0;                                     // the same on every device of a machine
-  if (count == 0) {
-    int device = 0, value = 0;
-    if (hipGetDevice(&device) == hipSuccess &&
-        hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0)
-      count = value;
-    else
-      count = 256;
-  }
-  return count;
-}
-
 // Weight rows per workgroup for the rotation epilogue, where a block pairs rows half a head apart: 16, 8 or 4.
 // Every workgroup reads and normalises all m input rows before its share of the weights, so the choice weighs
 // the bytes the busiest compute unit has to ask for: rounds of workgroups x (prologue + its weight rows).

@@ -329,7 +329,7 @@ extern "C" int ta_gemm_skinny_qkv_rope(const void* x, int lda, const void* W, co
   const int blocks = (M + 15) / 16;
   // Few tiles (a small model's joined matrix is a few dozen): the blocks of sixteen rows are dealt to workgroups
   // of their own, as many shares as it takes to fill the device; every share reads the matrix again.
-  const int shares = min(blocks, (256 + tiles - 1) / tiles);
+  const int shares = min(blocks, (compute_units() + tiles - 1) / tiles);
   const int per_share = (blocks + shares - 1) / shares;
   const dim3 grid(tiles, 1, (blocks + per_share - 1) / per_share);
 #define GO(MBV) skinny_gemm_kernel<MBV, 8, true, bf16_t, true><<<grid, 8 * WAVE, 0, stream>>>( \

@@ -1,8 +1,7 @@
 // An entry point of the kernel library that allocates nothing.
 //
-// It has no counterpart in the reference (MahadRana/tokenizer is host code throughout; its greedy pick is
-// qwen-infer/src/sample.rs:43-56).  It is for callers that cannot call hipMalloc, or anything that does: code
-// under HIP graph capture, tight serving loops, harnesses that forbid allocation.
+// It has no counterpart in the reference.  It is for callers that cannot call hipMalloc, or anything that does:
+// code under HIP graph capture, tight serving loops, harnesses that forbid allocation.
 #pragma once
 #include <hip/hip_runtime.h>
 

@@ -152,11 +152,12 @@ class Ops:
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_sample",
-                     "ta_sample_workspace_words", "ta_library_gemm_bf16"):
+                     "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
         self._workspaces: dict[int, torch.Tensor] = {}
+        self.compute_units = int(self._loaded.ta_compute_units())     # what the splits below aim to fill
 
     @staticmethod
     def _stream() -> ctypes.c_void_p:
@@ -532,9 +533,9 @@ class Ops:
             return 4 if k >= 2048 else 1
         if not (self.FUSED_ROWS < m <= self.SKINNY_ROWS) or k < self.SPLIT_K_FROM:
             return 1
-        if tiles >= 256:
+        if tiles >= self.compute_units:
             return 1
-        return max(1, min(-(-512 // tiles), k // 256))
+        return max(1, min(-(-2 * self.compute_units // tiles), k // 256))
 
     split_k_kind = "streaming"     # which kernel cuts K for 17 to 64 rows ("tiled": only the tiled one)
 
@@ -556,7 +557,7 @@ class Ops:
             return 1
         if m > 32:
             tiles = -(-n // 32)        # more than 32 rows: a workgroup takes two blocks of sixteen columns
-        return max(1, min(-(-256 // tiles), k // part))
+        return max(1, min(-(-self.compute_units // tiles), k // part))
 
     PENDING_SHORTEST_K = 512   # the shortest K that is cut when the parts may be left for the next norm
     SPLIT_K_FROM = 8192        # the shortest K that the tiled kernel cuts (shorter ones are the weight-streaming kernel's)

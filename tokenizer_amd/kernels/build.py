@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import concurrent.futures
 import glob
+import hashlib
 import os
 import shutil
 import subprocess
@@ -54,11 +55,52 @@ def library_candidates(name: str = LIB_NAME) -> list[str]:
     return [os.path.join(PACKAGE_DIR, name), os.path.join(fallback, name)]
 
 
-def find_library(name: str = LIB_NAME) -> str | None:
+def _first_built(name: str) -> str | None:
     for path in library_candidates(name):
         if os.path.exists(path):
             return path
     return None
+
+
+def kernel_sources() -> list[str]:
+    """Everything the kernel library is compiled from: the HIP files and the headers beside them."""
+    return sorted(glob.glob(os.path.join(SOURCE_DIR, "*.hip")) + glob.glob(os.path.join(SOURCE_DIR, "*.h")))
+
+
+def _digest(sources: list[str], flags: list[str]) -> str:
+    """A digest of what a library is built from: the text of its sources and the compiler's flags."""
+    digest = hashlib.sha256(" ".join(flags).encode())
+    for source in sources:
+        digest.update(os.path.basename(source).encode() + b"\0")
+        with open(source, "rb") as handle:
+            digest.update(handle.read())
+    return digest.hexdigest()
+
+
+def _stamp_of(path: str) -> str | None:
+    try:
+        with open(path + ".stamp") as handle:
+            return handle.read().strip()
+    except OSError:
+        return None
+
+
+def _write_stamp(path: str, digest: str) -> None:
+    with open(path + ".stamp", "w") as handle:
+        handle.write(digest + "\n")
+
+
+def find_library(name: str = LIB_NAME) -> str | None:
+    """A built kernel library that was built from the sources as they are now (an edited kernel beside an old
+    library would otherwise run the old code without a word): the build leaves a digest of its sources beside
+    the library, which is compared with theirs.  None if there is no such library, and the caller builds it."""
+    path = _first_built(name)
+    if path is None or name != LIB_NAME:
+        return path
+    if _stamp_of(path) != _digest(kernel_sources(), HIPCC_FLAGS):
+        _say(f"{path} was not built from the sources under {SOURCE_DIR} as they are now: it is not used")
+        return None
+    return path
 
 
 def _writable_target(name: str = LIB_NAME) -> str:
@@ -117,6 +159,7 @@ def build_library(verbose: bool = True) -> str:
         if proc.returncode != 0:
             raise RuntimeError(f"linking the kernel library failed:\n{proc.stderr[-4000:]}")
         os.replace(partial, target)
+        _write_stamp(target, _digest(kernel_sources(), HIPCC_FLAGS))
     if verbose:
         _say(f"built {target} in {time.time() - started:.1f} s")
     return target
@@ -135,12 +178,15 @@ def host_sources() -> list[str]:
 
 
 def find_host_library() -> str | None:
-    """A built host library that is not older than its sources."""
-    path = find_library(HOST_LIB_NAME)
+    """A built host library that was built from its sources as they are now."""
+    path = _first_built(HOST_LIB_NAME)
     if path is None:
         return None
-    newest = max((os.path.getmtime(f) for f in glob.glob(os.path.join(HOST_SOURCE_DIR, "*"))), default=0.0)
-    return path if os.path.getmtime(path) >= newest else None
+    return path if _stamp_of(path) == _digest(_host_inputs(), HOST_FLAGS) else None
+
+
+def _host_inputs() -> list[str]:
+    return sorted(glob.glob(os.path.join(HOST_SOURCE_DIR, "*.cpp")) + glob.glob(os.path.join(HOST_SOURCE_DIR, "*.h")))
 
 
 def build_host_library(verbose: bool = True) -> str:
@@ -156,6 +202,7 @@ def build_host_library(verbose: bool = True) -> str:
     if proc.returncode != 0:
         raise RuntimeError(f"compiling the host library failed:\n{proc.stderr[-4000:]}")
     os.replace(partial, target)
+    _write_stamp(target, _digest(_host_inputs(), HOST_FLAGS))
     if verbose:
         _say(f"built {target} in {time.time() - started:.1f} s")
     return target
