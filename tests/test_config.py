@@ -116,3 +116,30 @@ def test_a_new_architecture_registers_without_touching_the_package(tmp_path):
     assert cfg.width == 12 and cfg.depth == 1 and cfg.architecture == name
     with pytest.raises(ValueError):
         register_architecture(name, ToyConfig, lambda cfg: None)
+
+
+def test_the_frame_around_the_layers_is_chosen_by_the_spec():
+    import dataclasses
+    import torch
+    from tiny_configs import TINY
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.models.qwen2 import qwen2_spec
+    from tokenizer_amd.parts import FRAMES, DecoderModel, cache_needs, expected_tensors
+    spec = qwen2_spec(Qwen2Config.from_dict(TINY["A"][0]))
+    assert spec.frame == "decoder" and FRAMES.get("decoder") is DecoderModel
+    names = set(expected_tensors(spec))
+    with pytest.raises(KeyError, match="unknown model frame 'pyramid'; registered: .*decoder"):
+        expected_tensors(dataclasses.replace(spec, frame="pyramid"))
+
+    class WithTable(DecoderModel):
+        """A frame that reads one tensor more than the built-in one."""
+        @staticmethod
+        def expected_tensors(spec):
+            from tokenizer_amd.parts import TensorSpec
+            return dict(DecoderModel.expected_tensors(spec), **{"model.positions.weight": TensorSpec((spec.max_positions, spec.hidden_size))})
+
+    if "toy_with_table" not in FRAMES.kinds():
+        FRAMES.register("toy_with_table", WithTable)
+    other = dataclasses.replace(spec, frame="toy_with_table")
+    assert set(expected_tensors(other)) == names | {"model.positions.weight"}
+    assert cache_needs(other) == cache_needs(spec)

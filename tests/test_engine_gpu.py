@@ -553,6 +553,22 @@ def test_greedy_generation_through_the_entry_points(model_folders, tmp_path, dty
     assert f"generated ids: {out.tokens}" in run.stderr and "stop: MaxTokens" in run.stderr
     assert "tok/s (8 tokens, KV cache, total" in run.stderr
     assert run.stdout.split() == [str(t) for t in out.tokens]
+    # A warm request: the command line queues it through the scheduler, `generate` drives the step function itself;
+    # both draw the same ids from the request's own seed.
+    warm = GenerateParams(max_tokens=7, temperature=0.9, top_p=0.8, seed=11)
+    alone = generate(eng, prompt, warm)
+    run = subprocess.run([sys.executable, f"{root}/bin/qwen-infer", "--model", model_folders[name], "--dtype", dtype,
+                          "--max-tokens", "7", "--temperature", "0.9", "--top-p", "0.8", "--seed", "11",
+                          "--num-blocks", "8", "--token-ids", " ".join(map(str, prompt))],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert "max_tokens 7 temperature 0.9 top_p 0.8 seed 11 eos []" in run.stderr
+    assert f"generated ids: {alone.tokens}" in run.stderr
+    # A prompt the pool cannot hold is answered with the scheduler's message, not a traceback.
+    run = subprocess.run([sys.executable, f"{root}/bin/qwen-infer", "--model", model_folders[name], "--dtype", dtype,
+                          "--num-blocks", "2", "--token-ids", " ".join(map(str, random_ids(cfg["vocab_size"], 60, 6)))],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 1 and "error: kv pool has 2 blocks of 16; this sequence needs" in run.stderr
 
 
 def test_warm_requests_draw_on_the_device_as_they_would_alone(model_folders):

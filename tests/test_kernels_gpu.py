@@ -844,8 +844,8 @@ def test_linear_float32_is_true_float32(ops):
 def test_linear_float32_is_true_float32_at_every_row_count(ops, rows):
     """The same probe for each of the 32-bit product's kernels (one row, up to sixteen rows, the tiled kernel for
     more): operands that need 13 mantissa bits, over a K long enough for the tile loop to turn, in every row and
-    column of a tile and past its edge.  A reduced-precision matrix mode would be off by about 1e-2 per unit of the
-    sum; true 32-bit products and sums are within a few 1e-4 of the 64-bit result of sums near 500."""
+    column of a tile and past its edge.  A reduced-precision matrix mode would be off by
+    about 2e-2; true 32-bit products and sums are within a few 1e-4 of the 64-bit result of sums near 500."""
     k, n = 520, 150
     x = (1 + torch.arange(k, dtype=torch.float64)[None, :] * 2.0 ** -12
          + torch.arange(rows, dtype=torch.float64)[:, None] * 2.0 ** -13).float().cuda()
@@ -854,9 +854,9 @@ def test_linear_float32_is_true_float32_at_every_row_count(ops, rows):
     got = ops.linear(x, w, None)
     want = x.double() @ w.double().t()
     assert float((got.double() - want).abs().max()) < 2e-3
-    # What rounding the operands to bfloat16 or to a 10-bit mantissa would do to the same sums: far outside.
+    # What rounding the operands to bfloat16 would do to the same sums: several times the bound.
     low = x.bfloat16().double() @ w.bfloat16().double().t()
-    assert float((low - want).abs().max()) > 0.5
+    assert float((low - want).abs().max()) > 1e-2
 
 
 def test_argmax_first_maximum_wins(ops):

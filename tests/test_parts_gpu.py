@@ -686,3 +686,64 @@ def test_layers_without_a_sub_layer_and_parts_that_offer_their_fused_form(tmp_pa
         assert folded["qkv"] >= 2 and folded["gated"] >= 2, folded
     else:
         assert folded == {"qkv": 0, "gated": 0}
+
+
+# ------------------------------------------------------------------------------------------------
+# A model frame defined outside the package (tests/toy_scaled_frame.py): a scaled embedding, capped logits.
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_frame_of_its_own_registers_and_runs_through_engine_scheduler_and_replay(tmp_path, dtype):
+    """What stands around the layers is chosen by the spec (`ModelSpec.frame`), as every part is: a toy frame that
+    multiplies its embedding by a constant from its own config.json key and caps its logits is registered from a
+    test's file and runs through the engine (mixed batches with reused pages, decode steps replayed from graphs),
+    through the scheduler, and through `bin/trace_run` as a child process (which imports the file because the
+    environment names it), against the plain model with the embedding scaled by hand."""
+    import os
+    import trace_tools as tt
+    import tokenizer_amd as ta
+    import toy_scaled_frame as toy
+    from tiny_configs import TINY, random_ids
+    from tokenizer_amd.engine import Engine, GenerateParams, load_model
+
+    kind = torch.float32 if dtype == "float32" else torch.bfloat16
+    raw = dict(TINY["B"][0], architectures=[toy.ARCHITECTURE], embedding_scale=3.5, logit_cap=1.5)
+    folder = ta.write_random_model(toy.ToyScaledConfig.from_dict(raw), 5, str(tmp_path / "scaled"), norm_spread=0.3)
+    cfg, tensors = plain.load_folder(folder)
+    scaled = dict(tensors)
+    scaled["model.embed_tokens.weight"] = tensors["model.embed_tokens.weight"].float() * 3.5     # (the head is untied)
+    assert not raw["tie_word_embeddings"]
+
+    def want_logits(ids):
+        return torch.tanh(plain.all_logits(cfg, scaled, ids) / 1.5) * 1.5
+
+    reqs = {f"r{i}": random_ids(raw["vocab_size"], n, 90 + i) for i, n in enumerate([40, 7, 64, 33, 21])}
+    want = {rid: want_logits(ids) for rid, ids in reqs.items()}
+    # The scale matters: without it the logits are far away.
+    unscaled = torch.tanh(plain.all_logits(cfg, tensors, reqs["r0"]) / 1.5) * 1.5
+    assert float((unscaled - want["r0"]).abs().max()) > 0.1
+    model = load_model(folder, dtype)
+    assert type(model.decoder).__name__ == "ToyScaledDecoder"
+    for steps in (tt.mixed(reqs, 3), tt.decode_tail(reqs, 20)):
+        eng = Engine(model, max_tokens=tt.peak_tokens(steps), max_requests=4)
+        eng.pools.poison()
+        got = tt.run_in_process(eng, steps)
+        for rid in reqs:
+            close(got[rid], want[rid], kind)
+    # The scheduler: greedy ids against the plain model's (32-bit), and equal to the same request alone.
+    eng = Engine(model, num_pages=24, max_requests=3, max_num_batched_tokens=48)
+    ids = {eng.add_request(reqs[rid][:30], GenerateParams.greedy(6)): rid for rid in ("r0", "r2", "r3")}
+    results = eng.run()
+    for request, rid in ids.items():
+        tokens, seq = [], list(reqs[rid][:30])
+        for _ in range(6):
+            tokens.append(int(want_logits(seq)[-1].argmax()))
+            seq.append(tokens[-1])
+        if dtype == "float32":
+            assert results[request].tokens == tokens, rid
+        assert len(results[request].tokens) == 6
+    # bin/trace_run in a child process: the environment names the module that registers the frame.
+    steps = tt.portions({rid: reqs[rid] for rid in ("r0", "r1")}, 5)
+    env = dict(os.environ, TOKENIZER_AMD_PLUGINS="toy_scaled_frame",
+               PYTHONPATH=os.path.dirname(os.path.abspath(__file__)) + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    got = tt.run_program(folder, dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps), raw["vocab_size"], env=env)
+    for rid in ("r0", "r1"):
+        close(got[rid], want[rid], kind)

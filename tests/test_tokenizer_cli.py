@@ -164,3 +164,34 @@ def test_merges_in_the_host_library_follow_the_rule_spelled_out_here():
             assert tok.decode(want) == text
     long_piece = "ab" * 400                                    # more parts than the first buffer holds
     assert tok.decode(tok.encode(long_piece)) == long_piece
+
+
+def test_the_tokenizer_is_chosen_by_what_the_file_declares(tmp_path):
+    from tokenizer_amd.tokenizer import load_tokenizer, register_tokenizer, registered_tokenizers
+    folder = tmp_path / "model"
+    folder.mkdir()
+    (folder / "tokenizer.json").write_text(json.dumps(tiny_file()))
+    tok = load_tokenizer(str(folder))                                  # a folder, or the file itself
+    assert isinstance(tok, Tokenizer) and tok.encode("ab") == [256]
+    assert Tokenizer.load(str(folder / "tokenizer.json")).encode("ab") == [256]
+    # A file of another kind is refused with what it declares and what is known ...
+    other = {"model": {"type": "WordLevel", "vocab": {"a": 0, "b": 1}}, "pre_tokenizer": {"type": "Whitespace"}}
+    (folder / "tokenizer.json").write_text(json.dumps(other))
+    with pytest.raises(TokenizerError, match="model type 'WordLevel'.*byte_level_bpe"):
+        load_tokenizer(str(folder))
+    # ... until a kind that reads it is registered, from outside the package.
+
+    class Words:
+        def __init__(self, data):
+            self.ids = data["model"]["vocab"]
+
+        def encode(self, text):
+            return [self.ids[word] for word in text.split()]
+
+    if "toy_words" not in registered_tokenizers():
+        register_tokenizer("toy_words", lambda data: data.get("model", {}).get("type") == "WordLevel", Words)
+    assert load_tokenizer(str(folder)).encode("b a b") == [1, 0, 1]
+    with pytest.raises(ValueError, match="already registered"):
+        register_tokenizer("toy_words", lambda data: False, Words)
+    with pytest.raises(TokenizerError, match="cannot read"):
+        load_tokenizer(str(tmp_path / "nowhere"))

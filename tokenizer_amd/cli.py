@@ -110,16 +110,15 @@ def main(argv: list[str] | None = None) -> int:
         return 1
 
     from .config import load_config
-    from .engine import (Engine, GenerateParams, StopReason, generate, load_eos_token_ids, load_model,
-                         random_model)
-    from .tokenizer import Tokenizer
+    from .engine import Engine, Failure, GenerateParams, StopReason, load_eos_token_ids, load_model, random_model
+    from .tokenizer import load_tokenizer
 
     folder = args["model"]
     tokenizer = None
     if args["token_ids"]:
         prompt_ids = [int(part) for part in args["prompt"].replace(",", " ").split()]
     else:
-        tokenizer = Tokenizer.load_qwen(os.path.join(folder, "tokenizer.json"))
+        tokenizer = load_tokenizer(folder)          # of the kind the folder's tokenizer.json declares
         prompt_ids = tokenizer.encode(args["prompt"])
     if not prompt_ids:
         print("error: prompt encoded to no tokens", file=sys.stderr)
@@ -143,8 +142,14 @@ def main(argv: list[str] | None = None) -> int:
     token_bytes = (lambda token: tokenizer.decode_bytes([token])) if tokenizer else \
         (lambda token: f"{token} ".encode())
     started = time.perf_counter()
-    generated = generate(engine, prompt_ids, params, token_bytes)
+    # The request takes the way every request of a serving engine takes: queued, admitted with pages for its whole
+    # prompt, the prompt run in portions under the token budget, decoded (greedy steps in bursts), finished, freed.
+    request = engine.add_request(prompt_ids, params, token_bytes=token_bytes)
+    generated = engine.run()[request]
     elapsed = time.perf_counter() - started
+    if isinstance(generated, Failure):
+        print(f"error: {generated.message}", file=sys.stderr)
+        return 1
     print(generated.text)
     print(f"generated ids: {generated.tokens}", file=sys.stderr)
     print(f"stop: {generated.reason.value}", file=sys.stderr)

@@ -8,7 +8,7 @@ from ..cache import CacheManager, CachePools, OutOfPages
 from ..config import load_config
 from ..config.base import ModelConfig
 from ..config.registry import get_architecture
-from ..parts import DecoderModel, LayerCache, Runtime, cache_needs, expected_tensors
+from ..parts import LayerCache, Runtime, build_model, cache_needs, expected_tensors
 from ..weights import load_weights, random_tensors, stored_form
 from .batch import StepContext, StepEntry, build_context
 
@@ -33,7 +33,7 @@ class Model:
         self.device = torch.device(device)
         self.spec = get_architecture(config.architecture).build_spec(config)
         self.runtime = Runtime(self.dtype, self.device, ops if ops is not None else get_ops())
-        self.decoder = DecoderModel(self.spec, tensors, self.runtime)
+        self.decoder = build_model(self.spec, tensors, self.runtime)     # in the frame the spec names
         self.cache_needs = cache_needs(self.spec)
 
     @property

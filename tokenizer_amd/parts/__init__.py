@@ -1,11 +1,11 @@
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, Block, FeedForward, Mixer, Norm, NormFold,
+from .base import (BLOCKS, FEED_FORWARDS, FRAMES, MIXERS, NORMS, POSITIONS, Block, FeedForward, Mixer, Norm, NormFold,
                    Part, PositionEncoding, Registry, Runtime, StoreEpilogue, as_tensor)
 from .spec import (CacheNeed, FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
                    ScheduleEntry, TensorSpec)
 from . import norm, position, attention, feed_forward, block  # noqa: F401  (register the built-in parts)
-from .model import DecoderModel, LayerCache, cache_needs, expected_tensors
+from .model import DecoderModel, LayerCache, build_model, cache_needs, expected_tensors
 
-__all__ = ["BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITIONS", "Block", "FeedForward", "Mixer", "Norm",
+__all__ = ["BLOCKS", "FEED_FORWARDS", "FRAMES", "MIXERS", "NORMS", "POSITIONS", "Block", "FeedForward", "Mixer", "Norm",
            "NormFold", "Part", "PositionEncoding", "Registry", "Runtime", "StoreEpilogue", "as_tensor", "CacheNeed", "FeedForwardSpec", "LayerSpec",
            "MixerSpec", "ModelSpec", "NormSpec", "PositionSpec", "ScheduleEntry", "TensorSpec",
-           "DecoderModel", "LayerCache", "cache_needs", "expected_tensors"]
+           "DecoderModel", "LayerCache", "build_model", "cache_needs", "expected_tensors"]

@@ -28,6 +28,14 @@ Block           arranges two norms, a mixer and a feed-forward around the residu
                 be absent: None for the part and its norm):
                 forward(residual, delta, ctx, cache) -> delta still to be added.
 
+Frame           what stands around the layers: `ModelSpec.frame` names it.  Static `expected_tensors(spec)` (every
+                tensor name the model reads, with its `TensorSpec`) and `cache_needs(spec)` (one `CacheNeed` per
+                layer); built from (spec, tensors, runtime); `graph_safe`; `forward(ctx, layer_caches)` -> float32
+                logits [wanted, vocab].  The built-in "decoder" frame (`parts.model.DecoderModel`) is embedding,
+                layers in schedule order, final norm, head, with `embed(ctx)` and `logits(residual, delta, ctx)` as
+                the two places a subclass changes (a scaled embedding, a learned position table, a head bias, a cap
+                on the logits); its constants beyond the spec's fields travel in `ModelSpec.options`.
+
 Every part may also say `repeatable() -> Repeatable` (a block: `repeatable(cache)`): that on the device its forward
 does nothing but call the kernel library, and that those calls depend on the part only through the constants and the
 tensors it lists.  The model then records the calls of one such layer on a step's batch and makes them again for
@@ -79,6 +87,7 @@ POSITIONS = Registry("position encoding")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block")
+FRAMES = Registry("model frame")
 
 
 class Part:

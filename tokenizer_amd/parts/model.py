@@ -5,7 +5,7 @@ import dataclasses
 
 import torch
 
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Runtime, repeatable_of
+from .base import BLOCKS, FEED_FORWARDS, FRAMES, MIXERS, NORMS, Runtime, repeatable_of
 from .spec import CacheNeed, ModelSpec, TensorSpec
 
 
@@ -14,27 +14,18 @@ def _prefixed(prefix: str, specs: dict[str, TensorSpec]) -> dict[str, TensorSpec
 
 
 def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
-    """Every tensor name the model reads from the weight file, with its shape."""
-    out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size), std=spec.embedding_std)}
-    for layer in spec.layers:
-        if layer.mixer is not None:
-            out.update(_prefixed(layer.mixer_norm_prefix, NORMS.get(layer.mixer_norm.kind).tensor_specs(layer.mixer_norm)))
-            out.update(_prefixed(layer.mixer_prefix, MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer)))
-        if layer.feed_forward is not None:
-            out.update(_prefixed(layer.feed_forward_norm_prefix,
-                                 NORMS.get(layer.feed_forward_norm.kind).tensor_specs(layer.feed_forward_norm)))
-            out.update(_prefixed(layer.feed_forward_prefix,
-                                 FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward)))
-    out.update(_prefixed(spec.final_norm_prefix, NORMS.get(spec.final_norm.kind).tensor_specs(spec.final_norm)))
-    if not spec.tied_head:
-        out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
-    return out
+    """Every tensor name the model reads from the weight file, with its shape: its frame says."""
+    return FRAMES.get(spec.frame).expected_tensors(spec)
 
 
 def cache_needs(spec: ModelSpec) -> list[CacheNeed]:
-    """What each layer's mixer asks of the cache manager, by layer index (a layer without a mixer: nothing)."""
-    return [MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) if layer.mixer is not None else CacheNeed()
-            for layer in spec.layers]
+    """What each layer asks of the cache manager, by layer index: the model's frame says."""
+    return FRAMES.get(spec.frame).cache_needs(spec)
+
+
+def build_model(spec: ModelSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
+    """The model of `spec` in the frame it names."""
+    return FRAMES.get(spec.frame)(spec, tensors, runtime)
 
 
 def _strip(prefix: str, tensors: dict[str, torch.Tensor]) -> dict[str, torch.Tensor]:
@@ -123,9 +114,35 @@ def _addresses_put(recorded: tuple, wanted: tuple):
     return {a: b for a, b in put.items() if a != b}
 
 
+@FRAMES.register("decoder")
 class DecoderModel:
-    """Weights and parts of one model.  It owns no cache: `forward` is handed the step's context
-    (token ids, positions, block tables) and one `LayerCache` per schedule entry."""
+    """Weights and parts of one model: embedding, layers in schedule order, final norm, head.  It owns no cache:
+    `forward` is handed the step's context (token ids, positions, block tables) and one `LayerCache` per schedule
+    entry.  A frame that differs only before the first layer or behind the last overrides `embed` or `logits`
+    (and `expected_tensors`, if it reads tensors of its own)."""
+
+    @staticmethod
+    def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
+        out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size), std=spec.embedding_std)}
+        for layer in spec.layers:
+            if layer.mixer is not None:
+                out.update(_prefixed(layer.mixer_norm_prefix, NORMS.get(layer.mixer_norm.kind).tensor_specs(layer.mixer_norm)))
+                out.update(_prefixed(layer.mixer_prefix, MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer)))
+            if layer.feed_forward is not None:
+                out.update(_prefixed(layer.feed_forward_norm_prefix,
+                                     NORMS.get(layer.feed_forward_norm.kind).tensor_specs(layer.feed_forward_norm)))
+                out.update(_prefixed(layer.feed_forward_prefix,
+                                     FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward)))
+        out.update(_prefixed(spec.final_norm_prefix, NORMS.get(spec.final_norm.kind).tensor_specs(spec.final_norm)))
+        if not spec.tied_head:
+            out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
+        return out
+
+    @staticmethod
+    def cache_needs(spec: ModelSpec) -> list[CacheNeed]:
+        """(A layer without a mixer asks for nothing.)"""
+        return [MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) if layer.mixer is not None else CacheNeed()
+                for layer in spec.layers]
 
     def __init__(self, spec: ModelSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.spec, self.runtime = spec, runtime
@@ -164,11 +181,22 @@ class DecoderModel:
             cache.makes[layer] = make
         return cache.makes[layer]
 
+    def embed(self, ctx) -> torch.Tensor:
+        """The float32 residual stream [tokens, hidden] the first layer starts from."""
+        residual = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.runtime.device)
+        return self.runtime.ops.embedding(ctx.token_ids, self.embedding, residual)
+
+    def logits(self, residual: torch.Tensor, delta, ctx) -> torch.Tensor:
+        """Float32 logits at the wanted rows from the stream and what is still to be added to it.  Only the wanted
+        rows are normalised and multiplied with the head (the reference keeps the last row,
+        qwen-infer/src/model.rs:1224-1242)."""
+        wanted = self.final_norm.apply(residual, delta, rows=ctx.want_rows)
+        return self.runtime.ops.linear(wanted, self.head, out_dtype=torch.float32)
+
     def forward(self, ctx, layer_caches: list[LayerCache]) -> torch.Tensor:
         """Run the tokens of `ctx` through the schedule; float32 logits [len(want_rows), vocab]."""
         ops = self.runtime.ops
-        residual = torch.empty((ctx.n_tokens, self.spec.hidden_size), dtype=torch.float32, device=self.runtime.device)
-        ops.embedding(ctx.token_ids, self.embedding, residual)
+        residual = self.embed(ctx)
         delta = None
         # Like layers make the same library calls on a batch: the calls of the first are recorded and made again
         # for the others with their tensors' addresses put in place, which spares those layers' Python (about
@@ -212,7 +240,4 @@ class DecoderModel:
             delta = recorded.result               # the recorded layer's buffers hold this layer's output now
         if ctx.want_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.runtime.device)
-        # Only the wanted rows are normalised and multiplied with the head (the reference keeps
-        # the last row, qwen-infer/src/model.rs:1224-1242).
-        wanted = self.final_norm.apply(residual, delta, rows=ctx.want_rows)
-        return ops.linear(wanted, self.head, out_dtype=torch.float32)
+        return self.logits(residual, delta, ctx)

@@ -143,3 +143,5 @@ class ModelSpec:
     tied_head: bool
     head_name: str                # used when the head is not tied
     embedding_std: float = 0.02
+    frame: str = "decoder"        # what stands around the layers (`parts.base.FRAMES`)
+    options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)   # the frame's own constants

@@ -33,6 +33,29 @@ class UnknownToken(TokenizerError):
         self.token = token
 
 
+def read_tokenizer_json(path: str) -> dict:
+    try:
+        with open(path, encoding="utf-8") as fh:
+            data = json.load(fh)
+    except OSError as err:
+        raise TokenizerError(f"cannot read {path}: {err}") from None
+    except json.JSONDecodeError as err:
+        raise TokenizerError(f"{path} is not valid JSON: {err}") from None
+    if not isinstance(data, dict):
+        raise TokenizerError(f"{path} does not hold an object")
+    return data
+
+
+def declares_byte_level_bpe(data: dict) -> bool:
+    """Whether a parsed tokenizer.json declares the kind this module reads: a BPE model behind a ByteLevel
+    pre-tokenizer step (alone or in a Sequence)."""
+    model, pre = data.get("model"), data.get("pre_tokenizer")
+    if not isinstance(model, dict) or model.get("type") != "BPE" or not isinstance(pre, dict):
+        return False
+    steps = pre.get("pretokenizers") if pre.get("type") == "Sequence" else [pre]
+    return any(isinstance(step, dict) and step.get("type") == "ByteLevel" for step in steps or [])
+
+
 # ------------------------------------------------------------------------------------ the byte alphabet
 _SELF_SPELLED = (range(0x21, 0x7F), range(0xA1, 0xAD), range(0xAE, 0x100))     # printable, kept as they are
 
@@ -229,14 +252,13 @@ class Tokenizer:
     # -------------------------------------------------------------------- loading
     @classmethod
     def load_qwen(cls, path: str) -> "Tokenizer":
-        try:
-            with open(path, encoding="utf-8") as fh:
-                data = json.load(fh)
-        except OSError as err:
-            raise TokenizerError(f"cannot read {path}: {err}") from None
-        except json.JSONDecodeError as err:
-            raise TokenizerError(f"{path} is not valid JSON: {err}") from None
-        return cls.from_json(data)
+        return cls.from_json(read_tokenizer_json(path))
+
+    @staticmethod
+    def load(path: str):
+        """The tokenizer of a model folder or tokenizer.json, of whichever registered kind the file declares."""
+        from . import load_tokenizer
+        return load_tokenizer(path)
 
     @classmethod
     def from_json(cls, data: dict) -> "Tokenizer":
