@@ -220,19 +220,23 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
 
 
 def measure_peaks() -> dict:
-    """What this device reaches on the two yardsticks of the rooflines: reading a large buffer once (a library
-    reduction over 4 GiB) and a large square bf16 product through the library."""
+    """What this device reaches on the two yardsticks of the rooflines: reading a large buffer once (4 GiB, by a
+    library reduction and by the package's own read loop in the access pattern of its weight-streaming kernels;
+    the higher of the two counts) and a large square bf16 product through the library."""
     import torch
+    from tokenizer_amd.kernels import get_ops
     out = {}
     big = torch.empty(1 << 30, dtype=torch.float32, device="cuda:0").fill_(1.0)
-    for _ in range(2):
-        big.sum()
-    torch.cuda.synchronize()
-    started = time.perf_counter()
-    for _ in range(10):
-        big.sum()
-    torch.cuda.synchronize()
-    out["hbm_read_gbs"] = round(10 * big.numel() * 4 / (time.perf_counter() - started) / 1e9, 1)
+    for name, read in (("hbm_read_library_gbs", big.sum), ("hbm_read_loop_gbs", lambda: get_ops().read_stream(big))):
+        for _ in range(2):
+            read()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        for _ in range(10):
+            read()
+        torch.cuda.synchronize()
+        out[name] = round(10 * big.numel() * 4 / (time.perf_counter() - started) / 1e9, 1)
+    out["hbm_read_gbs"] = max(out["hbm_read_library_gbs"], out["hbm_read_loop_gbs"])
     del big
     n = 8192
     a = torch.randn(n, n, device="cuda:0").to(torch.bfloat16)
@@ -401,14 +405,22 @@ def main() -> int:
         points = {}
         for batch, steps in ((1, args.steps), (64, args.steps)):
             log(f"decode at batch {batch}: {steps} timed steps")
-            e, _ = run_decode(model, batch, steps, min(args.warmup, 4))
+            e, kv = run_decode(model, batch, steps, min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(batch * steps / e, 1)
+            # The same roofline figures as for the main batch: a step's time, the bytes it has to read (weights
+            # once, the live requests' keys and values), and their quotient against the published bandwidth.
+            gb = (weights + batch * kv * kv_token) / 1e9
+            points[f"decode_b{batch}_ms"] = round(e / steps * 1e3, 4)
+            points[f"decode_b{batch}_gb"] = round(gb, 4)
+            points[f"decode_b{batch}_hbm_frac"] = round(gb / (e / steps) / HBM_GBS, 4)
         record["points"] = points
         # The same two fractions against what this device reaches on the yardsticks themselves (a large read,
         # a large square product through the library), beside those against the published peaks.
         log("what the device reaches: a 4 GiB read and an 8,192-cubed bf16 product")
         reached = measure_peaks()
+        record["roofline"]["step_gb"] = round(step_bytes / 1e9, 4)
         record["roofline"]["measured_peak"] = reached["hbm_read_gbs"]
+        record["roofline"]["measured_peak_library_sum"] = reached["hbm_read_library_gbs"]
         record["roofline"]["frac_of_measured"] = round(achieved / reached["hbm_read_gbs"], 4)
         if args.dtype == "bfloat16":
             record["prefill"]["measured_peak_tflops"] = reached["bf16_gemm_tflops"]

@@ -994,3 +994,13 @@ def test_fused_products_for_every_cut(ops, ref, rows, waves):
     res_b = residual.clone()
     ref.linear_add(got, down, bias, res_b)
     torch.testing.assert_close(res_a, res_b, **linear_tol(torch.float32, got, down))
+
+
+def test_read_stream_reads_every_word_once(ops):
+    """The bandwidth yardstick leaves the xor of all it read: equal to the xor of the buffer's words, at sizes that
+    are and are not multiples of its eight loads a lane, with few and many workgroups."""
+    import numpy as np
+    for words, workgroups in ((4, 1), (256 * 8 * 4 * 3, 3), (1_000_000, 64), (12_345_680, None)):
+        data = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), dtype=torch.int32, device="cuda")
+        parts = ops.read_stream(data, workgroups).cpu().numpy().view(np.uint32)
+        assert int(np.bitwise_xor.reduce(parts)) == int(np.bitwise_xor.reduce(data.cpu().numpy().view(np.uint32))), words

@@ -250,3 +250,38 @@ extern "C" int ta_silu_gate(const void* in, void* out, int n_tokens, int inner, 
 
 // The number of compute units that the launchers plan for (the current device's).
 extern "C" int ta_compute_units() { return compute_units(); }
+
+// A yardstick, not a model kernel: reads `n16` words of sixteen bytes once, in the access pattern of the
+// weight-streaming kernels (a wave instruction reads 1 KB of one run, eight such loads of a lane in flight), and
+// leaves the xor of everything it read per workgroup in `out` so that no load can be dropped.  What it reaches is
+// what a kernel bound by HBM can reach on this device.
+typedef uint32_t word4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) read_stream_kernel(const word4* __restrict__ p, size_t n16, uint32_t* __restrict__ out) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  uint32_t acc = 0;
+  for (; i + 7 * stride < n16; i += 8 * stride) {
+    word4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(p + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < n16; i += stride) {
+    const word4 v = __builtin_nontemporal_load(p + i);
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, WAVE);
+  __shared__ uint32_t parts[4];
+  if ((threadIdx.x & 63) == 0) parts[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = parts[0] ^ parts[1] ^ parts[2] ^ parts[3];
+}
+
+// out: uint32 [workgroups]; bytes a multiple of 16; data 16-byte aligned.
+extern "C" int ta_read_stream(const void* data, size_t bytes, void* out, int workgroups, hipStream_t stream) {
+  if (bytes % 16 || workgroups <= 0 || ((uintptr_t)data & 15)) return -1;
+  read_stream_kernel<<<workgroups, 256, 0, stream>>>((const word4*)data, bytes / 16, (uint32_t*)out);
+  return LAUNCH_STATUS();
+}

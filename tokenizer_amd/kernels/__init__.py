@@ -152,7 +152,7 @@ class Ops:
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_sample",
-                     "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units"):
+                     "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
@@ -197,6 +197,20 @@ class Ops:
             yield tape
         finally:
             _RECORDING.library, _RECORDING.keep = before
+
+    # ------------------------------------------------------------------ yardstick
+    def read_stream(self, data: torch.Tensor, workgroups: int | None = None) -> torch.Tensor:
+        """Read every byte of `data` once in the access pattern of the weight-streaming kernels; returns the xor
+        of its 32-bit words per workgroup (uint32 as int32 [workgroups]).  A yardstick for what a kernel bound by
+        HBM reaches on this device; no model code calls it."""
+        _dev(data)
+        nbytes = data.numel() * data.element_size()
+        _need(nbytes % 16 == 0 and data.data_ptr() % 16 == 0, "the buffer must be whole 16-byte words")
+        workgroups = workgroups or 8 * self.compute_units
+        out = torch.empty(workgroups, dtype=torch.int32, device=data.device)
+        self._check(self.lib.ta_read_stream(_ptr(data), ctypes.c_size_t(nbytes), _ptr(out), workgroups, self._stream()),
+                    "read_stream")
+        return out
 
     # ------------------------------------------------------------------ embedding
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
