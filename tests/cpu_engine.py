@@ -5,7 +5,7 @@ import torch
 from kernel_refs import PlainOps
 
 
-def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_size=16, counting=True):
+def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_size=16, counting=True, bursts=False):
     from tokenizer_amd.engine import Engine, load_model
     model = load_model(folder, "float32", "cpu", ops=PlainOps())
     engine = Engine(model, num_pages=num_pages, page_size=page_size, max_requests=max_requests, prefix_cache=prefix_cache)
@@ -19,4 +19,34 @@ def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_si
 
     if counting:
         engine.step = step
+
+    def decode_greedy(rids, tokens, n_steps, on_step=None):
+        """`Engine.decode_greedy` as it behaves with captured graphs, one step at a time on the CPU: the ids of a
+        step reach `on_step` one step late, when the next step has already run, and when `on_step` returns False
+        the run ends behind that further step, whose ids are returned as well."""
+        from tokenizer_amd.engine import StepEntry
+        if n_steps <= 0:
+            return []
+        ran, picked, current, go_on = [], [], [int(t) for t in tokens], True
+        for k in range(n_steps):
+            entries = [StepEntry(rid, [token], [0]) for rid, token in zip(rids, current)]
+            current = [int(t) for t in engine.argmax(engine.step(entries))]
+            ran.append(current)
+            if k > 0:
+                picked.append(ran[k - 1])
+                if on_step is not None and on_step(k - 1, picked[-1]) is False:
+                    go_on = False
+            if not go_on:
+                break
+        picked.append(ran[len(picked)])
+        if on_step is not None and go_on:
+            on_step(len(picked) - 1, picked[-1])
+        return picked
+
+    # The scheduler runs greedy decode steps in bursts only over an engine that says it replays graphs; nothing is
+    # captured here, the double only takes the scheduler (and greedy `generate`) down that road when asked to.
+    if bursts:
+        engine.decode_greedy = decode_greedy
+        engine.use_graphs = True
+        engine._replays = lambda entries: False
     return engine

@@ -217,7 +217,7 @@ def test_requests_cancelled_at_random_keep_what_they_sampled(model_folders, seed
     num_pages = rng.choice([5, 8, 12, 30])
     config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 4]), num_blocks=num_pages, prefix_cache=rng.random() < 0.5,
                              max_num_batched_tokens=rng.choice([8, 24, 64]), prefill_chunk=rng.choice([None, 7, 16]))
-    engine = cpu_engine(folder, num_pages=num_pages, max_requests=config.max_batch_size,
+    engine = cpu_engine(folder, bursts=True, num_pages=num_pages, max_requests=config.max_batch_size,
                         prefix_cache=config.prefix_cache, counting=False)
     sched = Scheduler(engine, config)
     token_bytes = lambda token: bytes([97 + token % 7])
@@ -272,7 +272,7 @@ def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed
     config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 3, 5]), num_blocks=num_pages,
                              prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 16, 40]),
                              prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64)
-    engine = cpu_engine(folder, num_pages=num_pages, max_requests=config.max_batch_size,
+    engine = cpu_engine(folder, bursts=True, num_pages=num_pages, max_requests=config.max_batch_size,
                         prefix_cache=config.prefix_cache)
     sched = Scheduler(engine, config)
     shared = random_ids(256, 35, 900 + seed)
@@ -367,7 +367,7 @@ def test_requests_of_every_kind_get_what_they_get_alone(model_folders, seed):
     request equal those of the request generated alone (qwen-server/src/engine.rs:1328-1420 widened)."""
     name = "ABC"[seed % 3]
     vocab = {"A": 256, "B": 384, "C": 320}[name]
-    run_requests_of_every_kind(lambda folder, **kw: cpu_engine(folder, counting=False, **kw), model_folders[name],
+    run_requests_of_every_kind(lambda folder, **kw: cpu_engine(folder, counting=False, bursts=True, **kw), model_folders[name],
                                vocab, seed)
 
 
@@ -399,3 +399,37 @@ def test_a_pool_made_for_so_many_tokens_holds_them_at_any_page_size(model_folder
     for rid in range(4):
         engine.end_request(rid)
     engine.cache.check_invariants()
+
+
+def test_a_burst_the_pool_cannot_hold_is_shortened_instead_of_taking_pages_early(model_folders):
+    """Three sequences decode side by side in a pool that cannot hold all of them to their ends: sooner or later one
+    is preempted.  A burst of sixteen steps asks for the pages of all of them together and is halved until the pool
+    can hold it; it never leaves some sequences with pages they do not need yet while another finds none for its
+    next token.  So bursts preempt no more often, and forward no more tokens again, than single steps do, and give
+    the same tokens."""
+    folder = model_folders["A"]
+    prompts = [random_ids(256, n, 400 + i) for i, n in enumerate([15, 9, 30])]
+    stats = {}
+    for burst in (1, 16):
+        engine = cpu_engine(folder, bursts=True, num_pages=7, max_requests=3, counting=False)
+        sched = Scheduler(engine, SchedulerConfig(max_batch_size=3, num_blocks=7, prefix_cache=False, decode_burst=burst))
+        ids = [sched.add_request(prompt, GenerateParams.greedy(24)) for prompt in prompts]
+        results = sched.run()
+        for rid, prompt in zip(ids, prompts):
+            assert results[rid].tokens == solo(folder, prompt, GenerateParams.greedy(24)).tokens
+        sched.assert_idle()
+        stats[burst] = sched.stats
+    assert stats[1].preemptions >= 1                                   # the pool is too small for all of them
+    assert stats[16].preemptions <= stats[1].preemptions
+    assert stats[16].tokens_forwarded <= stats[1].tokens_forwarded
+    # With room for everything the bursts run at full length: far fewer iterations of the scheduler than tokens.
+    engine = cpu_engine(folder, bursts=True, num_pages=12, max_requests=3, counting=False)
+    sched = Scheduler(engine, SchedulerConfig(max_batch_size=3, num_blocks=12, prefix_cache=False, decode_burst=16))
+    ids = [sched.add_request(prompt, GenerateParams.greedy(20)) for prompt in prompts]
+    steps = 0
+    while sched.has_work():
+        sched.run(max_steps=1)
+        steps += 1
+    assert steps <= 8 and sched.stats.preemptions == 0
+    for rid, prompt in zip(ids, prompts):
+        assert sched.finished[rid].tokens == solo(folder, prompt, GenerateParams.greedy(20)).tokens

@@ -268,7 +268,8 @@ class Scheduler:
         """How many decode steps may follow each other on the device without a decision of the host between them:
         more than one only when the step is nothing but greedy decoding (the ids a step picks feed the next one
         there, `Engine.decode_greedy`), nothing waits that could join, no sequence reaches its last token before
-        the burst's last step, and the pages for all those tokens are there now."""
+        the burst's last step, and the pages for all those tokens of all sequences are there now (a burst the pool
+        cannot hold whole is halved until it can)."""
         burst = min(self.config.decode_burst, 64)
         if burst < 2 or not getattr(self.engine, "use_graphs", False) or not hasattr(self.engine, "decode_greedy"):
             return 1
@@ -280,11 +281,23 @@ class Scheduler:
             if count != 1 or first < seq.prompt_len or not completes or not seq.cursor.is_greedy:
                 return 1
             burst = min(burst, seq.params.max_tokens - seq.cursor.produced)
+        # The pages for all those tokens of all the sequences are taken together or not at all: a burst that only
+        # some sequences got their pages for would leave those holding pages they do not need yet, and the next
+        # plan might then find none for another sequence's single token and preempt, where single steps would
+        # still have fitted.  A burst the pool cannot hold is halved until it can.
+        while burst >= 2:
+            missing = [0] * len(self.cache.groups)
+            for seq, first, _, _ in plan:
+                for group, pages in enumerate(self.cache.pages_missing(seq.id, first + burst)):
+                    missing[group] += pages
+            if all(pages <= group.allocator.available() for pages, group in zip(missing, self.cache.groups)):
+                break
+            burst //= 2
         if burst < 2:
             return 1
         for seq, first, _, _ in plan:
             if not self.cache.reserve(seq.id, first + burst):       # tokens first .. first + burst - 1 get their pages
-                return 1                  # (pages some of them took already are theirs a few steps early, no more)
+                return 1                  # (cannot happen after the count above; pages taken so far are theirs early, no more)
         return burst
 
     def _run_burst(self, plan: list[tuple[Sequence, int, int, bool]], burst: int) -> None:
