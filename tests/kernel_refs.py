@@ -70,6 +70,8 @@ class PlainOps:
         page_size = k_pages.shape[2]
         group = n_q // n_kv
         for t in range(qkv.shape[0]):
+            if int(entry_of_token[t]) < 0:                   # a token that only fills the batch up
+                continue
             pos = int(positions[t])
             table = block_table[int(entry_of_token[t])]
             lo = max(0, pos - window) if window is not None else 0

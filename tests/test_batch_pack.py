@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from tokenizer_amd.cache import CacheManager
-from tokenizer_amd.engine.batch import StepEntry, build_context
+from tokenizer_amd.engine.batch import StepEntry, build_context, filled_counts
 from tokenizer_amd.parts.spec import CacheNeed
 
 
@@ -15,7 +15,9 @@ def needs():
     return [CacheNeed("full", 2, 16), CacheNeed("window", 2, 16, window=20), CacheNeed("none"), CacheNeed("full", 2, 16)]
 
 
-def expected_parts(manager, entries, table_width):
+def expected_parts(manager, entries, table_width, filled=None):
+    """The parts of a step's description; `filled`: the counts (tokens, entries, wanted places, tiles, single rows) it
+    is filled up to with parts that do nothing."""
     page = manager.page_size
     token_ids, positions, entry_of, cu_q, first, state, want, tiles, single = [], [], [], [0], [], [], [], [], []
     for e, entry in enumerate(entries):
@@ -32,6 +34,20 @@ def expected_parts(manager, entries, table_width):
         else:
             for offset in range(0, count, 16):
                 tiles += [e, offset]
+    real_tokens, real_entries = len(token_ids), len(entries)
+    more_tokens = more_entries = 0
+    if filled is not None:
+        n_tokens, n_entries, n_want, n_tiles, n_single = filled
+        more_tokens, more_entries = n_tokens - real_tokens, n_entries - real_entries
+        token_ids += [0] * more_tokens                            # a token of no request: id 0 at position 0,
+        positions += [0] * more_tokens
+        entry_of += [-1] * more_tokens                            # no entry
+        cu_q += [real_tokens] * more_entries                      # an entry without rows
+        first += [0] * more_entries
+        state += [0] * more_entries
+        want += [0] * (n_want - len(want))                        # a wanted place nobody looks at: row 0
+        tiles += [real_entries, 0] * (n_tiles - len(tiles) // 2)  # a tile in the first entry without rows
+        single += [-1] * (n_single - len(single))                 # no row
     parts = [token_ids, positions, entry_of, cu_q, first, state, want, tiles, single]
     for g in range(len(manager.groups)):
         tables = [manager.table(entry.rid, g) for entry in entries]
@@ -40,16 +56,19 @@ def expected_parts(manager, entries, table_width):
         for entry, table in zip(entries, tables):
             start = manager.seq_len(entry.rid)
             slots += [table[p // page] * page + p % page for p in range(start, start + len(entry.tokens))]
+        slots += [-1] * more_tokens                               # and no slot
         flat = []
         for table in tables:
             flat += table[:width] + [-1] * (width - len(table))     # pages held beyond a fixed width are left out
+        flat += [-1] * (width * more_entries)
         parts += [slots, flat]
     return parts
 
 
 @pytest.mark.parametrize("seed", range(6))
 @pytest.mark.parametrize("table_width", [None, 12])
-def test_packed_batch_matches_its_definition(seed, table_width):
+@pytest.mark.parametrize("fill", [False, True])
+def test_packed_batch_matches_its_definition(seed, table_width, fill):
     rng = random.Random(seed)
     manager = CacheManager(needs(), num_pages=40, page_size=16, max_requests=5)
     rids = ["a", 7, ("t", 1), 12345678901]                    # names, small integers and large ones alike
@@ -68,8 +87,11 @@ def test_packed_batch_matches_its_definition(seed, table_width):
         want = sorted(rng.sample(range(count), rng.randint(0, min(3, count))))
         assert manager.reserve(rid, lengths[rid] + count)
         entries.append(StepEntry(rid, tokens, want))
-    ctx = build_context(entries, manager, "cpu", table_width=table_width)
-    parts = expected_parts(manager, entries, table_width)
+    ctx = build_context(entries, manager, "cpu", table_width=table_width, fill=fill)
+    filled = filled_counts([len(e.tokens) for e in entries], [len(e.want) for e in entries]) if fill else None
+    parts = expected_parts(manager, entries, table_width, filled)
+    if fill:
+        assert (ctx.n_tokens, ctx.n_entries) == filled[:2] and ctx.n_wanted == sum(len(e.want) for e in entries)
     got = [ctx.token_ids, ctx.positions, ctx.entry_of_token, ctx.cu_q, ctx.first_position, ctx.state_slots,
            ctx.want_rows, ctx.q_tiles.reshape(-1), ctx.decode_rows]
     for g in range(len(manager.groups)):
@@ -125,3 +147,39 @@ def test_packing_refuses_what_does_not_fit():
     total, sizes, widths, info = manager.pack_batch(["b"], [[5]], [[0]], out)
     assert sizes[0] == 1 and info == [[0, 1, 64, manager.slot("b")]]
     assert manager.table("b", 1)[:2] == [-1, -1]                                       # behind the window of 20
+
+
+def test_the_counts_a_step_is_filled_up_to():
+    """Steps of single tokens stay as they are; any other step is rounded up to counts that steps which differ a
+    little share: always room for one entry without rows (where a tile that does nothing lies), tokens in steps of 8
+    up to 64 (where the kernels change with the row count) and of 64 beyond."""
+    assert filled_counts([1, 1, 1], [1, 1, 1]) == (3, 3, 3, 0, 3)
+    assert filled_counts([1], [0]) == (1, 1, 0, 0, 1)
+    assert filled_counts([5], [5]) == (8, 4, 8, 5, 0)
+    assert filled_counts([2, 1], [0, 1]) == (8, 12, 8, 5, 8)
+    assert filled_counts([137, 1, 1, 1], [1, 1, 1, 1]) == (192, 12, 8, 16, 8)
+    assert filled_counts([140] + [1] * 3, [0] + [1] * 3) == filled_counts([131, 20] + [1] * 5, [1, 0] + [1] * 5)
+    assert filled_counts([448] + [1] * 64, [1] * 65) == filled_counts([430, 9, 11] + [1] * 62, [1, 1, 1] + [1] * 62) \
+        == (512, 68, 72, 36, 64)
+    # Filled counts are never below the real ones, whatever the batch.
+    rng = random.Random(1)
+    for _ in range(300):
+        counts = [rng.choice([1, 1, 1, 2, 15, 16, 17, 64, 300]) for _ in range(rng.randint(1, 70))]
+        wants = [rng.randint(0, min(3, c)) for c in counts]
+        tokens, entries, wanted, tiles, single = filled_counts(counts, wants)
+        real_tiles = sum(-(-c // 16) for c in counts if c != 1)
+        real_single = sum(1 for c in counts if c == 1)
+        assert tokens >= sum(counts) and wanted >= sum(wants) and tiles >= real_tiles and single >= real_single
+        assert entries >= len(counts) and (entries > len(counts) or real_single == len(counts))
+
+
+def test_counts_below_the_batchs_are_refused():
+    manager = CacheManager([CacheNeed("full", 2, 16)], num_pages=8, page_size=16, max_requests=2)
+    manager.add_request("a")
+    assert manager.reserve("a", 20)
+    out = np.zeros(4096, dtype=np.int32)
+    for too_small in ((19, 2, 0, 4, 0), (24, 1, 0, 4, 0), (24, 2, 0, 1, 0)):      # (more tiles than real ones need an entry more)
+        with pytest.raises(ValueError, match="smaller"):
+            manager.pack_batch(["a"], [list(range(20))], [[]], out, None, too_small)
+    total, sizes, _, _ = manager.pack_batch(["a"], [list(range(20))], [[]], out, None, (24, 2, 8, 4, 0))
+    assert sizes[:9] == [24, 24, 24, 3, 2, 2, 8, 8, 0]

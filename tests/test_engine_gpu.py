@@ -400,17 +400,24 @@ def test_recurring_step_shapes_replay_graphs_and_equal_eager_steps(model_folders
         both(lambda: [StepEntry(1, take(7 + k), [])])     # shapes that never recur stay eager
     for _ in range(2):
         both(lambda: [StepEntry(3, take(96), [95])])      # the first shape again, for another request
-    for n in (13, 14, 15, 16):                            # more shapes than graphs are kept
-        for _ in range(4):
+    # Portions of 13 to 16 tokens are filled up to the same counts: one shape, one graph, whatever the length.
+    before = len(engines[0].graphs)
+    for n in (13, 14, 15, 16, 16, 13):
+        both(lambda: [StepEntry(1, take(n), [n - 1])])
+    assert len(engines[0].graphs) == before + 1
+    shape_of = lambda n: Engine._shape_of([StepEntry(3, [0] * n, [n - 1])])
+    assert shape_of(13) == shape_of(16) != shape_of(17)
+    for n in (20, 28, 36):                                # more shapes than graphs are kept
+        for _ in range(3):
             both(lambda: [StepEntry(3, take(n), [n - 1])])
     kept = [key[0] for key in engines[0].graphs if not isinstance(key[0], int)]
-    assert sorted(kept) == [((14, 1),), ((15, 1),), ((16, 1),)]          # the idle ones made room
-    for n in (14, 15, 16):
-        both(lambda: [StepEntry(1, take(n), [n - 1])])    # all three in use again ...
+    assert sorted(kept) == sorted(shape_of(n) for n in (20, 28, 36))          # the idle ones made room
+    for n in (19, 27, 35):
+        both(lambda: [StepEntry(1, take(n), [n - 1])])    # all three in use again (by portions a little shorter) ...
     for _ in range(3):
-        both(lambda: [StepEntry(1, take(17), [16])])      # ... so a further shape finds no room and runs eagerly
+        both(lambda: [StepEntry(1, take(44), [43])])      # ... so a further shape finds no room and runs eagerly
     kept = [key[0] for key in engines[0].graphs if not isinstance(key[0], int)]
-    assert sorted(kept) == [((14, 1),), ((15, 1),), ((16, 1),)]
+    assert sorted(kept) == sorted(shape_of(n) for n in (20, 28, 36))
     for eng in engines:
         eng.cache.check_invariants()
 

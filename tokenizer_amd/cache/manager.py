@@ -263,10 +263,13 @@ class CacheManager:
         self._lib.ta_cache_publish(self._core, self._handle_of(rid), pointer, len(keep))
 
     # ------------------------------------------------------------------- packing
-    def pack_batch(self, rids, token_lists, want_lists, out: np.ndarray, table_width: int | None = None):
+    def pack_batch(self, rids, token_lists, want_lists, out: np.ndarray, table_width: int | None = None,
+                   padded: tuple | None = None):
         """Write one step's batch description into the int32 array `out` (see `engine/batch.py` for the
-        order of its parts).  Returns (total length, the parts' lengths, the table width per group, and per
-        entry its first row, token count, first position and state slot)."""
+        order of its parts).  `padded`: five counts (tokens, entries, wanted places, tiles of sixteen prompt
+        tokens, single rows) up to which the description is filled with parts that do nothing.  Returns (total
+        length, the parts' lengths, the table width per group, and per entry its first row, token count, first
+        position and state slot)."""
         n = len(rids)
         ids = np.array([rid if _is_handle(rid) else self._ids[rid] for rid in rids], dtype=np.int64)
         n_tokens = np.array([len(t) for t in token_lists], dtype=np.int32)
@@ -282,10 +285,14 @@ class CacheManager:
         info = np.zeros(max(1, 4 * n), dtype=np.int32)
         as_i32 = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
         as_i64 = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int64))
+        fill = None if padded is None else np.asarray(padded, dtype=np.int64)
         total = self._lib.ta_cache_pack_batch(self._core, n, as_i64(ids), as_i32(n_tokens), as_i32(tokens),
                                               as_i32(n_want), as_i32(want),
-                                              -1 if table_width is None else table_width, as_i32(out), out.size,
+                                              -1 if table_width is None else table_width,
+                                              None if fill is None else as_i64(fill), as_i32(out), out.size,
                                               as_i64(sizes), as_i32(widths), as_i32(info))
+        if total == -9:
+            raise ValueError("an entry without tokens, or counts to fill up to that are smaller than the batch's")
         if total == -3:
             raise KeyError("a request of the batch is not live")
         if total == -5:
@@ -300,12 +307,16 @@ class CacheManager:
             raise RuntimeError(f"the batch could not be packed (status {total})")
         return int(total), sizes.tolist(), widths[:n_groups].tolist(), info[:4 * n].reshape(n, 4).tolist()
 
-    def packed_size(self, token_counts, want_counts, table_widths) -> int:
-        """Length of the packed description of a batch with these token and want counts and table widths."""
-        n, tokens = len(token_counts), sum(token_counts)
-        tiles = sum(-(-c // 16) for c in token_counts if c != 1)
-        single = sum(1 for c in token_counts if c == 1)
-        return (3 * tokens + (n + 1) + 2 * n + sum(want_counts) + 2 * tiles + single
+    def packed_size(self, token_counts, want_counts, table_widths, padded: tuple | None = None) -> int:
+        """Length of the packed description of a batch with these token and want counts and table widths (filled up
+        to the counts of `padded`, if given)."""
+        if padded is not None:
+            tokens, n, wanted, tiles, single = padded
+        else:
+            n, tokens, wanted = len(token_counts), sum(token_counts), sum(want_counts)
+            tiles = sum(-(-c // 16) for c in token_counts if c != 1)
+            single = sum(1 for c in token_counts if c == 1)
+        return (3 * tokens + (n + 1) + 2 * n + wanted + 2 * tiles + single
                 + sum(tokens + n * w for w in table_widths))
 
     # ------------------------------------------------------------------ checking

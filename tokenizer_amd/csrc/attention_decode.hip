@@ -22,7 +22,7 @@ __device__ __forceinline__ bf16x8 zero8() {
 }
 
 // D: head size (multiple of 16).  Pages: K [n_pages, n_kv, page_size, D], V^T [n_pages, n_kv, D, page_size],
-// page_size a multiple of 16.  rows: the token rows to serve (null: row i = item i).
+// page_size a multiple of 16.  rows: the token rows to serve (null: row i = item i; a negative row is passed over).
 // Token at position p sees keys max(0, p - window)..p (window < 0: from 0).
 // Partials: part_o [n_items, n_q, splits, D] (unnormalised), part_ml [n_items, n_q, splits, 2] (max, sum);
 // with splits == 1 the result goes straight to `out` [n_tokens, n_q * D].
@@ -46,6 +46,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int item = blockIdx.z;
   const int t = rows ? __builtin_amdgcn_readfirstlane(rows[item]) : item;   // the same for every lane: scalar
+  if (t < 0) return;                                       // a row that only fills the list up: nothing to do
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int heads_here = min(16, group - hb * 16);
@@ -245,6 +246,7 @@ decode_attention_merge(const float* __restrict__ part_o, const float* __restrict
                        const int* __restrict__ tiles, const int* __restrict__ cu_q) {
   const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
   int t = rows ? rows[item] : item;
+  if (t < 0) return;
   if (tiles) {
     // Items are (tile, token of the tile): the output row is the tile's first row + the token; a tile's padding
     // has no row.

@@ -8,7 +8,7 @@
 
 // q: rows of `q_stride` elements, head h at h*d.  out: [n_tokens, n_q*d].
 // Token t at position p of entry e sees keys max(0, p-window)..p (window < 0: all from 0), whose
-// pages are block_table[e, key / page_size].  Key pages: [n_pages, n_kv, page_size, d]; value pages
+// pages are block_table[e, key / page_size]; a token of entry -1 is passed over (its output row is not written).  Key pages: [n_pages, n_kv, page_size, d]; value pages
 // are transposed inside a page: [n_pages, n_kv, d, page_size].
 template <typename T>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
@@ -23,8 +23,10 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   __shared__ float p_s[ATT_WAVES][WAVE];
   const int t = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int entry = entry_of_token[t];
+  if (entry < 0) return;                                   // a token that only fills the batch up: it belongs to no request
   const int pos = positions[t];
-  const int* table = block_table + (size_t)entry_of_token[t] * table_stride;
+  const int* table = block_table + (size_t)entry * table_stride;
   const int kvh = h / (n_q / n_kv);
   const int lo = (window >= 0 && pos > window) ? pos - window : 0;
   const int n_keys = pos - lo + 1;

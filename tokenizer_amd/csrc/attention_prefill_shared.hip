@@ -281,6 +281,7 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   const int offset = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index + 1]);
   const int row0 = __builtin_amdgcn_readfirstlane(cu_q[entry]) + offset;
   const int n_valid = min(16, __builtin_amdgcn_readfirstlane(cu_q[entry + 1]) - row0);
+  if (n_valid <= 0) return;                                // a tile that only fills the list up (its entry has no rows)
   const int p0 = __builtin_amdgcn_readfirstlane(first_position[entry]) + offset;   // position of the tile's first token
   const int my_pos = p0 + min(col, n_valid - 1);          // padded columns repeat the last token
   const int my_row = row0 + min(col, n_valid - 1);

@@ -146,9 +146,9 @@ int ta_cache_check(void* c) {
   return g_message.empty() ? 0 : 1;
 }
 int64_t ta_cache_pack_batch(void* c, int n_entries, const int64_t* ids, const int* n_tokens, const int32_t* tokens,
-                            const int* n_want, const int* want, int table_width, int32_t* out, int64_t capacity,
-                            int64_t* sizes, int* widths, int* entry_info) {
-  return ((CacheCore*)c)->pack_batch(n_entries, ids, n_tokens, tokens, n_want, want, table_width, out, capacity,
+                            const int* n_want, const int* want, int table_width, const int64_t* padded, int32_t* out,
+                            int64_t capacity, int64_t* sizes, int* widths, int* entry_info) {
+  return ((CacheCore*)c)->pack_batch(n_entries, ids, n_tokens, tokens, n_want, want, table_width, padded, out, capacity,
                                      sizes, widths, entry_info);
 }
 

@@ -197,29 +197,42 @@ std::string CacheCore::check_invariants() const {
 }
 
 int64_t CacheCore::pack_batch(int n_entries, const int64_t* ids, const int* n_tokens, const int32_t* tokens,
-                              const int* n_want, const int* want, int table_width, int32_t* out,
-                              int64_t capacity, int64_t* sizes, int* widths, int* entry_info) const {
+                              const int* n_want, const int* want, int table_width, const int64_t* padded,
+                              int32_t* out, int64_t capacity, int64_t* sizes, int* widths, int* entry_info) const {
   const int n_groups = (int)groups_.size();
   std::vector<const Request*> requests(n_entries);
-  int64_t total_tokens = 0, total_want = 0, n_tiles = 0, n_single = 0;
+  int64_t real_tokens = 0, real_want = 0, real_tiles = 0, real_single = 0;
   for (int e = 0; e < n_entries; ++e) {
     requests[e] = find(ids[e]);
     if (!requests[e]) return CACHE_UNKNOWN_REQUEST;
     if (n_tokens[e] <= 0 || n_want[e] < 0) return CACHE_BAD_ARGUMENT;
-    total_tokens += n_tokens[e];
-    total_want += n_want[e];
-    if (n_tokens[e] == 1) ++n_single; else n_tiles += (n_tokens[e] + 15) / 16;
+    real_tokens += n_tokens[e];
+    real_want += n_want[e];
+    if (n_tokens[e] == 1) ++real_single; else real_tiles += (n_tokens[e] + 15) / 16;
+  }
+  // The description may be filled up to given counts (tokens, entries, wanted places, tiles, single rows) with
+  // parts that do nothing: so that steps whose counts differ a little have the same layout and launch sizes.
+  // A token past the real ones has id 0, position 0, no entry (-1) and no slot (-1); an entry past the real ones
+  // has no rows and a table of -1; a wanted place past the real ones is row 0; a tile past the real ones lies in
+  // the first such entry (no rows: kernels pass it over) and a single row past the real ones is -1.
+  const int n_real_entries = n_entries;
+  int64_t total_tokens = real_tokens, total_want = real_want, n_tiles = real_tiles, n_single = real_single;
+  if (padded) {
+    if (padded[0] < real_tokens || padded[1] < n_entries || padded[2] < real_want || padded[3] < real_tiles ||
+        padded[4] < real_single || (padded[3] > real_tiles && padded[1] == n_entries))
+      return CACHE_BAD_ARGUMENT;
+    total_tokens = padded[0]; n_entries = (int)padded[1]; total_want = padded[2]; n_tiles = padded[3]; n_single = padded[4];
   }
   for (int g = 0; g < n_groups; ++g) {
     int width = 1;
     if (table_width >= 0) {
       // A fixed width has to hold the pages up to each request's last token of this step; pages a request holds
       // beyond that are left out.
-      for (int e = 0; e < n_entries; ++e)
+      for (int e = 0; e < n_real_entries; ++e)
         if (pages_for_len(requests[e]->seq_len + n_tokens[e], page_size_) > table_width) return CACHE_TABLE_TOO_WIDE;
       width = table_width;
     } else {
-      for (int e = 0; e < n_entries; ++e) width = std::max(width, (int)requests[e]->tables[g].size());
+      for (int e = 0; e < n_real_entries; ++e) width = std::max(width, (int)requests[e]->tables[g].size());
     }
     widths[g] = width;
   }
@@ -244,7 +257,10 @@ int64_t CacheCore::pack_batch(int n_entries, const int64_t* ids, const int* n_to
 
   int64_t row = 0, token_at = 0, want_at = 0;
   cu_q[0] = 0;
-  for (int e = 0; e < n_entries; ++e) {
+  int32_t* const want_end = want_rows + total_want;
+  int32_t* const tiles_end = tiles + 2 * n_tiles;
+  int32_t* const single_end = single_rows + n_single;
+  for (int e = 0; e < n_real_entries; ++e) {
     const Request& request = *requests[e];
     const int start = request.seq_len, count = n_tokens[e];
     for (int i = 0; i < count; ++i) {
@@ -269,12 +285,19 @@ int64_t CacheCore::pack_batch(int n_entries, const int64_t* ids, const int* n_to
     token_at += count;
     want_at += n_want[e];
   }
+  for (int64_t t = real_tokens; t < total_tokens; ++t) { token_ids[t] = 0; positions[t] = 0; entry_of_token[t] = -1; }
+  for (int e = n_real_entries; e < n_entries; ++e) { cu_q[e + 1] = (int32_t)real_tokens; first_position[e] = 0; state_slots[e] = 0; }
+  while (want_rows < want_end) *want_rows++ = 0;
+  while (tiles < tiles_end) { *tiles++ = n_real_entries; *tiles++ = 0; }
+  while (single_rows < single_end) *single_rows++ = -1;
   for (int g = 0; g < n_groups; ++g) {
     int32_t* slots = group_base;
     int32_t* table_out = slots + total_tokens;
     group_base = table_out + (int64_t)n_entries * widths[g];
     int64_t at = 0;
-    for (int e = 0; e < n_entries; ++e) {
+    std::fill(slots + real_tokens, slots + total_tokens, -1);
+    std::fill(table_out + (int64_t)n_real_entries * widths[g], table_out + (int64_t)n_entries * widths[g], -1);
+    for (int e = 0; e < n_real_entries; ++e) {
       const std::vector<int>& table = requests[e]->tables[g];
       const int start = requests[e]->seq_len;
       for (int i = 0; i < n_tokens[e]; ++i) {

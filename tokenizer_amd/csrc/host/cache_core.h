@@ -71,10 +71,14 @@ class CacheCore {
   // else every table is written that wide: a request may hold more pages than that (a prompt's pages are
   // reserved whole while its first portions run), as long as the pages up to its last token of this step fit,
   // since no later one is read or written in the step.
+  // padded: null, or five counts (tokens, entries, wanted places, tiles, single rows), each at least what the batch
+  // has, up to which the description is filled with parts that do nothing (a token without entry or slot, an entry
+  // without rows, a tile in such an entry, a single row of -1, a wanted place that is row 0): steps whose counts
+  // differ a little then share one layout.  More tiles than the batch has need at least one entry more.
   // sizes: 9 + 2 * groups part lengths; widths: per group.  Returns the total length or a CacheStatus.
   int64_t pack_batch(int n_entries, const int64_t* ids, const int* n_tokens, const int32_t* tokens,
-                     const int* n_want, const int* want, int table_width, int32_t* out, int64_t capacity,
-                     int64_t* sizes, int* widths, int* entry_info) const;
+                     const int* n_want, const int* want, int table_width, const int64_t* padded, int32_t* out,
+                     int64_t capacity, int64_t* sizes, int* widths, int* entry_info) const;
 
  private:
   Request* find(int64_t id);

@@ -10,7 +10,7 @@ from ..config.base import ModelConfig
 from ..config.registry import get_architecture
 from ..parts import LayerCache, Runtime, build_model, cache_needs, expected_tensors
 from ..weights import load_weights, random_tensors, stored_form
-from .batch import StepContext, StepEntry, build_context
+from .batch import StepContext, StepEntry, build_context, filled_counts
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
@@ -65,23 +65,23 @@ def random_model(config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:
 
 
 class StepGraph:
-    """One captured HIP graph of a step of one shape: so many entries with so many tokens and wanted places
-    each (a decode step: one token each), contexts of up to `bucket` tokens.  The batch's tables live in
-    fixed buffers that are refilled before every replay; the graph ends with the greedy pick, so ids are
-    ready without a further launch."""
+    """One captured HIP graph of a step of one shape (a decode step: so many requests with one token each; any
+    other step: the counts of tokens, entries, wanted places, prompt tiles and single rows its description is
+    filled up to), contexts of up to `bucket` tokens.  The batch's tables live in fixed buffers that are refilled
+    before every replay; the graph ends with the greedy pick, so ids are ready without a further launch."""
 
     def __init__(self, engine: "Engine", entries: list[StepEntry], bucket: int):
         self.bucket = bucket
         self.width = -(-bucket // engine.cache.page_size)
         device = engine.model.device
-        probe = build_context(entries, engine.cache, device, table_width=self.width)
+        probe = build_context(entries, engine.cache, device, table_width=self.width, fill=True)
         size = sum(t.numel() for t in (probe.token_ids, probe.positions, probe.entry_of_token, probe.cu_q,
                                        probe.first_position, probe.state_slots, probe.want_rows, probe.q_tiles,
                                        probe.decode_rows))
         size += sum(t.numel() for t in probe.slots) + sum(t.numel() for t in probe.block_tables)
         self.host = torch.empty(size, dtype=torch.int32).pin_memory()
         self.dev = torch.empty(size, dtype=torch.int32, device=device)
-        self.ctx = build_context(entries, engine.cache, device, table_width=self.width, into=(self.host, self.dev))
+        self.ctx = build_context(entries, engine.cache, device, table_width=self.width, into=(self.host, self.dev), fill=True)
         self.ctx.max_position = bucket - 1          # what the kernels' launch sizes are planned for
         ops = engine.model.runtime.ops
         before = getattr(ops, "capturing", False)
@@ -108,6 +108,9 @@ class StepGraph:
         """Temperature / nucleus draws for every row of this graph's logits: the sampler's twenty small launches
         are captured once (per kind: with or without the rounds of the nucleus cut) and replayed."""
         rows = self.logits.shape[0]
+        given = len(temperature)                      # (the logits' rows past these only fill the step up: drawn and dropped)
+        fill = [1.0] * (rows - given)
+        temperature, top_p, uniform = list(temperature) + fill, list(top_p) + fill, list(uniform) + [0.5] * (rows - given)
         if self.draws is None:
             self.draws = {}
             self.draw_host = torch.empty((3, rows), dtype=torch.float32).pin_memory()
@@ -128,7 +131,7 @@ class StepGraph:
             self.draws[any_cut] = captured
         else:
             captured.replay()
-        return [int(v) for v in self.draw_ids.cpu().tolist()]      # (also waits until the pinned buffer is free again)
+        return [int(v) for v in self.draw_ids.cpu().tolist()][:given]      # (also waits until the pinned buffer is free again)
 
     def run(self, engine: "Engine", entries: list[StepEntry], tokens_on_device: torch.Tensor | None = None) -> torch.Tensor:
         """Pack the batch's description into the fixed buffers again and replay.  `tokens_on_device`: the token
@@ -139,7 +142,8 @@ class StepGraph:
             self.uploaded = torch.cuda.Event()
         manager = engine.cache
         total, _, _, _ = manager.pack_batch([e.rid for e in entries], [e.packed_tokens() for e in entries],
-                                            [e.want for e in entries], self.host.numpy(), self.width)
+                                            [e.want for e in entries], self.host.numpy(), self.width,
+                                            filled_counts([len(e.tokens) for e in entries], [len(e.want) for e in entries]))
         if total != self.host.numel():
             raise ValueError("the packed batch does not fit the graph's buffers")
         self.dev.copy_(self.host, non_blocking=True)
@@ -211,8 +215,8 @@ class Engine:
     def argmax(self, logits: torch.Tensor, rows: list[int] | None = None) -> list[int]:
         """Greedy ids of the given rows of a step's logits, picked on the device."""
         graph = self._graph_result
-        if graph is not None and logits is graph.logits and graph.ids is not None:
-            picked = graph.ids.cpu().tolist()           # the graph already picked them
+        if graph is not None and self._is_result_of(logits, graph) and graph.ids is not None:
+            picked = graph.ids.cpu().tolist()[:logits.shape[0]]    # the graph already picked them (and for the rows it was filled up with)
         else:
             picked = self.model.runtime.ops.argmax(logits).cpu().tolist()
         return picked if rows is None else [picked[row] for row in rows]
@@ -225,13 +229,20 @@ class Engine:
         device = logits.device
         any_cut = any(p < 1.0 for p in top_p)
         graph = self._graph_result
-        if graph is not None and logits is graph.logits and rows == list(range(logits.shape[0])):
+        if graph is not None and self._is_result_of(logits, graph) and rows == list(range(logits.shape[0])):
             return graph.draw(self, temperature, top_p, uniform, any_cut)
         picked = logits if rows == list(range(logits.shape[0])) else logits[torch.tensor(rows, device=device)]
         # One copy to the device for the three vectors.
         packed = torch.tensor([temperature, top_p, uniform], dtype=torch.float32).to(device, non_blocking=True)
         ids = self.model.runtime.ops.sample(picked.contiguous(), packed[0], packed[1], packed[2], any_cut=any_cut)
         return [int(v) for v in ids.cpu().tolist()]
+
+    @staticmethod
+    def _is_result_of(logits: torch.Tensor, graph: "StepGraph") -> bool:
+        """Whether `logits` are the rows a replay of `graph` left (all of them, or the leading ones: those of the
+        step's real entries)."""
+        return logits is graph.logits or (logits.data_ptr() == graph.logits.data_ptr() and logits.shape[1:] == graph.logits.shape[1:]
+                                          and logits.shape[0] <= graph.logits.shape[0])
 
     def rows_to_host(self, logits: torch.Tensor, rows: list[int]):
         return logits[rows].float().cpu().numpy()
@@ -295,10 +306,13 @@ class Engine:
     @staticmethod
     def _shape_of(entries: list[StepEntry]):
         """What fixes the layout of a step's tables and the sizes of its launches: the number of entries for a
-        plain decode step, else the tokens and wanted places of every entry in order."""
-        if all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            return len(entries)
-        return tuple((len(e.tokens), len(e.want)) for e in entries)
+        plain decode step; for a step of single tokens with other wishes, those; else the counts its description is
+        filled up to (`filled_counts`), which steps that differ a little have in common."""
+        if all(len(e.tokens) == 1 for e in entries):
+            if all(list(e.want) == [0] for e in entries):
+                return len(entries)
+            return ("single",) + tuple(len(e.want) for e in entries)
+        return ("filled",) + filled_counts([len(e.tokens) for e in entries], [len(e.want) for e in entries])
 
     def _graph_key(self, entries: list[StepEntry]) -> tuple:
         longest = max(self.cache.seq_len(e.rid) + len(e.tokens) for e in entries)
@@ -430,11 +444,14 @@ class Engine:
         if reserve:
             self.reserve(entries)
         self._graph_result = None
+        wanted = sum(len(entry.want) for entry in entries)
         if self._replays(entries):
             logits = self._graph_step(entries)
         else:
-            ctx = build_context(entries, self.cache, self.model.device)
+            ctx = build_context(entries, self.cache, self.model.device, fill=True)
             logits = self.model.decoder.forward(ctx, self.layer_caches)
+        if logits.shape[0] != wanted:
+            logits = logits[:wanted]        # the rows behind them belong to what the step was filled up with
         for entry in entries:
             self.cache.advance(entry.rid, self.cache.seq_len(entry.rid) + len(entry.tokens))
         self.steps += 1

@@ -55,8 +55,8 @@ _SIGNATURES = {
     "ta_cache_attach_shared_prefix": (_int, [_vp, _i64, _i32p, _int]),
     "ta_cache_publish": (_int, [_vp, _i64, _i32p, _int]),
     "ta_cache_check": (_int, [_vp]),
-    "ta_cache_pack_batch": (_i64, [_vp, _int, _i64p, _i32p, _i32p, _i32p, _i32p, _int, _i32p, _i64, _i64p, _i32p,
-                                   _i32p]),
+    "ta_cache_pack_batch": (_i64, [_vp, _int, _i64p, _i32p, _i32p, _i32p, _i32p, _int, _i64p, _i32p, _i64, _i64p,
+                                   _i32p, _i32p]),
     "ta_cache_request_ids": (_int, [_vp, _i64p]),
     "ta_sched_new": (_vp, [_vp, _int, _int, _int, _int]),
     "ta_sched_delete": (None, [_vp]),
