@@ -202,7 +202,8 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
         done = [results[i] for i in ids]
         assert all(isinstance(r, Generated) and r.completion_tokens == new_tokens for r in done)
         sched.assert_idle()                      # also gives the cached prefix pages back: the timed pass starts cold
-        log(f"{attempt} pass: {elapsed:.3f} s")
+        log(f"{attempt} pass: {elapsed:.3f} s; steps so far {engine.steps}, replayed {engine.steps_replayed}, "
+            f"graphs captured {engine.graphs_captured}")
     generated = sum(r.completion_tokens for r in done)
     stats = sched.stats
     return {"metric": f"output tokens/s of the workload {name} through the scheduler", "value": round(generated / elapsed, 1),
@@ -216,7 +217,9 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
                        "pages": pages, "page_size": 16, "temperature": temperature},
             "scheduler": {"steps": stats.steps, "tokens_forwarded": stats.tokens_forwarded, "max_running": stats.max_running,
                           "preemptions": stats.preemptions, "peak_pages": stats.peak_blocks,
-                          "forwarded_tokens_per_s": round(stats.tokens_forwarded / elapsed, 1)}}
+                          "forwarded_tokens_per_s": round(stats.tokens_forwarded / elapsed, 1),
+                          "engine_steps": engine.steps, "steps_replayed": engine.steps_replayed,
+                          "graphs_captured": engine.graphs_captured}}
 
 
 def measure_peaks() -> dict:

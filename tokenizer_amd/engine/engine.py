@@ -198,6 +198,8 @@ class Engine:
                                                 v_pages=v_pages, state=self.pools.states.get(source),
                                                 writes=entry.cache_of is None))
         self.steps = 0
+        self.steps_replayed = 0      # steps (decode steps and others) that replayed a captured graph
+        self.graphs_captured = 0
         # Decode steps (one token per request, its logits wanted) and other steps whose shape recurs replay a
         # captured graph; the logits of a step stay valid until the next step.
         self.use_graphs = (model.device.type == "cuda") if use_graphs is None else use_graphs
@@ -327,6 +329,8 @@ class Engine:
         if graph is None:
             graph = StepGraph(self, entries, key[1])       # its first eager run and the capture write the same
             self.graphs[key] = graph                         # keys and values the replay writes again
+            self.graphs_captured += 1
+        self.steps_replayed += 1
         graph.last_used = self.steps
         return graph
 
