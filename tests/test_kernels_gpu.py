@@ -817,6 +817,34 @@ def test_weight_streaming_product_with_two_column_blocks(ops, ref, shape, monkey
     assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
 
 
+@pytest.mark.parametrize("rows", [1, 7, 8, 9, 16])
+@pytest.mark.parametrize("k", [896, 72, 200, 64, 40])
+def test_vocabulary_projection_of_few_rows_reads_its_weights_line_by_line(ops, rows, k):
+    """Up to sixteen rows against tens of thousands of output columns: the weight-streaming kernel with four column
+    blocks a workgroup, whose weight loads touch eight rows' whole cache lines and are put right for the matrix
+    instruction by an exchange between lanes.  Against the plain product and against the same kernel with the older
+    loads (the same sums in another order): widths that end inside a workgroup's 64 columns, a K of whole lines, of
+    a line and a piece, of less than a line, one to sixteen rows (the upper half of the row block empty or not),
+    rows of a wider buffer, float32 and bfloat16 results."""
+    n = 70_003
+    x = rand((rows, k + 8), torch.bfloat16, 161)[:, :k]
+    w = rand((n, k), torch.bfloat16, 162, 0.1)
+    bias = rand((n,), torch.float32, 163)
+    want = x.float() @ w.float().t() + bias
+    results = []
+    for lines in (1, 0):
+        ops.lib.ta_skinny_lines(lines)
+        try:
+            got = ops.linear(x, w, bias, out_dtype=torch.float32)
+            half = ops.linear(x, w, bias)
+        finally:
+            ops.lib.ta_skinny_lines(1)
+        torch.testing.assert_close(got, want, **linear_tol(torch.float32, x, w))
+        torch.testing.assert_close(half.float(), want, **linear_tol(torch.bfloat16, x, w))
+        results.append(got)
+    torch.testing.assert_close(results[0], results[1], rtol=1e-5, atol=1e-4)
+
+
 @pytest.mark.parametrize("shape", [(1, 151, 37), (3, 50, 1000), (16, 33, 130), (9, 1000, 896), (16, 4, 8)])
 def test_linear_float32_of_few_rows(ops, ref, shape):
     # Up to sixteen float32 rows take the kernel that walks the weights once: widths that end inside a wave's four

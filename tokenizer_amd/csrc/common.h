@@ -53,6 +53,34 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// Sixteen rows of a matrix as a 16x16x32 matrix instruction wants them (lane (col, g): row col), read line by line.
+// The memory pipeline works a load off cache line by cache line, so a load that touches eight rows' whole lines of
+// 128 bytes streams far more than one that touches sixteen rows' half lines.  The rows are therefore read by two
+// loads, one for rows 0-7 (`lower`) and one for rows 8-15 (`upper`), in each of which lane (col, g) brings row
+// col % 8's sixteen bytes number 2 g + col / 8 of the line; `lines_to_rows` puts them right by one exchange between
+// lanes eight apart (a rotation within the row of sixteen lanes, no LDS): `first` = the sixteen bytes 2 g of row
+// col's line, `second` = the sixteen bytes 2 g + 1.  The other operand takes the same bytes of its rows.
+typedef uint32_t word4 __attribute__((ext_vector_type(4)));
+typedef __bf16 line_bf16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void lines_to_rows(const word4& lower, const word4& upper, bool low_lane, line_bf16x8& first,
+                                              line_bf16x8& second) {
+  word4 got;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int send = (int)(low_lane ? upper[i] : lower[i]);
+    got[i] = (uint32_t)__builtin_amdgcn_update_dpp(send, send, 0x128, 0xF, 0xF, false);   // row_ror:8: from the lane eight away
+  }
+  word4 a, b;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i] = low_lane ? lower[i] : got[i];
+    b[i] = low_lane ? got[i] : upper[i];
+  }
+  first = __builtin_bit_cast(line_bf16x8, a);
+  second = __builtin_bit_cast(line_bf16x8, b);
+}
+
 // The compute units of the device, asked of the runtime once (the same on every device of a machine); launchers
 // that weigh a launch's workgroups against the device use this, never a number of their own.
 static inline int compute_units() {
