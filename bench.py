@@ -185,6 +185,7 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
     pages = sum(-(-(len(p) + new_tokens) // 16) for p in prompts) + 16
     engine = Engine(model, num_pages=pages, page_size=16, max_requests=64, prefix_cache=prefix_cache)
     log(f"{name}: {len(prompts)} requests, {sum(len(p) for p in prompts)} prompt tokens, {new_tokens} new tokens each")
+    tokens_of_pass = []
     for attempt in ("warm-up", "timed"):        # the first pass captures the decode graphs and warms the library
         sched = Scheduler(engine, SchedulerConfig(max_batch_size=64, max_waiting=64, num_blocks=pages,
                                                   prefix_cache=prefix_cache, max_num_batched_tokens=token_budget))
@@ -201,6 +202,7 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
         elapsed = time.perf_counter() - started
         done = [results[i] for i in ids]
         assert all(isinstance(r, Generated) and r.completion_tokens == new_tokens for r in done)
+        tokens_of_pass.append([r.tokens for r in done])
         sched.assert_idle()                      # also gives the cached prefix pages back: the timed pass starts cold
         log(f"{attempt} pass: {elapsed:.3f} s; steps so far {engine.steps}, replayed {engine.steps_replayed}, "
             f"graphs captured {engine.graphs_captured}")
@@ -219,7 +221,12 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
                           "preemptions": stats.preemptions, "peak_pages": stats.peak_blocks,
                           "forwarded_tokens_per_s": round(stats.tokens_forwarded / elapsed, 1),
                           "engine_steps": engine.steps, "steps_replayed": engine.steps_replayed,
-                          "graphs_captured": engine.graphs_captured}}
+                          "graphs_captured": engine.graphs_captured,
+                          # Requests whose ids are the same in both passes (the first pass runs most steps eagerly,
+                          # the second replays them; a recorded step's products may be other kernels', which round
+                          # differently, so a greedy request may part ways at a near tie).
+                          "requests_with_equal_ids_in_both_passes": sum(
+                              a == b for a, b in zip(*tokens_of_pass))}}
 
 
 def measure_peaks() -> dict:

@@ -92,6 +92,49 @@ def test_portions_of_long_prompts_replay_graphs_narrower_than_their_tables(tmp_p
             check_greedy(cfg, tensors, prompt, got, dtype, 6)
 
 
+def test_a_shared_prefix_under_replayed_graphs_with_heads_of_128_in_groups_of_seven(tmp_path):
+    """Twelve requests that begin with the same 320 tokens, at the head shapes of the 7B model (28 query heads of
+    128 over 4 key heads, a width of 3,584, beyond what the fused products normalise themselves), in bfloat16
+    with the prefix cache: the first request's pages serve the others, whose remaining tokens run as portions
+    beside decoded tokens, and decode steps and recurring portions replay captured graphs.  In the second pass
+    over the same requests nearly every step is a replay.  In both passes every token is the plain
+    implementation's choice on the sequence the engine went along (the passes' tokens need not be equal: a
+    product of a recorded step may be another kernel's than the same product launched eagerly, and round
+    differently)."""
+    import tokenizer_amd as ta
+    from tokenizer_amd.config import Qwen2Config
+    from tokenizer_amd.engine import Generated, GenerateParams, Scheduler, SchedulerConfig
+    raw = dict(TINY["A"][0], num_hidden_layers=2, vocab_size=600, max_position_embeddings=512, sliding_window=512,
+               tie_word_embeddings=False, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+               intermediate_size=640)
+    folder = ta.write_random_model(Qwen2Config.from_dict(raw), 31, str(tmp_path / "heads128"), norm_spread=0.3)
+    cfg, tensors = plain.load_folder(folder)
+    shared = random_ids(600, 320, 70)
+    prompts = [shared + random_ids(600, 9 + 5 * i, 71 + i) for i in range(12)]
+    pages = sum(-(-(len(p) + 20) // 16) for p in prompts) + 8
+    eng = engine_for(folder, "bfloat16", num_pages=pages, max_requests=12, prefix_cache=True)
+    eng.pools.poison()
+    passes = []
+    for _ in range(2):
+        sched = Scheduler(eng, SchedulerConfig(max_batch_size=12, num_blocks=pages, prefix_cache=True,
+                                               max_num_batched_tokens=128))
+        rids = [sched.add_request(prompts[0], GenerateParams.greedy(20))]
+        sched.step()                          # the first prompt's first portion is cached when the others arrive
+        sched.step()
+        sched.step()
+        rids += [sched.add_request(p, GenerateParams.greedy(20)) for p in prompts[1:]]
+        before = (eng.steps, eng.steps_replayed)
+        results = sched.run()
+        assert all(isinstance(results[rid], Generated) for rid in rids)
+        assert sched.stats.prefix_hits >= 11 and sched.stats.prefix_tokens_reused >= 11 * 304
+        passes.append(([results[rid].tokens for rid in rids], eng.steps - before[0], eng.steps_replayed - before[1]))
+        sched.assert_idle()
+    assert passes[1][2] >= passes[1][1] - 6, "the second pass should replay nearly every step"
+    for got, _, _ in passes:
+        for prompt, tokens in zip(prompts, got):
+            check_greedy(cfg, tensors, prompt, tokens, "bfloat16", 20)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_steps_back_to_back_give_what_single_steps_give(model_folders, dtype):
     """Greedy decoding runs in bursts of steps whose ids stay on the device (the host reads them one step late).

@@ -37,6 +37,8 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
                         int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits) {
   constexpr int KS = (D + 31) / 32;   // 32-wide steps over the head size for Q K^T
   constexpr int DB = D / 16;          // 16-row blocks of O^T
+  HELD(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, block_table, table_stride, part_o, part_ml,
+       n_q, n_kv, page_size, window, scale, split_keys, splits);
   __shared__ float acc_s[DEC_WAVES][D][17];
   __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16];
 
@@ -45,15 +47,24 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int head_blocks = (group + 15) / 16;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int item = blockIdx.z;
-  const int t = rows ? __builtin_amdgcn_readfirstlane(rows[item]) : item;   // the same for every lane: scalar
+  const int t = rows ? scalar_int(rows + item) : item;      // the same for every lane
   if (t < 0) return;                                       // a row that only fills the list up: nothing to do
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
   const int heads_here = min(16, group - hb * 16);
   const int head = kvh * group + hb * 16 + col;          // valid when col < heads_here
-  const int pos = __builtin_amdgcn_readfirstlane(positions[t]);
   // entry_of_token null: every request has one token in the batch, request e is row e (one dependent load fewer).
-  const int* table = block_table + (size_t)(entry_of_token ? entry_of_token[t] : t) * table_stride;
+  const int* table = block_table + (size_t)(entry_of_token ? scalar_int(entry_of_token + t) : t) * table_stride;
+  // Without a window the split's first key does not hang on the position, so the pages of the wave's first block
+  // are looked up beside the position rather than after it (one trip fewer before the first keys are asked for).
+  // An entry past the request's pages may hold anything; it is only used for keys that exist (see load_block).
+  const int early_kb = split * split_keys + wave * 32;
+  int early_page0 = 0, early_page1 = 0;
+  if (window < 0) {
+    early_page0 = scalar_int(table + min(early_kb / page_size, table_stride - 1));
+    early_page1 = scalar_int(table + min((early_kb + 16) / page_size, table_stride - 1));
+  }
+  const int pos = scalar_int(positions + t);
   const int lo = (window >= 0 && pos > window) ? pos - window : 0;
   const int first = (lo / 32) * 32 + split * split_keys;  // first key of this split (a multiple of 32)
   const int last = min(pos, first + split_keys - 1);
@@ -82,10 +93,14 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     bf16x8 kf[2][KS];
     union VFrag { uint4 bits; bf16x8 v; } vf[DB];
     bool active;
+    int left;                                              // this lane's eight keys of the block that exist: 0 .. left
   };
   // All loads of a block are issued together: keys, and values (whose addresses do not wait for the scores).
+  // Nothing that was loaded is touched here (values of slots nobody wrote are set to zero when the block is used):
+  // a value that is used makes the wave wait for all it asked for before, one trip to memory for every such use.
   auto load_block = [&](KeyBlock& blk, int kb) {
     blk.active = (kb <= last) && (kb + 31 >= lo);
+    blk.left = 7;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -98,8 +113,14 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
       // what is read there never counts (scores outside lo..last are masked, such values are set to zero).  So
       // the branch is the same for the whole wave, and the addresses are a page number a lane away from scalars.
       const bool there0 = kb + 15 >= lo, there1 = kb + 16 <= last;
-      const int page0 = table[(there0 ? kb : kb + 16) / page_size];
-      const int page1 = table[(there1 ? kb + 16 : kb) / page_size];
+      int page0, page1;
+      if (window < 0 && kb == early_kb) {                    // (without a window the first half always holds keys)
+        page0 = early_page0;
+        page1 = there1 ? early_page1 : early_page0;
+      } else {
+        page0 = scalar_int(table + (there0 ? kb : kb + 16) / page_size);
+        page1 = scalar_int(table + (there1 ? kb + 16 : kb) / page_size);
+      }
       const uint32_t page_elems = (uint32_t)page_size * D;                  // same element count for K and V^T pages
       {
         const int half = col >> 3;
@@ -115,23 +136,27 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
         const int half = g >> 1;
         const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems + (uint32_t)col * page_size +
                             ((kb + 16 * half) % page_size) + 8 * (g & 1);
-        const int left = (half ? there1 : there0) ? last - (kb + 8 * g) : -1;   // keys of this lane that exist: 0..left
+        blk.left = (half ? there1 : there0) ? last - (kb + 8 * g) : -1;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          uint4 v = *reinterpret_cast<const uint4*>(vt_pages + at + db * 16 * page_size);
-          if (left < 7) {                                    // slots nobody wrote may hold anything: 0 * NaN would poison the sum
-            if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
-            if (left < 2) v.y = 0; else if (left < 3) v.y &= 0xffffu;
-            if (left < 4) v.z = 0; else if (left < 5) v.z &= 0xffffu;
-            if (left < 6) v.w = 0; else v.w &= 0xffffu;
-          }
-          blk.vf[db].bits = v;
-        }
+        for (int db = 0; db < DB; ++db)
+          blk.vf[db].bits = *reinterpret_cast<const uint4*>(vt_pages + at + db * 16 * page_size);
       }
     }
   };
   // One step of the online softmax over a block that has been brought in.
-  auto attend = [&](const KeyBlock& blk, int kb) {
+  auto attend = [&](KeyBlock& blk, int kb) {
+    if (blk.left < 7) {                                      // slots nobody wrote may hold anything: 0 * NaN would poison the sum
+      const int left = blk.left;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        uint4 v = blk.vf[db].bits;
+        if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
+        if (left < 2) v.y = 0; else if (left < 3) v.y &= 0xffffu;
+        if (left < 4) v.z = 0; else if (left < 5) v.z &= 0xffffu;
+        if (left < 6) v.w = 0; else v.w &= 0xffffu;
+        blk.vf[db].bits = v;
+      }
+    }
     float s[2][4];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -244,15 +269,16 @@ __global__ void __launch_bounds__(WAVE)
 decode_attention_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                        const int* __restrict__ rows, bf16_t* __restrict__ out, int n_q, int d, int splits,
                        const int* __restrict__ tiles, const int* __restrict__ cu_q) {
+  HELD(part_o, part_ml, rows, out, n_q, d, splits, tiles, cu_q);
   const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
-  int t = rows ? rows[item] : item;
+  int t = rows ? scalar_int(rows + item) : item;
   if (t < 0) return;
   if (tiles) {
     // Items are (tile, token of the tile): the output row is the tile's first row + the token; a tile's padding
     // has no row.
     const int tile = item >> 4, token = item & 15;
-    const int entry = tiles[2 * tile], row0 = cu_q[entry] + tiles[2 * tile + 1];
-    if (token >= cu_q[entry + 1] - row0) return;
+    const int entry = scalar_int(tiles + 2 * tile), row0 = scalar_int(cu_q + entry) + scalar_int(tiles + 2 * tile + 1);
+    if (token >= scalar_int(cu_q + entry + 1) - row0) return;
     t = row0 + token;
   }
   const size_t base = ((size_t)item * n_q + head) * splits;

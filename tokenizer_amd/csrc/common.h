@@ -29,6 +29,50 @@ __device__ __forceinline__ void st(bf16_t* p, float v) { p->bits = float_to_bf16
 // from threadIdx) can end up as exactly that.
 __device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
+// HELD(a, b, ...): the listed kernel arguments are in scalar registers from this point on.  Left to itself the compiler
+// fetches each piece of the argument block where it is first used, with a wait each time; a kernel that lists its
+// arguments once, at its start, fetches them all in one trip.  (One statement for all of them: the fetches of a
+// later statement would not be moved above an earlier one.)
+#define HELD_1(a) "s"(a)
+#define HELD_2(a, ...) "s"(a), HELD_1(__VA_ARGS__)
+#define HELD_3(a, ...) "s"(a), HELD_2(__VA_ARGS__)
+#define HELD_4(a, ...) "s"(a), HELD_3(__VA_ARGS__)
+#define HELD_5(a, ...) "s"(a), HELD_4(__VA_ARGS__)
+#define HELD_6(a, ...) "s"(a), HELD_5(__VA_ARGS__)
+#define HELD_7(a, ...) "s"(a), HELD_6(__VA_ARGS__)
+#define HELD_8(a, ...) "s"(a), HELD_7(__VA_ARGS__)
+#define HELD_9(a, ...) "s"(a), HELD_8(__VA_ARGS__)
+#define HELD_10(a, ...) "s"(a), HELD_9(__VA_ARGS__)
+#define HELD_11(a, ...) "s"(a), HELD_10(__VA_ARGS__)
+#define HELD_12(a, ...) "s"(a), HELD_11(__VA_ARGS__)
+#define HELD_13(a, ...) "s"(a), HELD_12(__VA_ARGS__)
+#define HELD_14(a, ...) "s"(a), HELD_13(__VA_ARGS__)
+#define HELD_15(a, ...) "s"(a), HELD_14(__VA_ARGS__)
+#define HELD_16(a, ...) "s"(a), HELD_15(__VA_ARGS__)
+#define HELD_17(a, ...) "s"(a), HELD_16(__VA_ARGS__)
+#define HELD_18(a, ...) "s"(a), HELD_17(__VA_ARGS__)
+#define HELD_19(a, ...) "s"(a), HELD_18(__VA_ARGS__)
+#define HELD_20(a, ...) "s"(a), HELD_19(__VA_ARGS__)
+#define HELD_21(a, ...) "s"(a), HELD_20(__VA_ARGS__)
+#define HELD_22(a, ...) "s"(a), HELD_21(__VA_ARGS__)
+#define HELD_23(a, ...) "s"(a), HELD_22(__VA_ARGS__)
+#define HELD_24(a, ...) "s"(a), HELD_23(__VA_ARGS__)
+#define HELD_PICK(_1, _2, _3, _4, _5, _6, _7, _8, _9, _10, _11, _12, _13, _14, _15, _16, _17, _18, _19, _20, _21, _22, \
+                  _23, _24, name, ...) name
+#define HELD(...)                                                                                                       \
+  asm volatile("" ::HELD_PICK(__VA_ARGS__, HELD_24, HELD_23, HELD_22, HELD_21, HELD_20, HELD_19, HELD_18, HELD_17,     \
+                              HELD_16, HELD_15, HELD_14, HELD_13, HELD_12, HELD_11, HELD_10, HELD_9, HELD_8, HELD_7,   \
+                              HELD_6, HELD_5, HELD_4, HELD_3, HELD_2, HELD_1)(__VA_ARGS__))
+
+// A load of an int that is the same for the whole wave, through the scalar unit: for tables that no kernel in flight
+// writes (positions, block tables, row lists).  The scalar unit has a counter of its own, so waiting for such a
+// value does not wait for the vector loads that are under way; the compiler takes this path by itself only
+// while it can prove that nothing in the kernel may have written the memory, which `HELD` above ends.
+__device__ __forceinline__ int scalar_int(const int* p) {
+  typedef const int __attribute__((address_space(4))) * constant_int;
+  return *(constant_int)(p);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);

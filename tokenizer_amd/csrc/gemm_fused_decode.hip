@@ -22,6 +22,7 @@ struct FusedArgs {
   const float* residual_in; const float* norm_weight; float eps;
   const bf16_t* w; const float* bias;
   int m, n, k;
+  int rows;                                                // weight rows per workgroup
   // EPI_GATED / plain output (bfloat16 [m, ldc])
   bf16_t* out; int ldc;
   // EPI_RESIDUAL
@@ -29,7 +30,6 @@ struct FusedArgs {
   // EPI_ROPE_STORE
   const int* positions; const float* cos_sin; const int* slots;
   bf16_t* k_pages; bf16_t* v_pages; int n_q, n_kv, d, page_size;
-  int rows;                                                // weight rows per workgroup
 };
 
 __device__ __forceinline__ bf16x8 fz8() {
@@ -37,6 +37,15 @@ __device__ __forceinline__ bf16x8 fz8() {
 #pragma unroll
   for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
   return z;
+}
+// Registers with whatever they hold, for lanes whose load is left out and whose products are never stored (a row
+// of the weights only feeds its own row of the result).  Zeros would do as well, but the compiler keeps one zero
+// for many purposes, copies a loaded value over it, and waits for the load to do so, in the middle of a batch of
+// loads: the batch then takes two trips to memory instead of one.
+__device__ __forceinline__ bf16x8 any8() {
+  bf16x8 v;
+  asm volatile("" : "=v"(v));
+  return v;
 }
 
 // A workgroup owns `p.rows` weight rows (output columns), in PASSES blocks of up to sixteen: the M side of the
@@ -47,8 +56,22 @@ __device__ __forceinline__ bf16x8 fz8() {
 // UN: steps of 32 along K that a wave requests at once.  ONE: the host has checked that a wave's whole share
 // of K is one such batch, so there is no loop, the batches of all passes are requested at the start, and a
 // small matrix is over after one trip to memory instead of several.
+//
+// The arguments are all asked for at the kernel's start (`HELD`): left to itself the compiler fetches each piece
+// of the argument block where it is first used, and a small kernel then begins with several trips to memory one
+// after the other.  What the epilogue needs from memory is asked for before the weights where a second load hangs
+// on a first one (the angle table's row on the position), and otherwise right after them and left alone until the
+// epilogue: a value that is used early makes the wave wait for everything it asked for before, the weights included.
 template <int NW, int EPI, bool NORM, int UN, bool ONE, int PASSES>
 __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs p) {
+  if constexpr (EPI == EPI_ROPE_STORE) {
+    HELD(p.a, p.lda, p.residual_in, p.norm_weight, p.eps, p.w, p.bias, p.m, p.n, p.k, p.rows, p.out, p.ldc,
+         p.positions, p.cos_sin, p.slots, p.k_pages, p.v_pages, p.n_q, p.n_kv, p.d, p.page_size);
+  } else if constexpr (EPI == EPI_GATED) {
+    HELD(p.a, p.lda, p.residual_in, p.norm_weight, p.eps, p.w, p.m, p.n, p.k, p.rows, p.out, p.ldc);
+  } else {
+    HELD(p.a, p.lda, p.w, p.bias, p.m, p.n, p.k, p.rows, p.residual_out);
+  }
   constexpr int SETS = (EPI == EPI_RESIDUAL) ? 1 : 2;
   constexpr int HELD = ONE ? PASSES : 1;                     // batches of weights held at once
   static_assert(EPI != EPI_ROPE_STORE || PASSES == 1, "the rotation pairs rows within one block");
@@ -96,6 +119,22 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   const int full_steps = K / 32;
   const int lds_stride = K + 8;
 
+  // The rotation's angles hang on the row's position: that chain starts before anything else is asked for (wave 0
+  // writes the results; lane (col, g) owns column m = col and rows 4g .. 4g+3 of each block).
+  float pre_cos[4] = {1.f, 1.f, 1.f, 1.f}, pre_sin[4] = {0.f, 0.f, 0.f, 0.f};
+  int pre_slot = -1;
+  if (EPI == EPI_ROPE_STORE && wave == 0 && col < M && 4 * g < R) {
+    pre_slot = p.slots ? p.slots[col] : -1;
+    if (paired && p.cos_sin) {
+      const float* cs = p.cos_sin + (size_t)p.positions[col] * p.d + row0 % p.d + 4 * g;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pre_cos[r] = cs[r];
+        pre_sin[r] = cs[p.d / 2 + r];
+      }
+    }
+  }
+
   // Weight fragments come from HBM and take longest; the first batch is requested before the prologue.
   // Step j of a wave's batch: steps come in pairs (128 contiguous bytes of a weight row, one cache line),
   // pair q of the batch starting at pair `base` is pair base + q * NW.
@@ -105,8 +144,10 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int step = min(step_of(base_pair, u), max(full_steps - 1, 0));   // clamped loads are not used
-      wf[held][u][0] = fz8();
-      if (SETS == 2) wf[held][u][SETS - 1] = fz8();
+      // (in the loop of the long walks the zeros stay: there the statement that leaves a register as it is would
+      // stand between the loop's loads and products, which the compiler then no longer moves past each other)
+      wf[held][u][0] = ONE ? any8() : fz8();
+      if (SETS == 2) wf[held][u][SETS - 1] = ONE ? any8() : fz8();
       if (w_lane[ps]) {
         wf[held][u][0] = *reinterpret_cast<const bf16x8*>(w0[ps] + step * 32);
         if (SETS == 2) wf[held][u][SETS - 1] = *reinterpret_cast<const bf16x8*>(w1[ps] + step * 32);
@@ -123,20 +164,17 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   if (ONE && !NORM) {                                      // the rows' fragments as well
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      af_one[u] = fz8();
-      if (a_lane) af_one[u] = *reinterpret_cast<const bf16x8*>(ar + min(step_of(wave, u), max(full_steps - 1, 0)) * 32);
+      // (every lane: a row past the end repeats the last one and only feeds columns that are never stored)
+      af_one[u] = *reinterpret_cast<const bf16x8*>(ar + min(step_of(wave, u), max(full_steps - 1, 0)) * 32);
     }
   }
 
-  // What the epilogue needs besides the sums is requested now as well (wave 0 writes the results;
-  // lane (col, g) owns column m = col and rows 4g .. 4g+3 of each block).
-  float pre_a[PASSES][4], pre_b[4] = {0.f, 0.f, 0.f, 0.f};     // bias, or the old residual
-  float pre_cos[4] = {1.f, 1.f, 1.f, 1.f}, pre_sin[4] = {0.f, 0.f, 0.f, 0.f};
-  int pre_slot = -1;
+  // What else the epilogue needs besides the sums is requested now as well, and not touched before the epilogue.
+  float pre_a[PASSES][4], pre_b[PASSES][4];                  // the old residual and the bias; or the two halves' bias
 #pragma unroll
   for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) pre_a[ps][r] = 0.f;
+    for (int r = 0; r < 4; ++r) pre_a[ps][r] = pre_b[ps][r] = 0.f;
   if (wave == 0 && col < M) {
     if (EPI == EPI_RESIDUAL) {
 #pragma unroll
@@ -144,20 +182,14 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int local = 16 * ps + 4 * g + r, n = row0 + local;
-          if (local < R && n < p.n) pre_a[ps][r] = p.residual_out[(size_t)col * p.n + n] + (p.bias ? p.bias[n] : 0.f);
+          if (local < R && n < p.n) {
+            pre_a[ps][r] = p.residual_out[(size_t)col * p.n + n];
+            if (p.bias) pre_b[ps][r] = p.bias[n];
+          }
         }
-    } else if (EPI == EPI_ROPE_STORE && 4 * g < R) {
-      pre_slot = p.slots ? p.slots[col] : -1;
+    } else if (EPI == EPI_ROPE_STORE && 4 * g < R && p.bias) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        if (p.bias) { pre_a[0][r] = p.bias[row0 + 4 * g + r]; pre_b[r] = p.bias[row1 + 4 * g + r]; }
-        if (paired && p.cos_sin) {
-          const float* cs = p.cos_sin + (size_t)p.positions[col] * p.d;
-          const int i = row0 % p.d + 4 * g + r;
-          pre_cos[r] = cs[i];
-          pre_sin[r] = cs[p.d / 2 + i];
-        }
-      }
+      for (int r = 0; r < 4; ++r) { pre_a[0][r] = p.bias[row0 + 4 * g + r]; pre_b[0][r] = p.bias[row1 + 4 * g + r]; }
     }
   }
 
@@ -301,7 +333,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
         float* dst = p.residual_out + (size_t)m * p.n + n;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (local + r < R && n + r < p.n) dst[r] = pre_a[ps][r] + v0[r];   // old residual (+ bias) from the start
+          if (local + r < R && n + r < p.n) dst[r] = (pre_a[ps][r] + pre_b[ps][r]) + v0[r];   // old residual (+ bias) from the start
       } else if (EPI == EPI_GATED) {
         const int n = row0 + local;
         bf16_t* dst = p.out + (size_t)m * p.ldc + n;
@@ -317,7 +349,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
           float r1[4], r2[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float x1 = v0[r] + pre_a[0][r], x2 = v1[r] + pre_b[r];
+            const float x1 = v0[r] + pre_a[0][r], x2 = v1[r] + pre_b[0][r];
             r1[r] = x1 * pre_cos[r] - x2 * pre_sin[r];              // cos 1, sin 0 without a rotation
             r2[r] = x2 * pre_cos[r] + x1 * pre_sin[r];
           }
