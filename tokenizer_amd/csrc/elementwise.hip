@@ -58,39 +58,45 @@ __device__ __forceinline__ void st4(bf16_t* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = raw;
 }
 
-template <typename T>
+// CHUNKS: runs of 1,024 floats that a row has (a thread takes four floats of each).  The old residual, the delta
+// and the norm weight are all asked for at the start (a thread past the end of the row asks for the row's last
+// floats and does not use them, so that no load stands behind a condition): one trip to memory where a chunk after
+// the other, and the weight after the sum, were up to five.
+template <typename T, int CHUNKS, bool DELTA>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta, const float* __restrict__ weight,
                        T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps, int store_residual) {
+  HELD(residual, delta, weight, out, rows, hidden, eps, store_residual);
   __shared__ float scratch[16];
   const int i = blockIdx.x;
-  const int r = rows ? rows[i] : i;
+  const int r = rows ? scalar_int(rows + i) : i;
   float* res = residual + (size_t)r * hidden;
-  const T* del = delta ? delta + (size_t)r * hidden : nullptr;
-  float4 x[4];
+  const T* del = delta + (size_t)r * hidden;
+  float4 x[CHUNKS], d[CHUNKS], gain[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int h = min((c * 256 + (int)threadIdx.x) * 4, hidden - 4);
+    x[c] = ld4(res + h);
+    if (DELTA) d[c] = ld4(del + h);
+    gain[c] = ld4(weight + h);
+  }
   float sq = 0.f;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int c = 0; c < CHUNKS; ++c) {
     const int h = (c * 256 + threadIdx.x) * 4;
-    x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (h < hidden) {
-      x[c] = ld4(res + h);
-      if (del) {
-        const float4 d = ld4(del + h);
-        x[c].x += d.x; x[c].y += d.y; x[c].z += d.z; x[c].w += d.w;
-      }
-      if (store_residual && del) st4(res + h, x[c]);
-    }
+    if (DELTA) { x[c].x += d[c].x; x[c].y += d[c].y; x[c].z += d[c].z; x[c].w += d[c].w; }
+    if (h >= hidden) x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    else if (DELTA && store_residual) st4(res + h, x[c]);
     sq += x[c].x * x[c].x + x[c].y * x[c].y + x[c].z * x[c].z + x[c].w * x[c].w;
   }
   const float total = block_sum(sq, scratch);
   const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
   T* dst = out + (size_t)i * hidden;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int c = 0; c < CHUNKS; ++c) {
     const int h = (c * 256 + threadIdx.x) * 4;
     if (h >= hidden) continue;
-    const float4 w = ld4(weight + h);
+    const float4 w = gain[c];
     st4(dst + h, make_float4(x[c].x * inv * w.x, x[c].y * inv * w.y, x[c].z * inv * w.z, x[c].w * inv * w.w));
   }
 }
@@ -98,52 +104,72 @@ add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta
 // The same with the delta still in parts: a product whose K was cut over workgroups left `splits` slabs of
 // float sums [M, hidden]; they are added in their order, the bias joins, the sum goes into the residual stream
 // (stored back) and the row is normalised.  One kernel instead of the addition and the norm after it.
-template <typename T>
+// CHUNKS: runs of 1,024 floats that a row has (a thread takes four floats of each).  Everything a thread needs (the
+// old residual, the bias, the norm weight and the first slabs) is asked for at once and nothing is used
+// before all of it is under way: asked for one after the other as they are needed, these are five trips to memory
+// in a kernel that is over after one.  A thread past the end of the row asks for the row's last floats and does
+// not use them (no load stands behind a condition).
+template <typename T, int CHUNKS>
 __global__ void __launch_bounds__(256)
 splitk_add_rmsnorm_kernel(float* __restrict__ residual, const float* __restrict__ partial, int splits,
                           const float* __restrict__ bias, const float* __restrict__ weight, T* __restrict__ out,
                           int n_rows, int hidden, float eps) {
+  HELD(residual, partial, splits, bias, weight, out, n_rows, hidden, eps);
   __shared__ float scratch[16];
   const int i = blockIdx.x;
   float* res = residual + (size_t)i * hidden;
-  float4 x[4];
+  const size_t slab_stride = (size_t)n_rows * hidden;
+  const float* bias_or_any = bias ? bias : weight;           // (without a bias: loaded from a valid place, not used)
+  constexpr int FIRST = CHUNKS == 1 ? 8 : 4;                 // slabs asked for at the start (registers: sixteen bytes each)
+  float4 old[CHUNKS], gain[CHUNKS], extra[CHUNKS], first[CHUNKS][FIRST];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int h = min((c * 256 + (int)threadIdx.x) * 4, hidden - 4);
+    old[c] = ld4(res + h);
+    extra[c] = ld4(bias_or_any + h);
+    gain[c] = ld4(weight + h);
+    const float* slab = partial + (size_t)i * hidden + h;
+#pragma unroll
+    for (int j = 0; j < FIRST; ++j) first[c][j] = ld4(slab + (size_t)min(j, splits - 1) * slab_stride);
+  }
+  float4 x[CHUNKS];
   float sq = 0.f;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int c = 0; c < CHUNKS; ++c) {
     const int h = (c * 256 + threadIdx.x) * 4;
-    x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (h < hidden) {
-      // Eight slabs are asked for at a time (a product cut into twenty parts is twenty trips otherwise); they are
-      // added in their order all the same.
-      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-      const float* slab = partial + (size_t)i * hidden + h;
-      const size_t slab_stride = (size_t)n_rows * hidden;
-      for (int s0 = 0; s0 < splits; s0 += 8) {
-        float4 v[8];
+    const int hc = min(h, hidden - 4);
+    // The slabs are added in their order, eight asked for at a time after the first ones.
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          v[j] = s0 + j < splits ? ld4(slab + (size_t)(s0 + j) * slab_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) { sum.x += v[j].x; sum.y += v[j].y; sum.z += v[j].z; sum.w += v[j].w; }
-      }
-      if (bias) {
-        const float4 b = ld4(bias + h);
-        sum.x += b.x; sum.y += b.y; sum.z += b.z; sum.w += b.w;
-      }
-      x[c] = ld4(res + h);
-      x[c].x += sum.x; x[c].y += sum.y; x[c].z += sum.z; x[c].w += sum.w;
-      st4(res + h, x[c]);
+    for (int j = 0; j < FIRST; ++j) {
+      const float4 v = j < splits ? first[c][j] : make_float4(0.f, 0.f, 0.f, 0.f);
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
     }
+    const float* slab = partial + (size_t)i * hidden + hc;
+    for (int s0 = FIRST; s0 < splits; s0 += 8) {
+      float4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = ld4(slab + (size_t)min(s0 + j, splits - 1) * slab_stride);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float4 u = s0 + j < splits ? v[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+        sum.x += u.x; sum.y += u.y; sum.z += u.z; sum.w += u.w;
+      }
+    }
+    if (bias) { sum.x += extra[c].x; sum.y += extra[c].y; sum.z += extra[c].z; sum.w += extra[c].w; }
+    x[c] = make_float4(old[c].x + sum.x, old[c].y + sum.y, old[c].z + sum.z, old[c].w + sum.w);
+    if (h < hidden) st4(res + h, x[c]);
+    else x[c] = make_float4(0.f, 0.f, 0.f, 0.f);
     sq += x[c].x * x[c].x + x[c].y * x[c].y + x[c].z * x[c].z + x[c].w * x[c].w;
   }
   const float total = block_sum(sq, scratch);
   const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
   T* dst = out + (size_t)i * hidden;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int c = 0; c < CHUNKS; ++c) {
     const int h = (c * 256 + threadIdx.x) * 4;
     if (h >= hidden) continue;
-    const float4 w = ld4(weight + h);
+    const float4 w = gain[c];
     st4(dst + h, make_float4(x[c].x * inv * w.x, x[c].y * inv * w.y, x[c].z * inv * w.z, x[c].w * inv * w.w));
   }
 }
@@ -196,12 +222,15 @@ extern "C" int ta_add_rmsnorm(void* residual, const void* delta, const void* wei
                               int dtype, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (hidden % 4 == 0 && hidden <= 4096) {
-    if (dtype == DT_F32)
-      add_rmsnorm_vec_kernel<float><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)delta, (const float*)weight,
-                                                                (float*)out, (const int*)rows, hidden, eps, store_residual);
-    else
-      add_rmsnorm_vec_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((float*)residual, (const bf16_t*)delta, (const float*)weight,
-                                                                 (bf16_t*)out, (const int*)rows, hidden, eps, store_residual);
+#define GO(TT, CC, DD) add_rmsnorm_vec_kernel<TT, CC, DD><<<n_rows, 256, 0, stream>>>( \
+    (float*)residual, (const TT*)delta, (const float*)weight, (TT*)out, (const int*)rows, hidden, eps, store_residual)
+#define GO_DELTA(TT, CC) if (delta) GO(TT, CC, true); else GO(TT, CC, false)
+#define GO_CHUNKS(TT) switch ((hidden + 1023) / 1024) { case 1: GO_DELTA(TT, 1); break; case 2: GO_DELTA(TT, 2); break; \
+                                                        case 3: GO_DELTA(TT, 3); break; default: GO_DELTA(TT, 4); break; }
+    if (dtype == DT_F32) GO_CHUNKS(float) else GO_CHUNKS(bf16_t)
+#undef GO_CHUNKS
+#undef GO_DELTA
+#undef GO
     return LAUNCH_STATUS();
   }
   if (dtype == DT_F32)
@@ -220,14 +249,13 @@ extern "C" int ta_splitk_add_rmsnorm(void* residual, const void* partial, int sp
                                      hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (hidden % 4 || hidden > 4096 || splits < 1 || !partial) return -1;
-  if (dtype == DT_F32)
-    splitk_add_rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)partial, splits,
-                                                                 (const float*)bias, (const float*)weight, (float*)out,
-                                                                 n_rows, hidden, eps);
-  else
-    splitk_add_rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((float*)residual, (const float*)partial, splits,
-                                                                  (const float*)bias, (const float*)weight, (bf16_t*)out,
-                                                                  n_rows, hidden, eps);
+#define GO(TT, CC) splitk_add_rmsnorm_kernel<TT, CC><<<n_rows, 256, 0, stream>>>( \
+    (float*)residual, (const float*)partial, splits, (const float*)bias, (const float*)weight, (TT*)out, n_rows, hidden, eps)
+#define GO_CHUNKS(TT) switch ((hidden + 1023) / 1024) { case 1: GO(TT, 1); break; case 2: GO(TT, 2); break; \
+                                                        case 3: GO(TT, 3); break; default: GO(TT, 4); break; }
+  if (dtype == DT_F32) GO_CHUNKS(float) else GO_CHUNKS(bf16_t)
+#undef GO_CHUNKS
+#undef GO
   return LAUNCH_STATUS();
 }
 
