@@ -36,6 +36,7 @@ __device__ __forceinline__ void prefill_block(
   // that holds that key in the second product.  Sixteen consecutive keys lie in one page.
   bf16x8 kf[4][KS];                                    // [2 u + t]: instruction t of half u
   union VFrag { uint4 bits; bf16x8 v; } vf[2][DB];
+  int left[2] = {7, 7};
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int base_key = kb + 32 * u;
@@ -51,8 +52,8 @@ __device__ __forceinline__ void prefill_block(
       // given back; after `hi`: it may not exist yet) borrows the other's page, a valid address; what is read
       // there never counts (scores outside the range are masked, such values are set to zero).
       const bool there0 = FULL || base_key + 15 >= lo, there1 = FULL || base_key + 16 <= hi;
-      const int page0 = table[(there0 ? base_key : base_key + 16) / page_size];
-      const int page1 = table[(there1 ? base_key + 16 : base_key) / page_size];
+      const int page0 = scalar_int(table + (there0 ? base_key : base_key + 16) / page_size);
+      const int page1 = scalar_int(table + (there1 ? base_key + 16 : base_key) / page_size);
       const uint32_t page_elems = (uint32_t)page_size * D;
       {
         const int half = col >> 3;
@@ -69,20 +70,27 @@ __device__ __forceinline__ void prefill_block(
         const int half = g >> 1;
         const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems + (uint32_t)col * page_size +
                             ((base_key + 16 * half) % page_size) + 8 * (g & 1);
+        // (Nothing that was loaded is touched before all of the block is asked for: a value that is used makes the
+        // wave wait for everything it asked for before.)
+        if (!FULL) left[u] = (half ? there1 : there0) ? hi - (base_key + 8 * g) : -1;    // keys of this lane that exist: 0..left
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          uint4 v = *reinterpret_cast<const uint4*>(vt_pages + at + db * 16 * page_size);
-          if (!FULL) {                                 // slots past the last key may never have been written
-            const int left = (half ? there1 : there0) ? hi - (base_key + 8 * g) : -1;    // keys of this lane that exist: 0..left
-            if (left < 7) {
-              if (left < 0) v.x = 0; else if (left < 1) v.x &= 0xffffu;
-              if (left < 2) v.y = 0; else if (left < 3) v.y &= 0xffffu;
-              if (left < 4) v.z = 0; else if (left < 5) v.z &= 0xffffu;
-              if (left < 6) v.w = 0; else v.w &= 0xffffu;
-            }
-          }
-          vf[u][db].bits = v;
-        }
+        for (int db = 0; db < DB; ++db)
+          vf[u][db].bits = *reinterpret_cast<const uint4*>(vt_pages + at + db * 16 * page_size);
+      }
+    }
+  }
+  if (!FULL) {                                             // slots past the last key may never have been written
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      if (left[u] >= 7) continue;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        uint4 v = vf[u][db].bits;
+        if (left[u] < 0) v.x = 0; else if (left[u] < 1) v.x &= 0xffffu;
+        if (left[u] < 2) v.y = 0; else if (left[u] < 3) v.y &= 0xffffu;
+        if (left[u] < 4) v.z = 0; else if (left[u] < 5) v.z &= 0xffffu;
+        if (left[u] < 6) v.w = 0; else v.w &= 0xffffu;
+        vf[u][db].bits = v;
       }
     }
   }
@@ -151,6 +159,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
                          int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
+  HELD(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position, block_table, table_stride, n_q, n_kv,
+       page_size, window, scale_log2);
   __shared__ float merge[NWV > 1 ? NWV - 1 : 1][HG][DB * 4 + 2][WAVE];
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int col = lane & 15, g = lane >> 4;
@@ -166,15 +176,18 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int heads_here = min(HG, group - hb * HG);
   const int head0 = kvh * group + hb * HG;
   const int tile_index = n_tiles - 1 - blockIdx.x / per_tile;
-  // What describes the tile is the same for every lane; taken through readfirstlane so that all that is derived
+  // What describes the tile is the same for every lane; taken through the scalar unit so that all that is derived
   // from it (which keys are visible, which blocks need no mask) lives in scalar registers and branches on it
   // are scalar branches.
-  const int entry = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index]);
-  const int offset = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index + 1]);
-  const int row0 = __builtin_amdgcn_readfirstlane(cu_q[entry]) + offset;
-  const int n_valid = min(16, __builtin_amdgcn_readfirstlane(cu_q[entry + 1]) - row0);
+  const int entry = scalar_int(tiles + 2 * tile_index);
+  const int offset = scalar_int(tiles + 2 * tile_index + 1);
+  const int entry_row = scalar_int(cu_q + entry), next_row = scalar_int(cu_q + entry + 1);
+  const int entry_position = scalar_int(first_position + entry);
+  HELD(entry_row, next_row, entry_position);               // (the three that hang on the entry: one trip)
+  const int row0 = entry_row + offset;
+  const int n_valid = min(16, next_row - row0);
   if (n_valid <= 0) return;                                // a tile that only fills the list up (its entry has no rows)
-  const int p0 = __builtin_amdgcn_readfirstlane(first_position[entry]) + offset;   // position of the tile's first token
+  const int p0 = entry_position + offset;                  // position of the tile's first token
   const int my_pos = p0 + min(col, n_valid - 1);          // padded columns repeat the last token
   const int my_row = row0 + min(col, n_valid - 1);
   const int hi = p0 + n_valid - 1;                         // last key any token of the tile sees

@@ -112,7 +112,7 @@ struct Carrier {
       if (key + 15 < tile.lo) index = tile.lo_page;
       if (key > tile.hi) index = tile.hi_page;
     }
-    page = tile.table[index];
+    page = scalar_int(tile.table + index);
     slot = at_slot;
     at_page += step_pages;
     at_slot += step_slots;
@@ -261,6 +261,8 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   constexpr int DB = D / 16;
   constexpr int NW = SHARED_WAVES;
   constexpr int STRIDE = 64 * KG;                          // keys a turn of the whole workgroup covers
+  HELD(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position, block_table, table_stride, n_q, n_kv,
+       page_size, window, scale_log2, key_splits, part_o, part_ml);
   extern __shared__ __attribute__((aligned(16))) char staged[];
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int head_wave = wave % NW, key_group = wave / NW;
@@ -277,12 +279,16 @@ prefill_attention_shared_kernel(const bf16_t* __restrict__ q, int q_stride, bf16
   const int heads_here = max(0, min(HG, group - first_head));  // a wave past the last head only brings blocks
   const int head0 = kvh * group + first_head;
   const int tile_index = n_tiles - 1 - block / per_tile;
-  const int entry = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index]);
-  const int offset = __builtin_amdgcn_readfirstlane(tiles[2 * tile_index + 1]);
-  const int row0 = __builtin_amdgcn_readfirstlane(cu_q[entry]) + offset;
-  const int n_valid = min(16, __builtin_amdgcn_readfirstlane(cu_q[entry + 1]) - row0);
+  // (Through the scalar unit, the three that hang on the entry asked for together: see scalar_int.)
+  const int entry = scalar_int(tiles + 2 * tile_index);
+  const int offset = scalar_int(tiles + 2 * tile_index + 1);
+  const int entry_row = scalar_int(cu_q + entry), next_row = scalar_int(cu_q + entry + 1);
+  const int entry_position = scalar_int(first_position + entry);
+  HELD(entry_row, next_row, entry_position);
+  const int row0 = entry_row + offset;
+  const int n_valid = min(16, next_row - row0);
   if (n_valid <= 0) return;                                // a tile that only fills the list up (its entry has no rows)
-  const int p0 = __builtin_amdgcn_readfirstlane(first_position[entry]) + offset;   // position of the tile's first token
+  const int p0 = entry_position + offset;                  // position of the tile's first token
   const int my_pos = p0 + min(col, n_valid - 1);          // padded columns repeat the last token
   const int my_row = row0 + min(col, n_valid - 1);
   const int hi = p0 + n_valid - 1;                         // last key any token of the tile sees
