@@ -13,6 +13,30 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restric
   for (int h = threadIdx.x; h < hidden; h += blockDim.x) dst[h] = ld(row + h);
 }
 
+// The same for bfloat16 tables whose rows are a multiple of eight long: sixteen bytes a thread.
+__global__ void __launch_bounds__(256)
+embedding_vec_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ table, float* __restrict__ out,
+                     int hidden, int vocab) {
+  HELD(ids, table, out, hidden, vocab);
+  const int t = blockIdx.x;
+  int id = scalar_int(ids + t);
+  if (id < 0 || id >= vocab) id = 0;  // the host rejects such ids before the launch
+  const uint4* row = reinterpret_cast<const uint4*>(table + (size_t)id * hidden);
+  float* dst = out + (size_t)t * hidden;
+  for (int h8 = threadIdx.x; h8 * 8 < hidden; h8 += blockDim.x) {
+    const uint4 raw = row[h8];
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+    *reinterpret_cast<float4*>(dst + h8 * 8) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(dst + h8 * 8 + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
+
 // For output row i: r = rows ? rows[i] : i;  x = residual[r] (+ delta[r]);
 // if store_residual: residual[r] = x;  out[i] = x / sqrt(mean(x^2) + eps) * weight.
 // Sum of squares, root and scaling are float.
@@ -212,6 +236,8 @@ extern "C" int ta_embedding(const void* ids, const void* table, void* out, int n
   if (n_tokens <= 0) return 0;
   if (dtype == DT_F32)
     embedding_kernel<float><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab);
+  else if (hidden % 8 == 0 && (((uintptr_t)table | (uintptr_t)out) & 15) == 0)
+    embedding_vec_kernel<<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
   else
     embedding_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
   return LAUNCH_STATUS();

@@ -38,9 +38,16 @@ argmax_pieces(const float* __restrict__ logits, float* __restrict__ partial_v, i
   const int begin = chunk * per, end = min(vocab, begin + per);
   float best = -INFINITY;
   int at = 0x7fffffff;
-  for (int i = begin + threadIdx.x; i < end; i += ARGMAX_THREADS) {
-    const float v = src[i];
-    if (v > best) { best = v; at = i; }          // ascending i per thread: its first maximum stays
+  // Eight loads at a time (one after the other, each would be a trip to memory of its own), compared in their order.
+  for (int i0 = begin + threadIdx.x; i0 < end; i0 += 8 * ARGMAX_THREADS) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = src[min(i0 + j * ARGMAX_THREADS, end - 1)];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = i0 + j * ARGMAX_THREADS;
+      if (i < end && v[j] > best) { best = v[j]; at = i; }    // ascending i per thread: its first maximum stays
+    }
   }
   block_best(best, at, best_s, at_s);
   if (threadIdx.x == 0) {
