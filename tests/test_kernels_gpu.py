@@ -46,7 +46,7 @@ def test_embedding(ops, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden", [200, 896, 72, 2048, 4100])
+@pytest.mark.parametrize("hidden", [200, 896, 72, 2048, 3000, 4096, 4100])
 @pytest.mark.parametrize("n", [33, 301])
 def test_add_rmsnorm(ops, ref, dtype, hidden, n):
     # (few and many rows; rows that fit the registers of a workgroup and rows that do not)
@@ -106,7 +106,7 @@ def test_rope_store(ops, ref, dtype, geometry):
     perm = torch.randperm(n_pages * page_size, generator=torch.Generator().manual_seed(9))[:n_tokens]
     slots = perm.int().cuda()
     slots[3] = -1
-    for use_bias, use_rot in ((True, True), (False, True), (False, False)):
+    for use_bias, use_rot in ((True, True), (False, True), (True, False), (False, False)):
         a, b = qkv.clone(), qkv.clone()
         ka = torch.zeros((n_pages, n_kv, page_size, d), dtype=dtype).cuda()
         kb = ka.clone()
@@ -789,6 +789,34 @@ def test_product_left_in_parts_and_added_by_the_norm(ops, ref, shape):
                             store_residual=False)
     assert torch.equal(res_c, residual)
     torch.testing.assert_close(out_c.float(), out_b[rows.long()], rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("hidden", [896, 1028, 2048, 3000, 3584, 4096])
+@pytest.mark.parametrize("splits", [1, 3, 8, 11, 20])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_parts_of_every_count_added_by_the_norm_at_every_row_length(ops, hidden, splits, with_bias):
+    # The norm that adds a product's parts has an instance for every 1,024 floats of a row's length and asks for its
+    # first parts, the bias, the residual and the norm weight at once: every count of parts around the eight (or four)
+    # it asks for first, with and without a bias, against sums in the same order in float32.
+    from tokenizer_amd.kernels import PendingSum
+    m = 19
+    parts = rand((splits, m, hidden), torch.float32, 11, 1.5)
+    bias = rand((hidden,), torch.float32, 12) if with_bias else None
+    gain = 1 + rand((hidden,), torch.float32, 13, 0.1)
+    residual = rand((m, hidden), torch.float32, 14, 2.0)
+    total = torch.zeros((m, hidden), dtype=torch.float32).cuda()
+    for part in parts:
+        total = total + part
+    if with_bias:
+        total = total + bias
+    want_residual = residual + total
+    want = want_residual * torch.rsqrt(want_residual.pow(2).mean(dim=1, keepdim=True) + 1e-6) * gain
+    for dtype in (torch.bfloat16, torch.float32):
+        got_residual = residual.clone()
+        out = ops.add_rmsnorm(got_residual, PendingSum(ops, parts, bias, dtype), gain, 1e-6,
+                              torch.empty((m, hidden), dtype=dtype).cuda())
+        assert torch.equal(got_residual, want_residual)
+        torch.testing.assert_close(out.float(), want, **tol(dtype))
 
 
 @pytest.mark.parametrize("shape", [(33, 48, 264), (64, 100, 896), (50, 900, 40), (64, 1000, 2048)])
