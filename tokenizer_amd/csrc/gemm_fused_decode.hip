@@ -62,16 +62,30 @@ __device__ __forceinline__ bf16x8 any8() {
 // after the other.  What the epilogue needs from memory is asked for before the weights where a second load hangs
 // on a first one (the angle table's row on the position), and otherwise right after them and left alone until the
 // epilogue: a value that is used early makes the wave wait for everything it asked for before, the weights included.
+//
+// The kernel takes its arguments one by one, those that every instance needs before its first load in the first
+// sixteen words of the argument block: the library is compiled so that these are in scalar registers when a wave
+// starts (`-amdgpu-kernarg-preload-count`; fourteen words in fact), and the products with the gated and the residual
+// epilogue then begin without any fetch of arguments (the bias, which only the epilogue needs, lies behind).  One pointer serves for the rows (bfloat16, or the float residual for the norm
+// prologue) and one for the result (bfloat16 rows, or the float residual that is added to), which never occur
+// together.  The rotation's own arguments lie behind; only wave 0, which writes the results, waits for them.
 template <int NW, int EPI, bool NORM, int UN, bool ONE, int PASSES>
-__global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs p) {
-  if constexpr (EPI == EPI_ROPE_STORE) {
-    HELD(p.a, p.lda, p.residual_in, p.norm_weight, p.eps, p.w, p.bias, p.m, p.n, p.k, p.rows, p.out, p.ldc,
-         p.positions, p.cos_sin, p.slots, p.k_pages, p.v_pages, p.n_q, p.n_kv, p.d, p.page_size);
-  } else if constexpr (EPI == EPI_GATED) {
-    HELD(p.a, p.lda, p.residual_in, p.norm_weight, p.eps, p.w, p.m, p.n, p.k, p.rows, p.out, p.ldc);
-  } else {
-    HELD(p.a, p.lda, p.w, p.bias, p.m, p.n, p.k, p.rows, p.residual_out);
-  }
+__global__ void __launch_bounds__(NW * WAVE)
+fused_decode_kernel(const bf16_t* w, const void* rows_in, void* result, const float* norm_weight,
+                    int m, int n, int k, int rows, int lda, float eps, const float* bias,
+                    const int* positions, const float* cos_sin, const int* slots, bf16_t* k_pages, bf16_t* v_pages,
+                    int n_q, int n_kv, int d, int page_size) {
+  HELD(w, rows_in, result, norm_weight, m, n, k, rows, lda, eps);          // (the fourteen words that are there)
+  if constexpr (EPI == EPI_ROPE_STORE) HELD(n_q, n_kv, d, page_size);      // (where a tile's rows lie)
+  FusedArgs p;
+  // (Rows with a norm weight are the float residual; without one they are bfloat16, normalised already or plain.)
+  p.a = norm_weight ? nullptr : (const bf16_t*)rows_in; p.lda = lda;
+  p.residual_in = norm_weight ? (const float*)rows_in : nullptr; p.norm_weight = norm_weight; p.eps = eps;
+  p.w = w; p.bias = bias; p.m = m; p.n = n; p.k = k; p.rows = rows;
+  p.out = (bf16_t*)result; p.ldc = EPI == EPI_GATED ? n / 2 : n_q * d;
+  p.residual_out = (float*)result;
+  p.positions = positions; p.cos_sin = cos_sin; p.slots = slots; p.k_pages = k_pages; p.v_pages = v_pages;
+  p.n_q = n_q; p.n_kv = n_kv; p.d = d; p.page_size = page_size;
   constexpr int SETS = (EPI == EPI_RESIDUAL) ? 1 : 2;
   constexpr int HELD = ONE ? PASSES : 1;                     // batches of weights held at once
   static_assert(EPI != EPI_ROPE_STORE || PASSES == 1, "the rotation pairs rows within one block");
@@ -123,6 +137,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   // writes the results; lane (col, g) owns column m = col and rows 4g .. 4g+3 of each block).
   float pre_cos[4] = {1.f, 1.f, 1.f, 1.f}, pre_sin[4] = {0.f, 0.f, 0.f, 0.f};
   int pre_slot = -1;
+  if (EPI == EPI_ROPE_STORE && wave == 0) HELD(bias, positions, cos_sin, slots, k_pages, v_pages);
   if (EPI == EPI_ROPE_STORE && wave == 0 && col < M && 4 * g < R) {
     pre_slot = p.slots ? p.slots[col] : -1;
     if (paired && p.cos_sin) {
@@ -175,6 +190,7 @@ __global__ void __launch_bounds__(NW * WAVE) fused_decode_kernel(const FusedArgs
   for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
     for (int r = 0; r < 4; ++r) pre_a[ps][r] = pre_b[ps][r] = 0.f;
+  if (EPI == EPI_RESIDUAL && wave == 0) HELD(bias);
   if (wave == 0 && col < M) {
     if (EPI == EPI_RESIDUAL) {
 #pragma unroll
@@ -383,7 +399,15 @@ static int launch_kernel(const FusedArgs& args, int tiles, hipStream_t stream) {
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
   }
-  fused_decode_kernel<NW, EPI, NORM, UN, ONE, PASSES><<<tiles, NW * WAVE, lds, stream>>>(args);
+  // The kernel tells the float residual from bfloat16 rows by whether there is a norm weight.
+  const bool from_residual = args.residual_in != nullptr;
+  if (from_residual != (args.norm_weight != nullptr) || (!from_residual && !args.a) || !args.w) return -1;
+  if (EPI == EPI_RESIDUAL ? !args.residual_out : !args.out) return -1;
+  fused_decode_kernel<NW, EPI, NORM, UN, ONE, PASSES><<<tiles, NW * WAVE, lds, stream>>>(
+      args.w, from_residual ? (const void*)args.residual_in : (const void*)args.a,
+      EPI == EPI_RESIDUAL ? (void*)args.residual_out : (void*)args.out, args.norm_weight, args.m, args.n,
+      args.k, args.rows, args.lda, args.eps, args.bias, args.positions, args.cos_sin, args.slots, args.k_pages, args.v_pages,
+      args.n_q, args.n_kv, args.d, args.page_size);
   return LAUNCH_STATUS();
 }
 

@@ -30,6 +30,10 @@ HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
                # Matrix-core accumulators stay in ordinary registers: the softmax and the epilogues work on
                # them with vector instructions, which cannot read the accumulation registers directly.
                "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+               # The first sixteen words of a kernel's arguments are in scalar registers when a wave starts,
+               # instead of being fetched by its first instructions (a trip to memory at the head of every kernel;
+               # kernels begin with code that fetches them all the same where the firmware does not do this).
+               "-mllvm", "-amdgpu-kernarg-preload-count=16",
                "-Wno-unused-command-line-argument"]
 
 
