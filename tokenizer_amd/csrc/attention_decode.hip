@@ -269,7 +269,7 @@ __global__ void __launch_bounds__(WAVE)
 decode_attention_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                        const int* __restrict__ rows, bf16_t* __restrict__ out, int n_q, int d, int splits,
                        const int* __restrict__ tiles, const int* __restrict__ cu_q) {
-  HELD(part_o, part_ml, rows, out, n_q, d, splits, tiles, cu_q);
+  HELD(part_o, part_ml, rows, out, n_q, d, splits, tiles);   // (the words that are there when a wave starts)
   const int item = blockIdx.x / n_q, head = blockIdx.x % n_q;
   int t = rows ? scalar_int(rows + item) : item;
   if (t < 0) return;

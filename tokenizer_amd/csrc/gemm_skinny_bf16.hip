@@ -51,9 +51,12 @@ struct RopeStore {
 // are one long stream over a big matrix.
 template <int MB, int NW, bool GATED, typename OutT, bool ROPE = false, int NB = 1, bool LINES = false>
 __global__ void __launch_bounds__(NW * WAVE)
-skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
-                   const float* __restrict__ bias, OutT* __restrict__ C, int ldc, int M, int N, int K_all,
-                   int k_chunk, float* __restrict__ partial, const RopeStore rope = RopeStore()) {
+skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, int k_chunk, const bf16_t* __restrict__ W,
+                   OutT* __restrict__ C, int ldc, int M, int N, int K_all, float* __restrict__ partial,
+                   const float* __restrict__ bias, const RopeStore rope = RopeStore()) {
+  // (What the walk over K needs stands in the first fourteen words of the arguments, which are in scalar registers
+  // when a wave starts; the bias and the rotation's arguments, which the epilogue needs, lie behind.)
+  HELD(A, lda, k_chunk, W, C, ldc, M, N, K_all, partial);
   static_assert(!ROPE || GATED, "the rotation uses the two sets of weight rows");
   static_assert(!ROPE || NB == 1, "the rotation pairs rows within one block");
   constexpr int HALVES = GATED ? 2 : 1;                     // gate and up rows (or the two halves of a head)
@@ -296,10 +299,10 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
   float* slabs = splits > 1 ? (float*)partial : nullptr;
   if (out_dtype == DT_F32)
     skinny_gemm_kernel<MB, NW, GATED, float, false, NB, LINES><<<grid, NW * WAVE, 0, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (float*)C, ldc, M, N, K, k_chunk, slabs);
+        (const bf16_t*)A, lda, k_chunk, (const bf16_t*)W, (float*)C, ldc, M, N, K, slabs, (const float*)bias);
   else
     skinny_gemm_kernel<MB, NW, GATED, bf16_t, false, NB, LINES><<<grid, NW * WAVE, 0, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)C, ldc, M, N, K, k_chunk, slabs);
+        (const bf16_t*)A, lda, k_chunk, (const bf16_t*)W, (bf16_t*)C, ldc, M, N, K, slabs, (const float*)bias);
   int status = LAUNCH_STATUS();
   if (status == 0 && splits > 1 && C) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
   return status;
@@ -395,7 +398,7 @@ extern "C" int ta_gemm_skinny_qkv_rope(const void* x, int lda, const void* W, co
   const int per_share = (blocks + shares - 1) / shares;
   const dim3 grid(tiles, 1, (blocks + per_share - 1) / per_share);
 #define GO(MBV) skinny_gemm_kernel<MBV, 8, true, bf16_t, true><<<grid, 8 * WAVE, 0, stream>>>( \
-    (const bf16_t*)x, lda, (const bf16_t*)W, (const float*)bias, (bf16_t*)q_out, n_q * d, M, N, K, K, nullptr, rope)
+    (const bf16_t*)x, lda, K, (const bf16_t*)W, (bf16_t*)q_out, n_q * d, M, N, K, nullptr, (const float*)bias, rope)
   switch (per_share) {
     case 1: GO(1); break;
     case 2: GO(2); break;
