@@ -141,7 +141,8 @@ def run_prefill(model, repeats: int = 7, portion: int | None = None):
     import torch
     from tokenizer_amd.engine import Engine, StepEntry
     engine = Engine(model, num_pages=PROMPT_LEN // 16 + 8, page_size=16, max_requests=1)
-    prompt = make_prompts(1, model.vocab_size, seed=2)[0]
+    import numpy as np
+    prompt = np.asarray(make_prompts(1, model.vocab_size, seed=2)[0], dtype=np.int64)   # ids as a tokenizer hands them on
     portion = portion or PROMPT_LEN
     best = None
     for _ in range(repeats + 1):

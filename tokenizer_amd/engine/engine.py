@@ -416,8 +416,10 @@ class Engine:
                 raise KeyError(f"request {entry.rid!r} is not live")
             if len(entry.tokens) == 0:
                 raise ValueError(f"request {entry.rid!r} brings no tokens")
-            if len(entry.tokens) > 64:                     # long portions: one conversion, kept for the packing
-                entry.token_array = np.asarray(entry.tokens, dtype=np.int64)
+            if isinstance(entry.tokens, np.ndarray) or len(entry.tokens) > 64:
+                # Long portions: one conversion, kept for the packing (none if the caller brings an array of ids).
+                if entry.token_array is None:
+                    entry.token_array = np.ascontiguousarray(entry.tokens, dtype=np.int64)
                 low, high = int(entry.token_array.min()), int(entry.token_array.max())
             else:
                 low, high = min(entry.tokens), max(entry.tokens)

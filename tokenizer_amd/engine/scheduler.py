@@ -23,6 +23,8 @@ import dataclasses
 import time
 from typing import Callable
 
+import numpy as np
+
 from .. import host as _host
 from .batch import StepEntry
 from .generate import (Control, GenerateParams, Generated, SampleCursor, Sampled, StopReason, _go_on,
@@ -208,9 +210,13 @@ class Scheduler:
         self._note_peaks()
         return bool(plan) or n_preempted > 0 or n_failed > 0
 
-    def _tokens(self, seq_id: int, first: int, count: int) -> list[int]:
+    def _tokens(self, seq_id: int, first: int, count: int):
+        """The sequence's tokens first .. first + count - 1: a list, or (long portions) an array, which the engine
+        takes as it is."""
         out = (ctypes.c_int32 * max(1, count))()
         self._lib.ta_sched_tokens(self._core, seq_id, first, count, out)
+        if count > 64:
+            return np.ctypeslib.as_array(out)[:count].astype(np.int64)
         return list(out[:count])
 
     def _run(self, plan: list[tuple[Sequence, int, int, bool]]) -> None:
