@@ -7,7 +7,7 @@ random ids and decodes every request on to 4,096 tokens (8 warm-up steps, 2,040 
 also times a prefill of 2,048 tokens and the same decoding at batch 1 and 64, and prints one
 JSON line.
 
-    python bench.py --workload mixed-1.5b | mixed-0.5b | prefix-7b [--token-budget N]
+    python bench.py --workload mixed-1.5b | mixed-0.5b | prefix-7b [--token-budget N] [--prompts-first]
 
 runs a whole serving workload through the scheduler instead (64 requests at Qwen2.5-1.5B or 0.5B sizes
 with prompts of 128 to 2,048 ids and 256 new tokens each; 64 requests at Qwen2.5-7B sizes that
@@ -160,9 +160,11 @@ def run_prefill(model, repeats: int = 7, portion: int | None = None):
     return best
 
 
-def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0, token_budget: int = 2048) -> dict:
+def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0, token_budget: int = 2048,
+                 prompts_first: bool = False) -> dict:
     """A serving workload through the scheduler: every request is admitted, its prompt cut into portions under
-    the token budget beside the others' decode tokens, decoded greedily to its length, and freed."""
+    the token budget beside the others' decode tokens (or, `prompts_first`, ahead of them), decoded greedily to
+    its length, and freed."""
     import numpy as np
     import torch
     from tokenizer_amd.config import Qwen2Config
@@ -189,7 +191,8 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
     tokens_of_pass = []
     for attempt in ("warm-up", "timed"):        # the first pass captures the decode graphs and warms the library
         sched = Scheduler(engine, SchedulerConfig(max_batch_size=64, max_waiting=64, num_blocks=pages,
-                                                  prefix_cache=prefix_cache, max_num_batched_tokens=token_budget))
+                                                  prefix_cache=prefix_cache, max_num_batched_tokens=token_budget,
+                                                  prompts_first=prompts_first))
         torch.cuda.synchronize()
         started = time.perf_counter()
         params = lambda i: (GenerateParams.greedy(new_tokens) if temperature == 0 else
@@ -216,7 +219,8 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
                        "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                        "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                        "requests": len(prompts), "prompt_tokens": sum(len(p) for p in prompts),
-                       "new_tokens_each": new_tokens, "token_budget": token_budget, "prefix_cache": prefix_cache,
+                       "new_tokens_each": new_tokens, "token_budget": token_budget, "prompts_first": prompts_first,
+                       "prefix_cache": prefix_cache,
                        "pages": pages, "page_size": 16, "temperature": temperature},
             "scheduler": {"steps": stats.steps, "tokens_forwarded": stats.tokens_forwarded, "max_running": stats.max_running,
                           "preemptions": stats.preemptions, "peak_pages": stats.peak_blocks,
@@ -335,6 +339,8 @@ def main() -> int:
                         help="with --attention: the launcher's choice, or one of the two prompt kernels")
     parser.add_argument("--token-budget", type=int, default=2048,
                         help="with --workload: the most tokens a step of the scheduler may hold")
+    parser.add_argument("--prompts-first", action="store_true",
+                        help="with --workload: portions of prompts take the token budget before decoding requests do")
     parser.add_argument("--temperature", type=float, default=0.0,
                         help="with --workload: draw with this temperature and top_p 0.95 instead of greedy picks")
     parser.add_argument("--prompt-len", type=int, default=None,
@@ -357,7 +363,8 @@ def main() -> int:
         print(json.dumps(measure_peaks()), flush=True)
         return 0
     if args.workload:
-        print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature, args.token_budget)), flush=True)
+        print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature, args.token_budget,
+                                      args.prompts_first)), flush=True)
         return 0
     sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
     if args.attention:

@@ -69,6 +69,31 @@ def test_token_budget_cuts_prompts_and_decoding_goes_first(model_folders):
     sched.assert_idle()
 
 
+def test_prompts_first_holds_decoding_back_until_the_prompts_are_through(model_folders):
+    """The reference's order within an iteration (new sequences are prefilled before the batched decode,
+    qwen-server/src/engine.rs:788-805) under a token budget: portions of prompts take the budget, decoding
+    sequences what is left of it; the tokens are the same as in the other order."""
+    folder = model_folders["A"]
+    engine = cpu_engine(folder, num_pages=64)
+    sched = Scheduler(engine, SchedulerConfig(max_num_batched_tokens=16, prefill_chunk=10, prompts_first=True))
+    long_a, long_b, short = random_ids(256, 37, 1), random_ids(256, 23, 2), random_ids(256, 3, 3)
+    first = sched.add_request(short, GenerateParams.greedy(6))
+    sched.step()                                         # the short one is through its prompt
+    a = sched.add_request(long_a, GenerateParams.greedy(3))
+    b = sched.add_request(long_b, GenerateParams.greedy(3))
+    results = sched.run()
+    assert all(sum(step) <= 16 for step in engine.forwards)
+    assert engine.forwards[0] == [3]
+    # 37 and 23 prompt tokens in portions of at most 10 under a budget of 16: the decoding request waits while
+    # they fill the budget and joins in the step that leaves room (7 + 5 + its one token).
+    assert engine.forwards[1:5] == [[10, 6], [10, 6], [10, 6], [7, 5, 1]]
+    assert engine.forwards[5] == [1, 1, 1]               # all three decode together from here
+    assert all(set(step) == {1} for step in engine.forwards[5:])
+    for rid, prompt, n in ((first, short, 6), (a, long_a, 3), (b, long_b, 3)):
+        assert results[rid].tokens == solo(folder, prompt, GenerateParams.greedy(n)).tokens
+    sched.assert_idle()
+
+
 def test_pages_run_out_the_newest_is_preempted_and_recomputed(model_folders):
     # Pool of 3 pages, two 16-token prompts, 4 tokens each: both need a second page once they decode.
     folder = model_folders["A"]
@@ -259,11 +284,12 @@ def test_requests_cancelled_at_random_keep_what_they_sampled(model_folders, seed
     sched.assert_idle()
 
 
+@pytest.mark.parametrize("prompts_first", [False, True])
 @pytest.mark.parametrize("seed", range(12))
-def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed):
+def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed, prompts_first):
     """Random prompts, output lengths, pool sizes, batch caps, token budgets, portion sizes and arrival times
-    (shared prefixes included): whatever the scheduler decides, every request gets the tokens it would get alone,
-    and when all is over no page, count or slot is left."""
+    (shared prefixes included), under either order of prompts and decoding: whatever the scheduler decides, every
+    request gets the tokens it would get alone, and when all is over no page, count or slot is left."""
     import random
     rng = random.Random(seed)
     folder = model_folders["A"]
@@ -271,7 +297,7 @@ def test_random_arrivals_pools_and_budgets_give_solo_results(model_folders, seed
     num_pages = rng.choice([4, 5, 6, 9, 24])
     config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 3, 5]), num_blocks=num_pages,
                              prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 16, 40]),
-                             prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64)
+                             prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64, prompts_first=prompts_first)
     engine = cpu_engine(folder, bursts=True, num_pages=num_pages, max_requests=config.max_batch_size,
                         prefix_cache=config.prefix_cache)
     sched = Scheduler(engine, config)

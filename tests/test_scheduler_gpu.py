@@ -29,8 +29,8 @@ def check_greedy(cfg, tensors, prompt, tokens, dtype, n_tokens):
         assert float(row.max() - row[token]) <= 4e-2 * max(1.0, float(row.abs().max())), (k, token)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_few_pages_a_shared_prefix_and_portions_on_the_device(model_folders, dtype):
+@pytest.mark.parametrize("dtype, prompts_first", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
+def test_few_pages_a_shared_prefix_and_portions_on_the_device(model_folders, dtype, prompts_first):
     """Six requests, three of which start with the same 40 tokens, through a pool of eight pages with prompts cut
     into portions of sixteen: some are preempted and recomputed, the later sharers take over the prefix's pages,
     decode steps and recurring portion shapes replay captured graphs.  Every request gets the plain
@@ -46,7 +46,7 @@ def test_few_pages_a_shared_prefix_and_portions_on_the_device(model_folders, dty
     eng = engine_for(model_folders[name], dtype, num_pages=8, max_requests=3, prefix_cache=True)
     eng.pools.poison()
     sched = Scheduler(eng, SchedulerConfig(max_batch_size=3, num_blocks=8, prefix_cache=True, prefill_chunk=16,
-                                           max_num_batched_tokens=48))
+                                           max_num_batched_tokens=48, prompts_first=prompts_first))
     rids = [sched.add_request(p, GenerateParams.greedy(12)) for p in prompts]
     results = sched.run()
     for rid, prompt in zip(rids, prompts):
@@ -184,11 +184,12 @@ def test_decode_steps_back_to_back_give_what_single_steps_give(model_folders, dt
         assert any(r.reason == StopReason.MaxTokens for r in bursts)
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2])
-def test_random_arrivals_pools_and_budgets_on_the_device(model_folders, seed):
+@pytest.mark.parametrize("seed, prompts_first", [(0, False), (1, False), (2, False), (3, True), (4, True), (5, True)])
+def test_random_arrivals_pools_and_budgets_on_the_device(model_folders, seed, prompts_first):
     """Random prompts (some with a shared beginning), output lengths, pool sizes, batch caps, token budgets,
-    portion sizes, burst lengths and arrival times, in float32 on the kernels with graphs: whatever the scheduler
-    decides, every request gets the plain implementation's tokens, and in the end nothing is left over."""
+    portion sizes, burst lengths and arrival times, decoding requests or prompts first, in float32 on the kernels
+    with graphs: whatever the scheduler decides, every request gets the plain implementation's tokens, and in the
+    end nothing is left over."""
     import random
     from tokenizer_amd.engine import Failure, GenerateParams, Scheduler, SchedulerConfig
     rng = random.Random(seed)
@@ -199,7 +200,7 @@ def test_random_arrivals_pools_and_budgets_on_the_device(model_folders, seed):
     config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 3, 5]), num_blocks=num_pages,
                              prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 16, 40]),
                              prefill_chunk=rng.choice([None, 5, 16]), max_waiting=64,
-                             decode_burst=rng.choice([1, 3, 16]))
+                             decode_burst=rng.choice([1, 3, 16]), prompts_first=prompts_first)
     eng = engine_for(model_folders[name], "float32", num_pages=num_pages, max_requests=config.max_batch_size,
                      prefix_cache=config.prefix_cache)
     eng.pools.poison()

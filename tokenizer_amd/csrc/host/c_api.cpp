@@ -153,9 +153,11 @@ int64_t ta_cache_pack_batch(void* c, int n_entries, const int64_t* ids, const in
 }
 
 // ---------------------------------------------------------------------------------------- scheduler
-void* ta_sched_new(void* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk) {
+void* ta_sched_new(void* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk,
+                   int prompts_first) {
   if (!cache || max_batch_size <= 0 || token_budget <= 0) return nullptr;
-  return new SchedulerCore((CacheCore*)cache, num_pages, max_batch_size, token_budget, prefill_chunk);
+  return new SchedulerCore((CacheCore*)cache, num_pages, max_batch_size, token_budget, prefill_chunk,
+                           prompts_first != 0);
 }
 void ta_sched_delete(void* s) { delete (SchedulerCore*)s; }
 int ta_sched_enqueue(void* s, int64_t id, const int32_t* prompt, int count) {

@@ -6,9 +6,10 @@ namespace ta {
 
 static int pages_for(int length, int page_size) { return (length + page_size - 1) / page_size; }
 
-SchedulerCore::SchedulerCore(CacheCore* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk)
+SchedulerCore::SchedulerCore(CacheCore* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk,
+                             bool prompts_first)
     : cache_(cache), num_pages_(num_pages), max_batch_size_(max_batch_size), token_budget_(token_budget),
-      prefill_chunk_(prefill_chunk > 0 ? prefill_chunk : token_budget) {}
+      prefill_chunk_(prefill_chunk > 0 ? prefill_chunk : token_budget), prompts_first_(prompts_first) {}
 
 const Sequence* SchedulerCore::find(int64_t id) const {
   auto found = sequences_.find(id);
@@ -81,11 +82,11 @@ void SchedulerCore::plan_step(std::vector<PlannedEntry>* planned, std::vector<in
                               std::vector<FailedEntry>* failed) {
   admit(failed);
   if (running_.empty()) return;
-  // Oldest first; decoding sequences before prompt portions.
+  // Oldest first; decoding sequences before prompt portions, or after them.
   std::vector<int64_t> order = running_;
   std::stable_sort(order.begin(), order.end(), [&](int64_t a, int64_t b) {
     const bool da = find(a)->decoding(), db = find(b)->decoding();
-    if (da != db) return da;
+    if (da != db) return prompts_first_ ? db : da;
     return a < b;
   });
   int budget = token_budget_;

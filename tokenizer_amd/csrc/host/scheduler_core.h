@@ -4,7 +4,10 @@
 // out, preempts the newest one, which gives back everything and is recomputed later (561-668); preempted
 // sequences return to the front of the queue, oldest first (369-376); a sequence that cannot fit in the whole
 // pool fails (473-487, 670-685).  Beyond the reference one iteration is a single mixed batch under a token
-// budget: one token for every decoding sequence first, then portions of prompts in order of arrival.
+// budget: one token for every decoding sequence first, then portions of prompts in order of arrival; or, with
+// `prompts_first`, the reference's own order within an iteration (new sequences are prefilled before the batched
+// decode, 788-805): portions of prompts take the budget first and decoding sequences what is left of it, so that
+// they wait while prompts stand in line and then decode together.
 // Sampling, stop conditions and results stay with the caller; this class owns the token lists, the order of
 // work and every exchange with the cache manager.
 #pragma once
@@ -33,7 +36,8 @@ struct FailedEntry { int64_t id; int pages_needed; };
 
 class SchedulerCore {
  public:
-  SchedulerCore(CacheCore* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk);
+  SchedulerCore(CacheCore* cache, int num_pages, int max_batch_size, int token_budget, int prefill_chunk,
+                bool prompts_first = false);
 
   int enqueue(int64_t id, const int32_t* prompt, int count);   // 0, or -1 if the id is known
   int append_token(int64_t id, int32_t token);
@@ -64,6 +68,7 @@ class SchedulerCore {
 
   CacheCore* cache_;
   int num_pages_, max_batch_size_, token_budget_, prefill_chunk_;
+  bool prompts_first_;
   std::unordered_map<int64_t, Sequence> sequences_;
   std::deque<int64_t> waiting_;
   std::vector<int64_t> running_;          // in order of admission

@@ -8,7 +8,9 @@ preempted sequences return to the front of the queue, oldest first (369-376); a 
 cannot fit in the whole pool fails with a message (473-487, 670-685).
 
 Beyond the reference, one iteration is a single mixed batch under a token budget: one token
-for every decoding sequence first, then portions of prompts in order of arrival.  A preempted
+for every decoding sequence first, then portions of prompts in order of arrival
+(`SchedulerConfig.prompts_first` turns that round: the reference's order within an iteration,
+new sequences prefilled before the batched decode, 788-805).  A preempted
 sequence is recomputed from its prompt and the tokens it sampled so far, and nothing is
 sampled again for positions that already have a token.
 
@@ -42,6 +44,11 @@ class SchedulerConfig:
     max_num_batched_tokens: int = 2048
     prefill_chunk: int | None = None
     decode_burst: int = 16       # greedy decode steps that may run back to back without the host in between
+    # Who takes the token budget first.  False: decoding sequences, one token each, then portions of prompts: a
+    # running request gets a token in every step whatever arrives.  True: portions of prompts, then decoding
+    # sequences with what is left: they wait while prompts stand in line and then decode together in full
+    # batches, fewer and cheaper steps for the same tokens when many requests arrive at once.
+    prompts_first: bool = False
 
 
 @dataclasses.dataclass
@@ -102,7 +109,8 @@ class Scheduler:
         self.config = config or SchedulerConfig()
         self._lib = _host.lib()
         self._core = self._lib.ta_sched_new(self.cache._core, self.cache.num_pages, self.config.max_batch_size,
-                                            self.config.max_num_batched_tokens, self.config.prefill_chunk or 0)
+                                            self.config.max_num_batched_tokens, self.config.prefill_chunk or 0,
+                                            1 if self.config.prompts_first else 0)
         if not self._core:
             raise ValueError("max_batch_size and max_num_batched_tokens must be positive")
         self._cache_core_owner = self.cache._core_owner      # the cache core outlives this scheduler's core

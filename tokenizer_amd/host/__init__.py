@@ -58,7 +58,7 @@ _SIGNATURES = {
     "ta_cache_pack_batch": (_i64, [_vp, _int, _i64p, _i32p, _i32p, _i32p, _i32p, _int, _i64p, _i32p, _i64, _i64p,
                                    _i32p, _i32p]),
     "ta_cache_request_ids": (_int, [_vp, _i64p]),
-    "ta_sched_new": (_vp, [_vp, _int, _int, _int, _int]),
+    "ta_sched_new": (_vp, [_vp, _int, _int, _int, _int, _int]),
     "ta_sched_delete": (None, [_vp]),
     "ta_sched_enqueue": (_int, [_vp, _i64, _i32p, _int]),
     "ta_sched_append_token": (_int, [_vp, _i64, ctypes.c_int32]),
