@@ -680,7 +680,8 @@ def test_skinny_rows_agree_with_the_tiled_kernel(ops, shape):
 
 
 @pytest.mark.parametrize("geometry", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 16), (4, 4, 128, 520, 32), (20, 2, 96, 264, 16),
-                                      (2, 1, 64, 1280, 16), (4, 2, 32, 2304, 16)])
+                                      (2, 1, 64, 1280, 16), (4, 2, 32, 2304, 16), (12, 2, 128, 1536, 16),
+                                      (3, 1, 64, 2048, 16), (2, 2, 32, 1800, 16)])
 @pytest.mark.parametrize("rows", [1, 8, 16, 17, 40, 64])
 def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
     # Up to 16 rows: the fused decode kernel, from the residual or from normalised rows; 17 to 64 rows: the
@@ -730,10 +731,12 @@ def test_fused_norm_qkv_rope(ops, ref, geometry, rows):
             assert float(kc.abs().max()) == 0 and float(vc.abs().max()) == 0
 
 
-# The last shapes: rows of 1,280 and 2,304 elements give the waves unequal shares of K in the kernels that ask for
-# a wave's whole share at once (some waves then have steps past the end, which must add nothing).
+# Rows of 1,280 and 2,304 elements give the waves unequal shares of K in the kernels that ask for
+# a wave's whole share at once (some waves then have steps past the end, which must add nothing); rows of 1,536 to
+# 2,048 are one trip of six or eight steps from normalised rows in LDS (in one block of weight rows, or in two where
+# the matrix has more than sixteen rows for every compute unit).
 @pytest.mark.parametrize("shape", [(1, 4864, 896), (8, 272, 96), (16, 176, 80), (5, 136, 72), (6, 1280, 2304),
-                                   (8, 2304, 1280)])
+                                   (8, 2304, 1280), (8, 8960, 1536), (3, 1104, 1536), (16, 600, 2048), (7, 5000, 1800)])
 def test_fused_norm_gated_and_linear_add(ops, ref, shape):
     rows, inner, hidden = shape
     residual = rand((rows, hidden), torch.float32, 50, 2.0)

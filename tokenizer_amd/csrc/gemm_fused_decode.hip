@@ -417,6 +417,14 @@ static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
   const int pairs = (args.k / 32 + 1) / 2;
   const int steps_per_wave = 2 * ((pairs + NW - 1) / NW);
   if (steps_per_wave <= 4) return launch_kernel<NW, EPI, NORM, 4, true, PASSES>(args, tiles, stream);
+  if constexpr (NORM && EPI == EPI_ROPE_STORE) {
+    // Rows in LDS: only the weights take registers, and a wave's whole share of up to eight steps is one trip
+    // (rows of 1,025 to 2,048 elements at eight waves: two trips in the loop below; q/k/v at 1,536: 8.4 -> 7.5 us).
+    // Not for the gated product: its matrix is several workgroups for every compute unit, and with the registers
+    // of a whole share only one of them fits a unit at a time (two blocks of rows: 19.9 -> 22.3 us).
+    if (steps_per_wave <= 6) return launch_kernel<NW, EPI, NORM, 6, true, PASSES>(args, tiles, stream);
+    if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, 8, true, PASSES>(args, tiles, stream);
+  }
   if constexpr (!NORM && PASSES == 1) {
     // Rows from memory: one trip for a wave's whole share if it fits the registers (128 a lane at 16 waves).
     if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, 8, true, 1>(args, tiles, stream);
