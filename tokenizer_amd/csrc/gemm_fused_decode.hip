@@ -417,13 +417,15 @@ static int launch_one(const FusedArgs& args, int tiles, hipStream_t stream) {
   const int pairs = (args.k / 32 + 1) / 2;
   const int steps_per_wave = 2 * ((pairs + NW - 1) / NW);
   if (steps_per_wave <= 4) return launch_kernel<NW, EPI, NORM, 4, true, PASSES>(args, tiles, stream);
-  if constexpr (NORM && EPI == EPI_ROPE_STORE) {
+  if constexpr (NORM && (EPI == EPI_ROPE_STORE || PASSES == 1)) {
     // Rows in LDS: only the weights take registers, and a wave's whole share of up to eight steps is one trip
     // (rows of 1,025 to 2,048 elements at eight waves: two trips in the loop below; q/k/v at 1,536: 8.4 -> 7.5 us).
-    // Not for the gated product: its matrix is several workgroups for every compute unit, and with the registers
-    // of a whole share only one of them fits a unit at a time (two blocks of rows: 19.9 -> 22.3 us).
+    // The gated product's matrix is several workgroups for every compute unit: it takes a whole share at once only
+    // while two workgroups' registers fit a unit together, which is one block of rows and six steps (with two blocks
+    // of rows 19.9 -> 22.3 us at 8,960 x 1,536, with eight steps 25.4 -> 31.3 us at 11,008 x 2,048).
     if (steps_per_wave <= 6) return launch_kernel<NW, EPI, NORM, 6, true, PASSES>(args, tiles, stream);
-    if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, 8, true, PASSES>(args, tiles, stream);
+    if constexpr (EPI == EPI_ROPE_STORE)
+      if (steps_per_wave <= 8) return launch_kernel<NW, EPI, NORM, 8, true, PASSES>(args, tiles, stream);
   }
   if constexpr (!NORM && PASSES == 1) {
     // Rows from memory: one trip for a wave's whole share if it fits the registers (128 a lane at 16 waves).
@@ -454,7 +456,9 @@ static int launch_rows(const FusedArgs& args, int tiles, int waves, hipStream_t 
 
 // Weight rows per workgroup for the rotation epilogue, where a block pairs rows half a head apart: 16, 8 or 4.
 // Every workgroup reads and normalises all m input rows before its share of the weights, so the choice weighs
-// the bytes the busiest compute unit has to ask for: rounds of workgroups x (prologue + its weight rows).
+// the bytes the busiest compute unit has to ask for: rounds of workgroups x (prologue + its weight rows + what a
+// unit could have streamed during the trips to memory that every workgroup begins with; without that last term one
+// row of 3,584 took three rounds of four weight rows, 17.7 us, where one round of sixteen takes 14.0).
 static int rows_per_tile(int n_q, int n_kv, int d, int m, int k, bool norm, int rows_override) {
   if (rows_override == 16 || rows_override == 8 || rows_override == 4) return rows_override;
   const long units = compute_units();
@@ -463,7 +467,7 @@ static int rows_per_tile(int n_q, int n_kv, int d, int m, int k, bool norm, int 
   long best_cost = -1;
   for (int r = 16; r >= 4; r /= 2) {
     const long tiles = (long)(n_q + n_kv) * (d / 2 / r) + (long)n_kv * d / r;
-    const long cost = ((tiles + units - 1) / units) * (prologue + 2L * r * k * 2);
+    const long cost = ((tiles + units - 1) / units) * (prologue + 2L * r * k * 2 + 64 * 1024);
     if (best_cost < 0 || cost < best_cost) { best = r; best_cost = cost; }
   }
   return best;
@@ -481,6 +485,24 @@ static int rows_per_workgroup(int n_rows, int rows_override) {
   // rows of 896: 19 rows 8.6 us, 10 rows 8.2 us; with two rounds, 8,960 rows of 1,536, the halves are slower).
   if (rounds == 1 && rows > 16 && rows < 32) rows = (n_rows + 2 * units - 1) / (2 * units);
   return rows < 4 ? 4 : rows;
+}
+
+// The gated product from rows in LDS: where the even shares would be two blocks of rows a workgroup (17 to 32) and
+// a wave's share of K at eight waves is at most six steps, workgroups of one block whose weights are asked for at
+// once are over sooner: as many rounds of workgroups as blocks of sixteen need, in equal shares (8,960 rows of 1,536:
+// 18 rows in two blocks 19.9 us, 12 rows 19.3 us at eight input rows; 18.3 and 17.3 us at one).  Up to eight input
+// rows: every workgroup brings all of them in first, and half as many workgroups again weigh more than they save
+// at sixteen (22.9 and 24.8 us).
+static int rows_per_gated_workgroup(int n_rows, int m, int k, int rows_override) {
+  int rows = rows_per_workgroup(n_rows, rows_override);
+  if (rows_override >= 1 && rows_override <= 32) return rows;
+  const int pairs = (k / 32 + 1) / 2;
+  if (rows > 16 && m <= 8 && 2 * ((pairs + 7) / 8) <= 6) {
+    const int units = compute_units();
+    const int rounds = (n_rows + units * 16 - 1) / (units * 16);
+    rows = (n_rows + units * rounds - 1) / (units * rounds);
+  }
+  return rows;
 }
 
 // Rows that are normalised already go through LDS (the NORM instances, which then copy instead of normalising)
@@ -538,7 +560,7 @@ extern "C" int ta_fused_norm_gated(const void* residual, const void* norm_weight
   FusedArgs a = {};
   a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
-  a.rows = rows_per_workgroup(n / 2, rows);
+  a.rows = rows_per_gated_workgroup(n / 2, m, k, rows);
   return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
 }
 
@@ -550,7 +572,7 @@ extern "C" int ta_fused_gated(const void* x, int lda, const void* w, void* out, 
   FusedArgs a = {};
   a.a = (const bf16_t*)x; a.lda = lda;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
-  a.rows = rows_per_workgroup(n / 2, rows);
+  a.rows = stage_rows(m, k) ? rows_per_gated_workgroup(n / 2, m, k, rows) : rows_per_workgroup(n / 2, rows);
   if (stage_rows(m, k)) return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
   return launch_rows<EPI_GATED, false>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
 }
