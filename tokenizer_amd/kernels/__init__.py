@@ -390,6 +390,7 @@ class Ops:
     #                               an instance, -1 = never, 0 = where the launcher expects it to be the faster one
     prefill_key_splits = True     # whether the prompt kernel may cut a tile's keys over workgroups (tests switch it off)
     target_workgroups = 1024      # what the split of the key range aims at
+    min_split_keys = 128          # ... in parts of at least so many keys (a block of 32 for each of a workgroup's four waves)
     PLAN_KEYS = 512               # launch shapes depend on the context only through its multiple of this
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
@@ -405,7 +406,7 @@ class Ops:
             max_keys = min(max_keys, window + 32)
         head_blocks = -(-(n_q // n_kv) // 16)
         per_split = max(1, self.target_workgroups // max(1, n_items * n_kv * head_blocks))
-        split_keys = max(128, -(-max_keys // per_split))
+        split_keys = max(self.min_split_keys, -(-max_keys // per_split))
         split_keys = -(-split_keys // 32) * 32
         splits = max(1, -(-(max_keys + 31) // split_keys))
         part_o = part_ml = None
