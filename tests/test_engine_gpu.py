@@ -423,14 +423,18 @@ def test_recurring_step_shapes_replay_graphs_and_equal_eager_steps(model_folders
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, dtype, monkeypatch):
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, dtype, name, monkeypatch):
     """`decode_greedy` feeds each step's ids to the next on the device and reads them a step late; it must pick
     what stepping one by one picks, also across a change of graph (the context bucket is made small), and an
-    early end returns exactly one step more than was asked for."""
+    early end returns exactly one step more than was asked for.  Between its steps the device itself turns a
+    step's description into the next one's, and the host uploads one only where that is not what it would upload
+    (a request has entered a new page or, in C's layers with a window, given one back; another graph): far fewer
+    uploads than steps, and the same ids."""
     from tokenizer_amd.engine import Engine, StepEntry
-    name = "B"
     vocab = TINY[name][0]["vocab_size"]
     monkeypatch.setattr(Engine, "GRAPH_BUCKET", 48)
+    monkeypatch.setattr(Engine, "NEXT_STEP_ON_DEVICE", True)
     prompts = {rid: random_ids(vocab, n, 90 + rid) for rid, n in enumerate([40, 3, 21])}
     runs = []
     for pipelined in (True, False):
@@ -442,6 +446,8 @@ def test_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, dtype, 
         if pipelined:
             picked = eng.decode_greedy(list(prompts), first, 30)
             assert len(eng.graphs) >= 2                      # the contexts crossed a bucket's end
+            uploads = sum(graph.uploads for graph in eng.graphs.values())
+            assert all(graph.advances for graph in eng.graphs.values()) and 2 <= uploads <= 20
         else:
             picked, current = [], first
             for _ in range(30):

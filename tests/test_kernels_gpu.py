@@ -4,7 +4,7 @@ import math
 import pytest
 import torch
 
-from tokenizer_amd.kernels import PendingSum
+from tokenizer_amd.kernels import KernelError, PendingSum
 
 from kernel_refs import PlainOps
 
@@ -969,6 +969,41 @@ def test_sampling_kernel_follows_the_reference_rules(ops, ref):
     assert ops.sample(flat, ones, ones, torch.arange(8).cuda() / 8 + 0.01).cpu().tolist() == list(range(8))
     # All -inf: nothing to weigh, the first index, as the greedy scan gives.
     assert ops.sample(torch.full((1, 50), float("-inf")).cuda(), ones[:1], ones[:1], us[:1]).item() == 0
+
+
+@pytest.mark.parametrize("rows, vocab, widths, page_size", [(1, 33, [3], 16), (8, 5000, [40, 7], 16), (37, 151936, [9], 32),
+                                                            (64, 700, [5, 5, 2, 11], 48)])
+def test_greedy_pick_that_writes_the_next_steps_description(ops, rows, vocab, widths, page_size):
+    """The pick itself is `argmax`'s; the ids become the next tokens, positions and first positions go up by one,
+    and each group's slots are page * page size + offset of the new position, looked up in the request's row of
+    that group's table: -1 where the page is not there, the row's last entry where the position lies past the
+    table (what the host never relies on)."""
+    import numpy as np
+    rng = np.random.default_rng(rows + vocab)
+    logits = torch.tensor(rng.normal(size=(rows, vocab)).astype(np.float32)).cuda()
+    ids = torch.full((rows,), -7, dtype=torch.int32).cuda()
+    reach = min(widths) * page_size
+    start = rng.integers(0, reach + 40, size=rows).astype(np.int32)          # some past the narrowest table's end
+    start[0] = page_size - 1                                                  # the next position opens a page
+    positions, first = torch.tensor(start).cuda(), torch.tensor(start).cuda()
+    tables, slots = [], []
+    for width in widths:
+        table = rng.permutation(rows * width).astype(np.int32).reshape(rows, width)
+        table[rng.random((rows, width)) < 0.2] = -1
+        tables.append(torch.tensor(table).cuda())
+        slots.append(torch.full((rows,), -5, dtype=torch.int32).cuda())
+    picked = ops.argmax_next_step(logits, ids, positions, first, slots, tables, page_size)
+    assert torch.equal(picked, ops.argmax(logits)) and torch.equal(ids, picked)
+    after = start + 1
+    assert positions.cpu().numpy().tolist() == after.tolist() and first.cpu().numpy().tolist() == after.tolist()
+    for width, table, slot in zip(widths, tables, slots):
+        page = table.cpu().numpy()[np.arange(rows), np.minimum(after // page_size, width - 1)]
+        want = np.where(page < 0, -1, page * page_size + after % page_size)
+        assert slot.cpu().numpy().tolist() == want.tolist()
+    with pytest.raises(KernelError):                                          # five groups; positions of another size
+        ops.argmax_next_step(logits, ids, positions, first, (slots * 5)[:5], (tables * 5)[:5], page_size)
+    with pytest.raises(KernelError):
+        ops.argmax_next_step(logits, ids, torch.zeros(rows + 1, dtype=torch.int32).cuda(), first, slots, tables, page_size)
 
 
 @pytest.mark.parametrize("vocab", [151936, 50257, 33])

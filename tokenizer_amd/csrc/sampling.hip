@@ -74,6 +74,84 @@ argmax_rows(const float* __restrict__ partial_v, const int* __restrict__ partial
   if (threadIdx.x == 0) out[row] = (at == 0x7fffffff) ? 0 : at;
 }
 
+// What the description of a decode step (one token per request, row i = request i) needs to describe the step
+// after it, in which every request is one position further: the picked ids as the next tokens, positions and first
+// positions one up, and for every cache group the slot of the new position from the request's row of the block
+// table (an entry past the row's end is not looked up: the last one stands in, and the host fills the description
+// in again before a step for which that matters; a page that is not there gives no slot).
+#define NEXT_STEP_GROUPS 4
+struct NextStep {
+  int* token_ids; int* positions; int* first_position;
+  int page_size, n_groups;
+  int* slots[NEXT_STEP_GROUPS];
+  const int* tables[NEXT_STEP_GROUPS];
+  int widths[NEXT_STEP_GROUPS];
+};
+
+// Stage two of the greedy pick as above, which also turns the step's description into the next step's: a run
+// of decode steps then needs nothing from the host between its steps.
+__global__ void __launch_bounds__(ARGMAX_THREADS)
+argmax_rows_next(const float* __restrict__ partial_v, const int* __restrict__ partial_i, int* __restrict__ out,
+                 int chunks, NextStep next) {
+  __shared__ float best_s[ARGMAX_THREADS / WAVE];
+  __shared__ int at_s[ARGMAX_THREADS / WAVE];
+  const int row = blockIdx.x;
+  float best = -INFINITY;
+  int at = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += ARGMAX_THREADS) {
+    const float v = partial_v[(size_t)row * chunks + c];
+    const int a = partial_i[(size_t)row * chunks + c];
+    if (better(v, a, best, at)) { best = v; at = a; }
+  }
+  block_best(best, at, best_s, at_s);
+  if (threadIdx.x == 0) {
+    const int id = (at == 0x7fffffff) ? 0 : at;
+    out[row] = id;
+    next.token_ids[row] = id;
+    const int p = next.positions[row] + 1;
+    next.positions[row] = p;
+    next.first_position[row] = p;
+#pragma unroll
+    for (int g = 0; g < NEXT_STEP_GROUPS; ++g) {
+      if (g < next.n_groups) {
+        const int width = next.widths[g];
+        const int page = next.tables[g][(size_t)row * width + min(p / next.page_size, width - 1)];
+        next.slots[g][row] = page < 0 ? -1 : page * next.page_size + p % next.page_size;
+      }
+    }
+  }
+}
+
+// token_ids, positions, first_position int32 [n_rows]; for each of the n_groups (at most four) cache groups
+// slots int32 [n_rows] and its block table int32 [n_rows, width].
+extern "C" int ta_argmax_next_step(const void* logits, void* out, void* partial_v, void* partial_i, int n_rows,
+                                   int vocab, int chunks, void* token_ids, void* positions, void* first_position,
+                                   int page_size, int n_groups, void* slots0, const void* table0, int width0,
+                                   void* slots1, const void* table1, int width1, void* slots2, const void* table2,
+                                   int width2, void* slots3, const void* table3, int width3, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (chunks < 1 || vocab < 1 || page_size < 1 || n_groups < 0 || n_groups > NEXT_STEP_GROUPS) return -1;
+  if (!logits || !out || !partial_v || !partial_i || !token_ids || !positions || !first_position) return -1;
+  NextStep next = {};
+  next.token_ids = (int*)token_ids; next.positions = (int*)positions; next.first_position = (int*)first_position;
+  next.page_size = page_size; next.n_groups = n_groups;
+  void* const slots[NEXT_STEP_GROUPS] = {slots0, slots1, slots2, slots3};
+  const void* const tables[NEXT_STEP_GROUPS] = {table0, table1, table2, table3};
+  const int widths[NEXT_STEP_GROUPS] = {width0, width1, width2, width3};
+  for (int g = 0; g < n_groups; ++g) {
+    if (!slots[g] || !tables[g] || widths[g] < 1) return -1;
+    next.slots[g] = (int*)slots[g]; next.tables[g] = (const int*)tables[g]; next.widths[g] = widths[g];
+  }
+  dim3 grid(chunks, n_rows);
+  argmax_pieces<<<grid, ARGMAX_THREADS, 0, stream>>>((const float*)logits, (float*)partial_v, (int*)partial_i,
+                                                    vocab, chunks);
+  int status = LAUNCH_STATUS();
+  if (status) return status;
+  argmax_rows_next<<<n_rows, ARGMAX_THREADS, 0, stream>>>((const float*)partial_v, (const int*)partial_i, (int*)out,
+                                                          chunks, next);
+  return LAUNCH_STATUS();
+}
+
 extern "C" int ta_argmax(const void* logits, void* out, void* partial_v, void* partial_i, int n_rows, int vocab,
                          int chunks, hipStream_t stream) {
   if (n_rows <= 0) return 0;

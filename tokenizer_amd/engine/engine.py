@@ -93,13 +93,26 @@ class StepGraph:
                 engine.model.decoder.forward(self.ctx, engine.layer_caches)
             torch.cuda.current_stream(device).wait_stream(side)
             torch.cuda.synchronize(device)
+            # A plain decode step (one token per request, its logits wanted) may end by turning its own description
+            # into the next step's on the device (`Ops.argmax_next_step`): in a run of such steps the host then
+            # has nothing to upload between them, as long as what it would upload is what the device holds already.
+            ctx = self.ctx
+            self.advances = (engine.NEXT_STEP_ON_DEVICE
+                             and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+                             and len(ctx.slots) <= getattr(ops, "NEXT_STEP_GROUPS", -1))
             self.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self.graph, pool=engine.graph_pool):
                 self.logits = engine.model.decoder.forward(self.ctx, engine.layer_caches)
-                self.ids = ops.argmax(self.logits) if self.logits.shape[0] else None
+                if self.advances:
+                    self.ids = ops.argmax_next_step(self.logits, ctx.token_ids, ctx.positions, ctx.first_position,
+                                                    ctx.slots, ctx.block_tables, ctx.page_size)
+                else:
+                    self.ids = ops.argmax(self.logits) if self.logits.shape[0] else None
         finally:
             ops.capturing = before
         self.uploaded = None
+        self.uploads = 0                            # times the description went to the device
+        self.on_device = None                       # what the device's copy of the description holds, where that is known
         self.last_used = 0
         self.draws = None                           # captured graphs of the sampler over these logits, made on demand
 
@@ -146,12 +159,39 @@ class StepGraph:
                                             filled_counts([len(e.tokens) for e in entries], [len(e.want) for e in entries]))
         if total != self.host.numel():
             raise ValueError("the packed batch does not fit the graph's buffers")
-        self.dev.copy_(self.host, non_blocking=True)
-        self.uploaded.record()
-        if tokens_on_device is not None:
-            self.dev[:len(entries)].copy_(tokens_on_device, non_blocking=True)   # the token ids lead the buffer
+        count = len(entries)
+        packed = self.host.numpy()
+        # (The token ids lead the buffer.  A step that takes them from this graph's last pick finds them in place.)
+        in_place = (self.advances and tokens_on_device is self.ids and self.on_device is not None
+                    and np.array_equal(packed[count:], self.on_device[count:]))
+        if not in_place:
+            self.dev.copy_(self.host, non_blocking=True)
+            self.uploaded.record()
+            self.uploads += 1
+            if tokens_on_device is not None:
+                self.dev[:count].copy_(tokens_on_device, non_blocking=True)
         self.graph.replay()
+        if self.advances:
+            self.on_device = self._next_description(packed, count, manager.page_size)
         return self.logits
+
+    def _next_description(self, packed: np.ndarray, count: int, page_size: int) -> np.ndarray:
+        """What `Ops.argmax_next_step` makes of a plain decode step's description (all but the token ids, which
+        only the device knows): the layout is `CacheCore::pack_batch`'s for `count` entries of one token."""
+        after = packed.copy()
+        positions = after[count:2 * count]
+        positions += 1
+        at = 3 * count + count + 1                         # past token ids, positions, entries of tokens, first rows
+        after[at:at + count] += 1                          # first positions
+        at += 4 * count                                    # past state slots, wanted rows (no tiles), single rows
+        rows = np.arange(count)
+        for _ in range(len(self.ctx.slots)):
+            table = after[at + count:at + count + count * self.width].reshape(count, self.width)
+            page = table[rows, np.minimum(positions // page_size, self.width - 1)]
+            after[at:at + count] = np.where(page < 0, -1, page * page_size + positions % page_size)
+            at += count + count * self.width
+        assert at == after.size
+        return after
 
 
 class Engine:
@@ -168,6 +208,14 @@ class Engine:
     GRAPH_TOKENS = 2048     # steps with more tokens than this are not captured: the device is the slower side
     GRAPH_AFTER = 3         # a shape is captured when it comes up for this many times ...
     SHAPES_REMEMBERED = 64  # ... among this many shapes seen last
+    # Whether the graphs of plain decode steps end with the kernel that writes the next step's description in place
+    # (see `StepGraph`): a decode step then needs neither the upload of its description nor the copy of the picked ids,
+    # two small copies of about 8 us together before a step of 0.8 to 1.5 ms at 0.5B sizes.  Off: such a graph must
+    # never be replayed without the host's check in `StepGraph.run` before it (each replay moves every request one
+    # position on, and positions that run past the pages a request holds make the attention read addresses that are
+    # not there), which is so for every replay in this package; it has been run through the tests that name it
+    # only, not through the whole suite and the serving workloads.
+    NEXT_STEP_ON_DEVICE = False
 
     def __init__(self, model: Model, num_pages: int | None = None, page_size: int = 16, max_requests: int = 8,
                  max_tokens: int | None = None, prefix_cache: bool = False, use_graphs: bool | None = None,

@@ -151,7 +151,7 @@ class Ops:
                      "ta_gemm_f32", "ta_gemm_bf16", "ta_gemm_bf16_splitk", "ta_gemm_skinny_bf16",
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
-                     "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_sample",
+                     "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_argmax_next_step", "ta_sample",
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
@@ -738,6 +738,41 @@ class Ops:
         partial_i = torch.empty((n_rows, chunks), dtype=torch.int32, device=logits.device)
         self._check(self.lib.ta_argmax(_ptr(logits), _ptr(out), _ptr(partial_v), _ptr(partial_i), n_rows, vocab,
                                        chunks, self._stream()), "argmax")
+        return out
+
+    NEXT_STEP_GROUPS = 4          # cache groups `argmax_next_step` can advance
+
+    def argmax_next_step(self, logits: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,
+                         first_position: torch.Tensor, slots: list[torch.Tensor], block_tables: list[torch.Tensor],
+                         page_size: int) -> torch.Tensor:
+        """`argmax` for a decode step of one token per request (row i of the logits = request i), which also turns
+        the step's description into the next step's, in place: the picked ids become `token_ids`, `positions` and
+        `first_position` go up by one, and every cache group's `slots` are looked up for the new positions in its
+        block table [B, width] (a position past the table's width takes the last entry; a page that is not there
+        gives slot -1).  All int32 [B]."""
+        _dev(logits, token_ids, positions, first_position, *slots, *block_tables)
+        _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits must be float32 [B, V]")
+        n_rows, vocab = logits.shape
+        _need(len(slots) == len(block_tables) <= self.NEXT_STEP_GROUPS, "one table per group of slots, four at most")
+        for t in (token_ids, positions, first_position, *slots):
+            _need(t.dtype == torch.int32 and t.numel() == n_rows and t.is_contiguous(), "the description is int32 [B]")
+        for table in block_tables:
+            _need(table.dtype == torch.int32 and table.dim() == 2 and table.shape[0] == n_rows and table.shape[1] >= 1
+                  and table.is_contiguous(), "block tables are int32 [B, width]")
+        _need(page_size >= 1, "page size")
+        out = torch.empty(n_rows, dtype=torch.int32, device=logits.device)
+        chunks = max(1, min(256, vocab // 2048, 2048 // max(1, n_rows)))
+        partial_v = torch.empty((n_rows, chunks), dtype=torch.float32, device=logits.device)
+        partial_i = torch.empty((n_rows, chunks), dtype=torch.int32, device=logits.device)
+        groups = []
+        for g in range(self.NEXT_STEP_GROUPS):
+            if g < len(slots):
+                groups += [_ptr(slots[g]), _ptr(block_tables[g]), int(block_tables[g].shape[1])]
+            else:
+                groups += [_ptr(None), _ptr(None), 0]
+        self._check(self.lib.ta_argmax_next_step(_ptr(logits), _ptr(out), _ptr(partial_v), _ptr(partial_i), n_rows, vocab,
+                                                 chunks, _ptr(token_ids), _ptr(positions), _ptr(first_position),
+                                                 int(page_size), len(slots), *groups, self._stream()), "argmax_next_step")
         return out
 
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniform: torch.Tensor,
