@@ -106,6 +106,51 @@ def test_packed_batch_matches_its_definition(seed, table_width, fill):
     manager.check_invariants()
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_the_next_decode_steps_description_is_what_packing_it_again_gives(seed):
+    """A step of single tokens, every request then one token further, packed again: the same as what
+    `next_decode_description` makes of the first description (the token ids aside), which is what the device is
+    left with when a decode graph ends with `Ops.argmax_next_step`.  Where a request needs a page it does not hold
+    yet, or a window gives one back, the two differ, and the engine uploads."""
+    from tokenizer_amd.engine.engine import next_decode_description
+    rng = random.Random(seed)
+    manager = CacheManager(needs(), num_pages=60, page_size=16, max_requests=6)
+    n_groups, width = len(manager.groups), 8
+    rids = list(range(rng.randint(1, 6)))
+    for rid in rids:
+        manager.add_request(rid)
+        held = rng.choice([1, 3, 15, 16, 31, 47, 60])
+        assert manager.reserve(rid, held + 1)
+        manager.advance(rid, held)
+
+    def packed():
+        entries = [StepEntry(rid, [rng.randrange(1000)], [0]) for rid in rids]
+        return build_context(entries, manager, "cpu", table_width=width)
+
+    def flat(ctx):
+        parts = [ctx.token_ids, ctx.positions, ctx.entry_of_token, ctx.cu_q, ctx.first_position, ctx.state_slots,
+                 ctx.want_rows, ctx.q_tiles.reshape(-1), ctx.decode_rows]
+        for g in range(n_groups):
+            parts += [ctx.slots[g], ctx.block_tables[g].reshape(-1)]
+        return np.concatenate([part.numpy() for part in parts])
+
+    for _ in range(20):
+        before = flat(packed())
+        tables = [[list(manager.table(rid, g)) for rid in rids] for g in range(n_groups)]
+        for rid in rids:
+            manager.advance(rid, manager.seq_len(rid) + 1)          # the step ran
+            assert manager.reserve(rid, manager.seq_len(rid) + 1)   # pages for the next one
+        predicted = next_decode_description(before, len(rids), 16, width, n_groups)
+        again = flat(packed())
+        same_tables = tables == [[list(manager.table(rid, g)) for rid in rids] for g in range(n_groups)]
+        n = len(rids)
+        assert np.array_equal(predicted[n:], again[n:]) == same_tables
+        if not same_tables:
+            # A new page or one given back: everything but the tables and the slots that hang on them still agrees.
+            assert np.array_equal(predicted[n:8 * n + 1], again[n:8 * n + 1])
+    manager.check_invariants()
+
+
 def test_a_fixed_width_leaves_out_pages_beyond_the_steps_last_token():
     """A prompt's pages are reserved whole while its first portions run: the request's table is then wider than a
     step's fixed width needs to be, and only the pages up to the step's last token are written."""

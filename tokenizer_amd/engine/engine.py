@@ -172,26 +172,29 @@ class StepGraph:
                 self.dev[:count].copy_(tokens_on_device, non_blocking=True)
         self.graph.replay()
         if self.advances:
-            self.on_device = self._next_description(packed, count, manager.page_size)
+            self.on_device = next_decode_description(packed, count, manager.page_size, self.width, len(self.ctx.slots))
         return self.logits
 
-    def _next_description(self, packed: np.ndarray, count: int, page_size: int) -> np.ndarray:
-        """What `Ops.argmax_next_step` makes of a plain decode step's description (all but the token ids, which
-        only the device knows): the layout is `CacheCore::pack_batch`'s for `count` entries of one token."""
-        after = packed.copy()
-        positions = after[count:2 * count]
-        positions += 1
-        at = 3 * count + count + 1                         # past token ids, positions, entries of tokens, first rows
-        after[at:at + count] += 1                          # first positions
-        at += 4 * count                                    # past state slots, wanted rows (no tiles), single rows
-        rows = np.arange(count)
-        for _ in range(len(self.ctx.slots)):
-            table = after[at + count:at + count + count * self.width].reshape(count, self.width)
-            page = table[rows, np.minimum(positions // page_size, self.width - 1)]
-            after[at:at + count] = np.where(page < 0, -1, page * page_size + positions % page_size)
-            at += count + count * self.width
-        assert at == after.size
-        return after
+
+def next_decode_description(packed: np.ndarray, count: int, page_size: int, width: int, n_groups: int) -> np.ndarray:
+    """What `Ops.argmax_next_step` makes of a plain decode step's description (all but the token ids, which only
+    the device knows): the layout is `CacheCore::pack_batch`'s for `count` entries of one token each, with tables of
+    `width` pages for each of the `n_groups` cache groups."""
+    after = packed.copy()
+    positions = after[count:2 * count]
+    positions += 1
+    at = 3 * count + count + 1                             # past token ids, positions, entries of tokens, first rows
+    after[at:at + count] += 1                              # first positions
+    at += 4 * count                                        # past state slots, wanted rows (no tiles), single rows
+    rows = np.arange(count)
+    for _ in range(n_groups):
+        table = after[at + count:at + count + count * width].reshape(count, width)
+        page = table[rows, np.minimum(positions // page_size, width - 1)]
+        after[at:at + count] = np.where(page < 0, -1, page * page_size + positions % page_size)
+        at += count + count * width
+    if at != after.size:
+        raise ValueError("not the description of a step of single tokens")
+    return after
 
 
 class Engine:
