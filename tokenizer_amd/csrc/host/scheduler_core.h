@@ -5,9 +5,10 @@
 // sequences return to the front of the queue, oldest first (369-376); a sequence that cannot fit in the whole
 // pool fails (473-487, 670-685).  Beyond the reference one iteration is a single mixed batch under a token
 // budget: one token for every decoding sequence first, then portions of prompts in order of arrival; or, with
-// `prompts_first`, the reference's own order within an iteration (new sequences are prefilled before the batched
-// decode, 788-805): portions of prompts take the budget first and decoding sequences what is left of it, so that
-// they wait while prompts stand in line and then decode together.
+// `prompts_first`, in the reference's order within an iteration (new sequences are prefilled before the batched
+// decode, 788-805), which under a budget means more than an order: portions of prompts take the budget first and
+// decoding sequences what is left of it, so that they wait while prompts stand in line and then decode together
+// (the reference has no budget: there every decoding sequence still gets its token in the same iteration).
 // Sampling, stop conditions and results stay with the caller; this class owns the token lists, the order of
 // work and every exchange with the cache manager.
 #pragma once

@@ -9,8 +9,9 @@ cannot fit in the whole pool fails with a message (473-487, 670-685).
 
 Beyond the reference, one iteration is a single mixed batch under a token budget: one token
 for every decoding sequence first, then portions of prompts in order of arrival
-(`SchedulerConfig.prompts_first` turns that round: the reference's order within an iteration,
-new sequences prefilled before the batched decode, 788-805).  A preempted
+(`SchedulerConfig.prompts_first` turns that round, as the reference orders an iteration, new
+sequences prefilled before the batched decode, 788-805; under a budget the decoding sequences
+then wait while prompts fill it, which the reference, having no budget, does not make them do).  A preempted
 sequence is recomputed from its prompt and the tokens it sampled so far, and nothing is
 sampled again for positions that already have a token.
 
