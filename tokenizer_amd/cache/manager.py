@@ -19,7 +19,7 @@ import numpy as np
 
 from .. import host as _host
 from ..parts.spec import CacheNeed
-from .allocator import PageAllocator, pages_for_len
+from .allocator import PageAllocator
 
 
 class OutOfPages(RuntimeError):

@@ -10,7 +10,7 @@ from ..config.base import ModelConfig
 from ..config.registry import get_architecture
 from ..parts import LayerCache, Runtime, build_model, cache_needs, expected_tensors
 from ..weights import load_weights, random_tensors, stored_form
-from .batch import StepContext, StepEntry, build_context, filled_counts
+from .batch import StepEntry, build_context, filled_counts
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}

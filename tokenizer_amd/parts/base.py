@@ -45,7 +45,7 @@ their Python.  The promise is the class's own: a subclass does not inherit it an
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Callable
+from typing import Any
 
 import torch
 
