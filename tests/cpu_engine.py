@@ -20,17 +20,22 @@ def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_si
     if counting:
         engine.step = step
 
-    def decode_greedy(rids, tokens, n_steps, on_step=None):
-        """`Engine.decode_greedy` as it behaves with captured graphs, one step at a time on the CPU: the ids of a
-        step reach `on_step` one step late, when the next step has already run, and when `on_step` returns False
-        the run ends behind that further step, whose ids are returned as well."""
+    def decode_run(rids, tokens, n_steps, on_step=None, draw=None):
+        """`Engine.decode_greedy` (and, with `draw`, `Engine.decode_sampled`) as it behaves with captured graphs, one
+        step at a time on the CPU: the ids of a step reach `on_step` one step late, when the next step has already
+        run (and taken its uniform numbers), and when `on_step` returns False the run ends behind that further
+        step, whose ids are returned as well."""
         from tokenizer_amd.engine import StepEntry
         if n_steps <= 0:
             return []
         ran, picked, current, go_on = [], [], [int(t) for t in tokens], True
         for k in range(n_steps):
             entries = [StepEntry(rid, [token], [0]) for rid, token in zip(rids, current)]
-            current = [int(t) for t in engine.argmax(engine.step(entries))]
+            logits = engine.step(entries)
+            if draw is None:
+                current = [int(t) for t in engine.argmax(logits)]
+            else:
+                current = [int(t) for t in engine.sample(logits, list(range(len(rids))), *draw(k))]
             ran.append(current)
             if k > 0:
                 picked.append(ran[k - 1])
@@ -46,7 +51,8 @@ def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_si
     # The scheduler runs greedy decode steps in bursts only over an engine that says it replays graphs; nothing is
     # captured here, the double only takes the scheduler (and greedy `generate`) down that road when asked to.
     if bursts:
-        engine.decode_greedy = decode_greedy
+        engine.decode_greedy = lambda rids, tokens, n_steps, on_step=None: decode_run(rids, tokens, n_steps, on_step)
+        engine.decode_sampled = lambda rids, tokens, n_steps, draw, on_step=None: decode_run(rids, tokens, n_steps, on_step, draw)
         engine.use_graphs = True
         engine._replays = lambda entries: False
     return engine

@@ -464,6 +464,50 @@ def test_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, dtype, 
     assert runs[0] == runs[2] and runs[1] == runs[3]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_drawn_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, dtype, monkeypatch):
+    """`decode_sampled` draws every step's ids on the device, feeds them to the next step there and reads them a
+    step late: with the same uniform numbers it gives what stepping and drawing one by one gives, across a change
+    of graph, with and without a nucleus cut; `draw` is asked once for every step that is launched, also when the
+    run is ended early."""
+    import random
+    from tokenizer_amd.engine import Engine, StepEntry
+    name = "B"
+    vocab = TINY[name][0]["vocab_size"]
+    monkeypatch.setattr(Engine, "GRAPH_BUCKET", 48)
+    prompts = {rid: random_ids(vocab, n, 70 + rid) for rid, n in enumerate([38, 5, 20])}
+    temperature = [0.8, 1.3, 1.0]
+    for top_p in ([1.0, 1.0, 1.0], [0.9, 1.0, 0.5]):
+        rng = random.Random(11)
+        uniforms = [[rng.random() for _ in prompts] for _ in range(40)]
+        runs = []
+        for pipelined in (True, False):
+            eng = engine_for(model_folders[name], dtype, max_tokens=512, max_requests=4)
+            first = []
+            for rid, ids in prompts.items():
+                eng.add_request(rid)
+                first.append(eng.argmax(eng.step([StepEntry(rid, ids, [len(ids) - 1])]))[0])
+            asked = []
+            draw = lambda k: (asked.append(k), (temperature, top_p, uniforms[len(asked) - 1]))[1]
+            if pipelined:
+                picked = eng.decode_sampled(list(prompts), first, 30, draw)
+                assert len(eng.graphs) >= 2 and asked == list(range(30))
+                more = eng.decode_sampled(list(prompts), picked[-1], 10, draw, on_step=lambda k, ids: k < 3)
+                assert len(more) == 5 and asked[30:] == [0, 1, 2, 3, 4]
+            else:
+                picked, current = [], first
+                for k in range(35):
+                    logits = eng.step([StepEntry(rid, [t], [0]) for rid, t in zip(prompts, current)])
+                    current = eng.sample(logits, [0, 1, 2], temperature, top_p, uniforms[k])
+                    picked.append(current)
+                picked, more = picked[:30], picked[30:]
+            runs.append(picked + more)
+            assert all(0 <= t < vocab for ids in picked + more for t in ids)
+            eng.cache.check_invariants()
+        assert runs[0] == runs[1]
+        assert len({tuple(ids) for ids in runs[0]}) > 20          # draws, not one id again and again
+
+
 def sharpened(folder, out_folder, factor):
     """A copy of a model folder whose query and key projections are scaled up: attention becomes nearly
     one-hot, so a wrong key, page or window edge changes the logits by far more than any rounding."""

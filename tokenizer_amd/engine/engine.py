@@ -116,21 +116,26 @@ class StepGraph:
         self.last_used = 0
         self.draws = None                           # captured graphs of the sampler over these logits, made on demand
 
-    def draw(self, engine: "Engine", temperature: list[float], top_p: list[float], uniform: list[float],
-             any_cut: bool) -> list[int]:
-        """Temperature / nucleus draws for every row of this graph's logits: the sampler's twenty small launches
-        are captured once (per kind: with or without the rounds of the nucleus cut) and replayed."""
+    def draw_on_device(self, engine: "Engine", temperature: list[float], top_p: list[float], uniform: list[float],
+                       any_cut: bool) -> torch.Tensor:
+        """Temperature / nucleus draws for every row of this graph's logits, left on the device (int32, one per
+        row; the rows past the given ones only fill the step up): the sampler's twenty small launches are captured
+        once (per kind: with or without the rounds of the nucleus cut) and replayed.  Nothing waits for the result
+        here."""
         rows = self.logits.shape[0]
-        given = len(temperature)                      # (the logits' rows past these only fill the step up: drawn and dropped)
+        given = len(temperature)
         fill = [1.0] * (rows - given)
         temperature, top_p, uniform = list(temperature) + fill, list(top_p) + fill, list(uniform) + [0.5] * (rows - given)
         if self.draws is None:
             self.draws = {}
             self.draw_host = torch.empty((3, rows), dtype=torch.float32).pin_memory()
             self.draw_params = torch.empty((3, rows), dtype=torch.float32, device=self.logits.device)
-            self.draw_ids = torch.empty(rows, dtype=torch.int32, device=self.logits.device)
+            self.draw_ids = torch.zeros(rows, dtype=torch.int32, device=self.logits.device)
+            self.draw_uploaded = torch.cuda.Event()
+        self.draw_uploaded.synchronize()              # the last draw's numbers have left the pinned buffer
         self.draw_host.copy_(torch.tensor([temperature, top_p, uniform], dtype=torch.float32))
         self.draw_params.copy_(self.draw_host, non_blocking=True)
+        self.draw_uploaded.record()
         ops = engine.model.runtime.ops
         launch = lambda: ops.sample(self.logits, self.draw_params[0], self.draw_params[1], self.draw_params[2],
                                     out=self.draw_ids, any_cut=any_cut)
@@ -144,7 +149,13 @@ class StepGraph:
             self.draws[any_cut] = captured
         else:
             captured.replay()
-        return [int(v) for v in self.draw_ids.cpu().tolist()][:given]      # (also waits until the pinned buffer is free again)
+        return self.draw_ids
+
+    def draw(self, engine: "Engine", temperature: list[float], top_p: list[float], uniform: list[float],
+             any_cut: bool) -> list[int]:
+        """The same draws, brought to the host: one id for each of the given rows."""
+        ids = self.draw_on_device(engine, temperature, top_p, uniform, any_cut)
+        return [int(v) for v in ids.cpu().tolist()][:len(temperature)]
 
     def run(self, engine: "Engine", entries: list[StepEntry], tokens_on_device: torch.Tensor | None = None) -> torch.Tensor:
         """Pack the batch's description into the fixed buffers again and replay.  `tokens_on_device`: the token
@@ -169,7 +180,7 @@ class StepGraph:
             self.uploaded.record()
             self.uploads += 1
             if tokens_on_device is not None:
-                self.dev[:count].copy_(tokens_on_device, non_blocking=True)
+                self.dev[:count].copy_(tokens_on_device[:count], non_blocking=True)
         self.graph.replay()
         if self.advances:
             self.on_device = next_decode_description(packed, count, manager.page_size, self.width, len(self.ctx.slots))
@@ -310,23 +321,34 @@ class Engine:
         called as each step's ids arrive; if it returns False the run ends after the step already launched (whose
         ids are still returned: the caller drops what it does not want; the cache holds those tokens too).
         Without captured graphs the steps run one by one through `step`."""
+        return self._decode_run(rids, tokens, n_steps, on_step, None)
+
+    def decode_sampled(self, rids: list, tokens: list[int], n_steps: int, draw, on_step=None) -> list[list[int]]:
+        """The same run of decode steps with temperature / nucleus draws in place of the greedy pick.  `draw(k)`
+        gives step k's (temperature, top_p, uniform) lists, one number of each per request; it is asked when step
+        k is launched, once for every step that runs (so a request's generator hands out exactly one uniform
+        number per token it is given, also when the run ends early)."""
+        return self._decode_run(rids, tokens, n_steps, on_step, draw)
+
+    def _decode_run(self, rids: list, tokens: list[int], n_steps: int, on_step, draw) -> list[list[int]]:
         if n_steps <= 0:
             return []
         if len(rids) != len(tokens) or not rids:
             raise ValueError("one next token per request")
+        count = len(rids)
         if not self.use_graphs:
             picked, current = [], list(tokens)
             for k in range(n_steps):
-                current = self.argmax(self.step([StepEntry(rid, [int(t)], [0]) for rid, t in zip(rids, current)]))
+                logits = self.step([StepEntry(rid, [int(t)], [0]) for rid, t in zip(rids, current)])
+                current = self.argmax(logits) if draw is None else self.sample(logits, list(range(count)), *draw(k))
                 picked.append(list(current))
                 if on_step is not None and on_step(k, picked[-1]) is False:
                     break
             return picked
-        count = len(rids)
         landing = [torch.empty(count, dtype=torch.int32).pin_memory() for _ in range(2)]
         arrived = [torch.cuda.Event(), torch.cuda.Event()]
         picked: list[list[int]] = []
-        previous: StepGraph | None = None
+        previous: torch.Tensor | None = None           # where the step before left its ids, on the device
         go_on = True
         for k in range(n_steps):
             # Only the first step's token ids are known here; later steps take theirs from the step before.
@@ -334,18 +356,22 @@ class Engine:
             self.validate(entries)
             self.reserve(entries)
             graph = self._graph_for(entries)
-            graph.run(self, entries, tokens_on_device=previous.ids if previous is not None else None)
+            graph.run(self, entries, tokens_on_device=previous)
             for entry in entries:
                 self.cache.advance(entry.rid, self.cache.seq_len(entry.rid) + 1)
             self.steps += 1
-            landing[k % 2].copy_(graph.ids, non_blocking=True)      # queued before the next replay overwrites the ids
+            if draw is None:
+                previous = graph.ids
+            else:
+                temperature, top_p, uniform = draw(k)
+                previous = graph.draw_on_device(self, temperature, top_p, uniform, any(p < 1.0 for p in top_p))
+            landing[k % 2].copy_(previous[:count], non_blocking=True)   # queued before the next replay overwrites the ids
             arrived[k % 2].record()
             if k > 0:
                 arrived[(k - 1) % 2].synchronize()
                 picked.append(landing[(k - 1) % 2].tolist())
                 if on_step is not None and on_step(k - 1, picked[-1]) is False:
                     go_on = False
-            previous = graph
             if not go_on:
                 break
         last = len(picked)

@@ -281,19 +281,25 @@ class Scheduler:
     # ---------------------------------------------------------------------- bursts
     def _burst_length(self, plan: list[tuple[Sequence, int, int, bool]]) -> int:
         """How many decode steps may follow each other on the device without a decision of the host between them:
-        more than one only when the step is nothing but greedy decoding (the ids a step picks feed the next one
-        there, `Engine.decode_greedy`), nothing waits that could join, no sequence reaches its last token before
-        the burst's last step, and the pages for all those tokens of all sequences are there now (a burst the pool
+        more than one only when the step is nothing but decoding, greedy for every sequence or drawn on the device
+        for every sequence (the ids a step picks feed the next one there, `Engine.decode_greedy` and
+        `Engine.decode_sampled`), nothing waits that could join, no sequence reaches its last token before the
+        burst's last step, and the pages for all those tokens of all sequences are there now (a burst the pool
         cannot hold whole is halved until it can)."""
         burst = min(self.config.decode_burst, 64)
         if burst < 2 or not getattr(self.engine, "use_graphs", False) or not hasattr(self.engine, "decode_greedy"):
+            return 1
+        greedy = [seq.cursor.is_greedy for seq, _, _, _ in plan]
+        if any(greedy) and not all(greedy):
+            return 1                     # picks and draws side by side: one step at a time
+        if not any(greedy) and not (hasattr(self.engine, "decode_sampled") and hasattr(self.engine, "sample")):
             return 1
         if self._get(_WAITING) and len(plan) < self.config.max_batch_size:
             return 1                     # the queue's front waits for pages: a finished sequence should let it in at once
         if len(plan) != self._get(_RUNNING):
             return 1                     # the token budget left a running sequence out of this step: it is next
         for seq, first, count, completes in plan:
-            if count != 1 or first < seq.prompt_len or not completes or not seq.cursor.is_greedy:
+            if count != 1 or first < seq.prompt_len or not completes:
                 return 1
             burst = min(burst, seq.params.max_tokens - seq.cursor.produced)
         # The pages for all those tokens of all the sequences are taken together or not at all: a burst that only
@@ -316,9 +322,10 @@ class Scheduler:
         return burst
 
     def _run_burst(self, plan: list[tuple[Sequence, int, int, bool]], burst: int) -> None:
-        """`burst` greedy decode steps of the planned sequences back to back.  Ids reach the host one step late;
-        when one of them ends a sequence (end-of-sequence id, stop string, the caller's callback), the step after
-        it is already on its way: the others keep its tokens, the finished sequence's one is dropped."""
+        """`burst` decode steps of the planned sequences back to back, all greedy or all drawn on the device (each
+        sequence's generator gives one uniform number for every step that is launched).  Ids reach the host one
+        step late; when one of them ends a sequence (end-of-sequence id, stop string, the caller's callback), the
+        step after it is already on its way: the others keep its tokens, the finished sequence's one is dropped."""
         seqs = [seq for seq, _, _, _ in plan]
         tokens = [self._tokens(seq.id, first, 1)[0] for seq, first, _, _ in plan]
         handled = 0
@@ -346,7 +353,14 @@ class Scheduler:
                     self._lib.ta_sched_append_token(self._core, seq.id, int(outcome))
             return go_on
 
-        picked = self.engine.decode_greedy([seq.id for seq in seqs], tokens, burst, on_step=lambda k, ids: take(ids))
+        rids = [seq.id for seq in seqs]
+        if seqs[0].cursor.is_greedy:
+            picked = self.engine.decode_greedy(rids, tokens, burst, on_step=lambda k, ids: take(ids))
+        else:
+            cursors = [seq.cursor for seq in seqs]
+            draw = lambda k: ([c.params.temperature for c in cursors], [c.params.top_p for c in cursors],
+                              [c.next_uniform() for c in cursors])
+            picked = self.engine.decode_sampled(rids, tokens, burst, draw, on_step=lambda k, ids: take(ids))
         for ids in picked[handled:]:      # the step that was under way when a sequence ended
             take(ids)
 
