@@ -32,10 +32,14 @@ def cpu_engine(folder, num_pages=64, max_requests=8, prefix_cache=False, page_si
         for k in range(n_steps):
             entries = [StepEntry(rid, [token], [0]) for rid, token in zip(rids, current)]
             logits = engine.step(entries)
-            if draw is None:
-                current = [int(t) for t in engine.argmax(logits)]
-            else:
-                current = [int(t) for t in engine.sample(logits, list(range(len(rids))), *draw(k))]
+            current = [int(t) for t in engine.argmax(logits)]
+            if draw is not None:                              # rows with temperature 0 keep the greedy pick
+                temperature, top_p, uniform = draw(k)
+                warm = [row for row, t in enumerate(temperature) if t != 0]
+                drawn = engine.sample(logits, warm, [temperature[r] for r in warm], [top_p[r] for r in warm],
+                                      [uniform[r] for r in warm]) if warm else []
+                for row, token in zip(warm, drawn):
+                    current[row] = int(token)
             ran.append(current)
             if k > 0:
                 picked.append(ran[k - 1])

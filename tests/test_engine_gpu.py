@@ -476,8 +476,10 @@ def test_drawn_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, d
     vocab = TINY[name][0]["vocab_size"]
     monkeypatch.setattr(Engine, "GRAPH_BUCKET", 48)
     prompts = {rid: random_ids(vocab, n, 70 + rid) for rid, n in enumerate([38, 5, 20])}
-    temperature = [0.8, 1.3, 1.0]
-    for top_p in ([1.0, 1.0, 1.0], [0.9, 1.0, 0.5]):
+    # (In the last round of cases the second request is greedy: it keeps the greedy pick among the others' draws.)
+    for temperature, top_p in (([0.8, 1.3, 1.0], [1.0, 1.0, 1.0]), ([0.8, 1.3, 1.0], [0.9, 1.0, 0.5]),
+                               ([0.8, 0.0, 1.0], [0.9, 1.0, 1.0])):
+        warm = [row for row, t in enumerate(temperature) if t != 0]
         rng = random.Random(11)
         uniforms = [[rng.random() for _ in prompts] for _ in range(40)]
         runs = []
@@ -498,7 +500,11 @@ def test_drawn_decode_steps_back_to_back_equal_steps_one_by_one(model_folders, d
                 picked, current = [], first
                 for k in range(35):
                     logits = eng.step([StepEntry(rid, [t], [0]) for rid, t in zip(prompts, current)])
-                    current = eng.sample(logits, [0, 1, 2], temperature, top_p, uniforms[k])
+                    current = eng.argmax(logits)
+                    drawn = eng.sample(logits, warm, [temperature[r] for r in warm], [top_p[r] for r in warm],
+                                       [uniforms[k][r] for r in warm])
+                    for row, token in zip(warm, drawn):
+                        current[row] = token
                     picked.append(current)
                 picked, more = picked[:30], picked[30:]
             runs.append(picked + more)

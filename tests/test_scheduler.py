@@ -50,9 +50,10 @@ def test_warm_requests_in_a_batch_draw_as_they_would_alone(model_folders):
 
 
 def test_warm_requests_decode_in_bursts_and_draw_as_they_would_alone(model_folders):
-    """Requests that all draw with a temperature decode in bursts too (`Engine.decode_sampled`: the draws stay on
-    the device, each request's generator gives one uniform number for every step that is launched); one of them
-    ends early on an end-of-sequence id in the middle of a burst, and every one gets the tokens it gets alone."""
+    """Requests that draw with a temperature decode in bursts too, a greedy one among them (`Engine.decode_sampled`:
+    the draws stay on the device, each drawing request's generator gives one uniform number for every step that is
+    launched); one of them ends early on an end-of-sequence id in the middle of a burst, and every one gets the
+    tokens it gets alone."""
     folder = model_folders["B"]
     engine = cpu_engine(folder, bursts=True)
     runs = []
@@ -60,10 +61,11 @@ def test_warm_requests_decode_in_bursts_and_draw_as_they_would_alone(model_folde
     engine.decode_sampled = lambda rids, tokens, n_steps, draw, on_step=None: (
         runs.append((len(rids), n_steps)), inner(rids, tokens, n_steps, draw, on_step))[1]
     sched = Scheduler(engine, SchedulerConfig(decode_burst=8))
-    ps = prompts(3, [4, 9, 2], vocab=384)
+    ps = prompts(4, [4, 9, 2, 6], vocab=384)
     params = [GenerateParams(max_tokens=21, temperature=1.3, top_p=0.95, seed=5),
               GenerateParams(max_tokens=30, temperature=0.7, top_p=1.0, seed=6),
-              GenerateParams(max_tokens=17, temperature=1.0, top_p=0.6, seed=5)]
+              GenerateParams(max_tokens=17, temperature=1.0, top_p=0.6, seed=5),
+              GenerateParams.greedy(25)]                      # a greedy one among them keeps its greedy picks
     alone = [solo(folder, p, q) for p, q in zip(ps, params)]
     params[1].eos = [alone[1].tokens[12]]                    # the second request ends where it first meets this id
     alone[1] = solo(folder, ps[1], params[1])
@@ -72,7 +74,7 @@ def test_warm_requests_decode_in_bursts_and_draw_as_they_would_alone(model_folde
     results = sched.run()
     for rid, want in zip(ids, alone):
         assert (results[rid].tokens, results[rid].reason) == (want.tokens, want.reason)
-    assert runs and runs[0] == (3, 8) and any(count == 2 for count, _ in runs)     # bursts of all three, then of two
+    assert runs and runs[0] == (4, 8) and any(count == 3 for count, _ in runs)     # bursts of all four, then of three
     sched.assert_idle()
 
 

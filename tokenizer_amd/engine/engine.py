@@ -327,8 +327,20 @@ class Engine:
         """The same run of decode steps with temperature / nucleus draws in place of the greedy pick.  `draw(k)`
         gives step k's (temperature, top_p, uniform) lists, one number of each per request; it is asked when step
         k is launched, once for every step that runs (so a request's generator hands out exactly one uniform
-        number per token it is given, also when the run ends early)."""
+        number per token it is given, also when the run ends early).  A request whose temperature is 0 keeps the
+        greedy pick (its other two numbers are not looked at)."""
         return self._decode_run(rids, tokens, n_steps, on_step, draw)
+
+    @staticmethod
+    def _warm_numbers(temperature, top_p, uniform):
+        """The sampler's numbers for a step in which rows with temperature 0 take the greedy pick instead: those
+        rows are drawn with harmless numbers and their draws thrown away.  Returns the lists and which rows are
+        greedy."""
+        greedy = [t == 0 for t in temperature]
+        if not any(greedy):
+            return list(temperature), list(top_p), list(uniform), greedy
+        return ([1.0 if g else t for g, t in zip(greedy, temperature)], [1.0 if g else p for g, p in zip(greedy, top_p)],
+                [0.5 if g else u for g, u in zip(greedy, uniform)], greedy)
 
     def _decode_run(self, rids: list, tokens: list[int], n_steps: int, on_step, draw) -> list[list[int]]:
         if n_steps <= 0:
@@ -340,7 +352,11 @@ class Engine:
             picked, current = [], list(tokens)
             for k in range(n_steps):
                 logits = self.step([StepEntry(rid, [int(t)], [0]) for rid, t in zip(rids, current)])
-                current = self.argmax(logits) if draw is None else self.sample(logits, list(range(count)), *draw(k))
+                current = self.argmax(logits)
+                if draw is not None:
+                    temperature, top_p, uniform, greedy = self._warm_numbers(*draw(k))
+                    drawn = self.sample(logits, list(range(count)), temperature, top_p, uniform)
+                    current = [pick if g else token for g, pick, token in zip(greedy, current, drawn)]
                 picked.append(list(current))
                 if on_step is not None and on_step(k, picked[-1]) is False:
                     break
@@ -349,6 +365,7 @@ class Engine:
         arrived = [torch.cuda.Event(), torch.cuda.Event()]
         picked: list[list[int]] = []
         previous: torch.Tensor | None = None           # where the step before left its ids, on the device
+        greedy_rows, greedy_mask = None, None          # which requests keep the greedy pick in a run with draws
         go_on = True
         for k in range(n_steps):
             # Only the first step's token ids are known here; later steps take theirs from the step before.
@@ -363,8 +380,12 @@ class Engine:
             if draw is None:
                 previous = graph.ids
             else:
-                temperature, top_p, uniform = draw(k)
+                temperature, top_p, uniform, greedy = self._warm_numbers(*draw(k))
                 previous = graph.draw_on_device(self, temperature, top_p, uniform, any(p < 1.0 for p in top_p))
+                if any(greedy):
+                    if greedy != greedy_rows:
+                        greedy_rows, greedy_mask = greedy, torch.tensor(greedy, device=previous.device)
+                    previous = torch.where(greedy_mask, graph.ids[:count], previous[:count])
             landing[k % 2].copy_(previous[:count], non_blocking=True)   # queued before the next replay overwrites the ids
             arrived[k % 2].record()
             if k > 0:

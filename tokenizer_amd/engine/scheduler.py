@@ -281,19 +281,16 @@ class Scheduler:
     # ---------------------------------------------------------------------- bursts
     def _burst_length(self, plan: list[tuple[Sequence, int, int, bool]]) -> int:
         """How many decode steps may follow each other on the device without a decision of the host between them:
-        more than one only when the step is nothing but decoding, greedy for every sequence or drawn on the device
-        for every sequence (the ids a step picks feed the next one there, `Engine.decode_greedy` and
-        `Engine.decode_sampled`), nothing waits that could join, no sequence reaches its last token before the
+        more than one only when the step is nothing but decoding, greedy or drawn on the device (the ids a step
+        picks feed the next one there, `Engine.decode_greedy` and `Engine.decode_sampled`), nothing waits that could join, no sequence reaches its last token before the
         burst's last step, and the pages for all those tokens of all sequences are there now (a burst the pool
         cannot hold whole is halved until it can)."""
         burst = min(self.config.decode_burst, 64)
         if burst < 2 or not getattr(self.engine, "use_graphs", False) or not hasattr(self.engine, "decode_greedy"):
             return 1
-        greedy = [seq.cursor.is_greedy for seq, _, _, _ in plan]
-        if any(greedy) and not all(greedy):
-            return 1                     # picks and draws side by side: one step at a time
-        if not any(greedy) and not (hasattr(self.engine, "decode_sampled") and hasattr(self.engine, "sample")):
-            return 1
+        if (not all(seq.cursor.is_greedy for seq, _, _, _ in plan)
+                and not (hasattr(self.engine, "decode_sampled") and hasattr(self.engine, "sample"))):
+            return 1                     # draws that only the host can make: one step at a time
         if self._get(_WAITING) and len(plan) < self.config.max_batch_size:
             return 1                     # the queue's front waits for pages: a finished sequence should let it in at once
         if len(plan) != self._get(_RUNNING):
@@ -322,8 +319,8 @@ class Scheduler:
         return burst
 
     def _run_burst(self, plan: list[tuple[Sequence, int, int, bool]], burst: int) -> None:
-        """`burst` decode steps of the planned sequences back to back, all greedy or all drawn on the device (each
-        sequence's generator gives one uniform number for every step that is launched).  Ids reach the host one
+        """`burst` decode steps of the planned sequences back to back, greedy or drawn on the device (the generator
+        of a sequence that draws gives one uniform number for every step that is launched).  Ids reach the host one
         step late; when one of them ends a sequence (end-of-sequence id, stop string, the caller's callback), the
         step after it is already on its way: the others keep its tokens, the finished sequence's one is dropped."""
         seqs = [seq for seq, _, _, _ in plan]
@@ -354,12 +351,13 @@ class Scheduler:
             return go_on
 
         rids = [seq.id for seq in seqs]
-        if seqs[0].cursor.is_greedy:
+        cursors = [seq.cursor for seq in seqs]
+        if all(c.is_greedy for c in cursors):
             picked = self.engine.decode_greedy(rids, tokens, burst, on_step=lambda k, ids: take(ids))
         else:
-            cursors = [seq.cursor for seq in seqs]
+            # (A greedy sequence among them has temperature 0, keeps the greedy pick and has no number to give.)
             draw = lambda k: ([c.params.temperature for c in cursors], [c.params.top_p for c in cursors],
-                              [c.next_uniform() for c in cursors])
+                              [0.5 if c.is_greedy else c.next_uniform() for c in cursors])
             picked = self.engine.decode_sampled(rids, tokens, burst, draw, on_step=lambda k, ids: take(ids))
         for ids in picked[handled:]:      # the step that was under way when a sequence ended
             take(ids)
