@@ -58,9 +58,12 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
             done = Sampled([], "", [], StopReason.Cancelled, 0)
         else:
             outcome = _next(engine, cursor, logits, token_bytes, on_chunk)
-            if not isinstance(outcome, Sampled) and cursor.is_greedy and hasattr(engine, "decode_greedy"):
-                # Greedy: the remaining steps run back to back on the device; the cursor sees each id one step
-                # late and ends the run when it stops (at most one forward is then run for nothing).
+            on_device = hasattr(engine, "decode_greedy") and (
+                cursor.is_greedy or (hasattr(engine, "decode_sampled") and hasattr(engine, "sample")))
+            if not isinstance(outcome, Sampled) and on_device:
+                # The remaining steps run back to back on the device, greedy picks or draws (the cursor gives a
+                # step's uniform number when it is launched); the cursor sees each id one step late and ends the
+                # run when it stops (at most one forward is then run for nothing).
                 ended = []
 
                 def on_step(_k, ids):
@@ -70,7 +73,11 @@ def generate_with(engine, prompt: list[int], params: GenerateParams, token_bytes
                         return False
                     return True
 
-                engine.decode_greedy([rid], [int(outcome)], params.max_tokens - cursor.produced, on_step)
+                if cursor.is_greedy:
+                    engine.decode_greedy([rid], [int(outcome)], params.max_tokens - cursor.produced, on_step)
+                else:
+                    draw = lambda _k: ([params.temperature], [params.top_p], [cursor.next_uniform()])
+                    engine.decode_sampled([rid], [int(outcome)], params.max_tokens - cursor.produced, draw, on_step)
                 outcome = ended[0]
             while not isinstance(outcome, Sampled):
                 logits = engine.step([StepEntry(rid, [int(outcome)], [0])])
