@@ -161,7 +161,7 @@ def run_prefill(model, repeats: int = 7, portion: int | None = None):
 
 
 def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0, token_budget: int = 2048,
-                 prompts_first: bool = False) -> dict:
+                 prompts_first: bool = False, decode_burst: int | None = None) -> dict:
     """A serving workload through the scheduler: every request is admitted, its prompt cut into portions under
     the token budget beside the others' decode tokens (or, `prompts_first`, ahead of them), decoded greedily to
     its length, and freed."""
@@ -192,7 +192,8 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
     for attempt in ("warm-up", "timed"):        # the first pass captures the decode graphs and warms the library
         sched = Scheduler(engine, SchedulerConfig(max_batch_size=64, max_waiting=64, num_blocks=pages,
                                                   prefix_cache=prefix_cache, max_num_batched_tokens=token_budget,
-                                                  prompts_first=prompts_first))
+                                                  prompts_first=prompts_first,
+                                                  **({} if decode_burst is None else {"decode_burst": decode_burst})))
         torch.cuda.synchronize()
         started = time.perf_counter()
         params = lambda i: (GenerateParams.greedy(new_tokens) if temperature == 0 else
@@ -220,6 +221,7 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
                        "head_dim": cfg.derived_head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                        "requests": len(prompts), "prompt_tokens": sum(len(p) for p in prompts),
                        "new_tokens_each": new_tokens, "token_budget": token_budget, "prompts_first": prompts_first,
+                       "decode_burst": sched.config.decode_burst,
                        "prefix_cache": prefix_cache,
                        "pages": pages, "page_size": 16, "temperature": temperature},
             "scheduler": {"steps": stats.steps, "tokens_forwarded": stats.tokens_forwarded, "max_running": stats.max_running,
@@ -341,6 +343,8 @@ def main() -> int:
                         help="with --workload: the most tokens a step of the scheduler may hold")
     parser.add_argument("--prompts-first", action="store_true",
                         help="with --workload: portions of prompts take the token budget before decoding requests do")
+    parser.add_argument("--decode-burst", type=int, default=None,
+                        help="with --workload: decode steps the scheduler lets run back to back (its default: 16)")
     parser.add_argument("--temperature", type=float, default=0.0,
                         help="with --workload: draw with this temperature and top_p 0.95 instead of greedy picks")
     parser.add_argument("--prompt-len", type=int, default=None,
@@ -364,7 +368,7 @@ def main() -> int:
         return 0
     if args.workload:
         print(json.dumps(run_workload(args.workload, args.layers, args.dtype, args.temperature, args.token_budget,
-                                      args.prompts_first)), flush=True)
+                                      args.prompts_first, args.decode_burst)), flush=True)
         return 0
     sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
     if args.attention:
