@@ -378,7 +378,7 @@ def requests_of_every_kind(rng, vocab, seed):
     return sorted(plan, key=lambda item: item[0])
 
 
-def run_requests_of_every_kind(make_engine, folder, vocab, seed):
+def run_requests_of_every_kind(make_engine, folder, vocab, seed, prompts_first=False):
     """Drive a scheduler over `make_engine(...)` with random limits through such requests; every result must be
     what the same request gives when it is generated alone."""
     import random
@@ -387,7 +387,7 @@ def run_requests_of_every_kind(make_engine, folder, vocab, seed):
     config = SchedulerConfig(max_batch_size=rng.choice([1, 2, 4, 6]), num_blocks=num_pages,
                              prefix_cache=rng.random() < 0.5, max_num_batched_tokens=rng.choice([8, 24, 64]),
                              prefill_chunk=rng.choice([None, 7, 16]), max_waiting=64,
-                             decode_burst=rng.choice([1, 4, 16]))
+                             decode_burst=rng.choice([1, 4, 16]), prompts_first=prompts_first)
     engine = make_engine(folder, num_pages=num_pages, max_requests=config.max_batch_size,
                          prefix_cache=config.prefix_cache)
     alone = make_engine(folder, num_pages=40, max_requests=1, prefix_cache=False)
@@ -415,15 +415,17 @@ def run_requests_of_every_kind(make_engine, folder, vocab, seed):
     sched.assert_idle()
 
 
+@pytest.mark.parametrize("prompts_first", [False, True])
 @pytest.mark.parametrize("seed", range(8))
-def test_requests_of_every_kind_get_what_they_get_alone(model_folders, seed):
+def test_requests_of_every_kind_get_what_they_get_alone(model_folders, seed, prompts_first):
     """Greedy and warm requests, nucleus cuts, end-of-sequence ids, stop strings and zero budgets side by side, under
-    random pools, batch caps, token budgets and portion sizes: tokens, text, chunks, reason and counts of every
-    request equal those of the request generated alone (qwen-server/src/engine.rs:1328-1420 widened)."""
+    random pools, batch caps, token budgets and portion sizes, decoding or prompts first: tokens, text, chunks,
+    reason and counts of every request equal those of the request generated alone
+    (qwen-server/src/engine.rs:1328-1420 widened)."""
     name = "ABC"[seed % 3]
     vocab = {"A": 256, "B": 384, "C": 320}[name]
     run_requests_of_every_kind(lambda folder, **kw: cpu_engine(folder, counting=False, bursts=True, **kw), model_folders[name],
-                               vocab, seed)
+                               vocab, seed, prompts_first)
 
 
 def test_a_step_that_may_not_reserve_refuses_an_entry_without_pages(model_folders):

@@ -235,8 +235,9 @@ def test_random_arrivals_pools_and_budgets_on_the_device(model_folders, seed, pr
 @pytest.mark.parametrize("seed", range(8, 24))
 def test_requests_of_every_kind_on_the_device(model_folders, seed):
     """The host-side test of the same name on the kernels, in float32 with graphs, bursts of decode steps and
-    draws on the device: every request gets what it gets alone."""
+    draws on the device (the later seeds with prompts before decoding): every request gets what it gets alone."""
     from test_scheduler import run_requests_of_every_kind
     name = "ABC"[seed % 3]
     vocab = {"A": 256, "B": 384, "C": 320}[name]
-    run_requests_of_every_kind(lambda folder, **kw: engine_for(folder, "float32", **kw), model_folders[name], vocab, seed)
+    run_requests_of_every_kind(lambda folder, **kw: engine_for(folder, "float32", **kw), model_folders[name], vocab, seed,
+                               prompts_first=seed >= 16)
