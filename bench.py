@@ -4,7 +4,8 @@
 
 A step is one decode step of the whole batch.  The default run prefills 8 prompts of 2,048
 random ids and decodes every request on to 4,096 tokens (8 warm-up steps, 2,040 timed ones); it
-also times a prefill of 2,048 tokens and the same decoding at batch 1 and 64, and prints one
+also times a prefill of 2,048 tokens, the same decoding at batch 1 and 64 and, at the record's own sizes, the
+serving workload mixed-0.5b under a token budget of 512 (with decoding and with prompts first), and prints one
 JSON line.
 
     python bench.py --workload mixed-1.5b | mixed-0.5b | prefix-7b [--token-budget N] [--prompts-first]
@@ -161,7 +162,7 @@ def run_prefill(model, repeats: int = 7, portion: int | None = None):
 
 
 def run_workload(name: str, layers: int | None, dtype: str, temperature: float = 0.0, token_budget: int = 2048,
-                 prompts_first: bool = False, decode_burst: int | None = None) -> dict:
+                 prompts_first: bool = False, decode_burst: int | None = None, model=None) -> dict:
     """A serving workload through the scheduler: every request is admitted, its prompt cut into portions under
     the token budget beside the others' decode tokens (or, `prompts_first`, ahead of them), decoded greedily to
     its length, and freed."""
@@ -183,8 +184,9 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
         raise SystemExit(f"unknown workload {name!r}")
     full_layers = raw["num_hidden_layers"]
     cfg = Qwen2Config.from_dict(dict(raw, num_hidden_layers=layers or full_layers))
-    log(f"building random weights ({cfg.num_hidden_layers} of {full_layers} layers, {dtype})")
-    model = random_model(cfg, seed=0, dtype=dtype, device="cuda:0")
+    if model is None:
+        log(f"building random weights ({cfg.num_hidden_layers} of {full_layers} layers, {dtype})")
+        model = random_model(cfg, seed=0, dtype=dtype, device="cuda:0")
     pages = sum(-(-(len(p) + new_tokens) // 16) for p in prompts) + 16
     engine = Engine(model, num_pages=pages, page_size=16, max_requests=64, prefix_cache=prefix_cache)
     log(f"{name}: {len(prompts)} requests, {sum(len(p) for p in prompts)} prompt tokens, {new_tokens} new tokens each")
@@ -447,6 +449,20 @@ def main() -> int:
         if args.dtype == "bfloat16":
             record["prefill"]["measured_peak_tflops"] = reached["bf16_gemm_tflops"]
             record["prefill"]["frac_of_measured"] = round(flops / seconds / (reached["bf16_gemm_tflops"] * 1e12), 5)
+        if args.size == "0.5b" and args.layers == full_layers:
+            # The serving workload at these sizes through the scheduler (64 requests, prompts of 128 to 2,048 ids,
+            # 256 new tokens each, a token budget of 512), with decoding and with prompts first.  What goes wrong
+            # here is said in the record and does not cost it the figures above.
+            try:
+                serving = {"workload": "mixed-0.5b", "token_budget": 512, "unit": "output tokens/s"}
+                for key, first in (("decoding_first", False), ("prompts_first", True)):
+                    log(f"serving workload mixed-0.5b, budget 512, {key.replace('_', ' ')}")
+                    run = run_workload("mixed-0.5b", None, args.dtype, token_budget=512, prompts_first=first, model=model)
+                    serving[key] = run["value"]
+                    serving[key + "_s"] = run["seconds"]
+                record["serving"] = serving
+            except Exception as err:                                  # noqa: BLE001 (whatever it is, it is reported)
+                record["serving"] = {"error": f"{type(err).__name__}: {err}"[:300]}
     print(json.dumps(record), flush=True)
     return 0
 
