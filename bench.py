@@ -5,8 +5,8 @@
 A step is one decode step of the whole batch.  The default run prefills 8 prompts of 2,048
 random ids and decodes every request on to 4,096 tokens (8 warm-up steps, 2,040 timed ones); it
 also times a prefill of 2,048 tokens, the same decoding at batch 1 and 64 and, at the record's own sizes, the
-serving workload mixed-0.5b under a token budget of 512 (with decoding and with prompts first), and prints one
-JSON line.
+serving workload mixed-0.5b under a token budget of 512 (with decoding and with prompts first) and the decoding
+at batch 8 at Qwen2.5-1.5B and 7B sizes, and prints one JSON line.
 
     python bench.py --workload mixed-1.5b | mixed-0.5b | prefix-7b [--token-budget N] [--prompts-first]
 
@@ -463,6 +463,28 @@ def main() -> int:
                 record["serving"] = serving
             except Exception as err:                                  # noqa: BLE001 (whatever it is, it is reported)
                 record["serving"] = {"error": f"{type(err).__name__}: {err}"[:300]}
+            # The same decoding at batch 8 at the sizes of the larger models of the family (all their layers), whose
+            # steps are nearer to what the memory can deliver: tokens/s, a step's time, the bytes it has to read and
+            # their quotient against the published bandwidth, as for the record's own sizes.
+            del model
+            torch.cuda.empty_cache()
+            larger = {}
+            for name, raw in (("1.5b", QWEN2_1_5B), ("7b", QWEN2_7B)):
+                try:
+                    log(f"decode at batch 8 at Qwen2.5-{name.upper()} sizes: {args.steps} timed steps")
+                    other_cfg = Qwen2Config.from_dict(dict(raw))
+                    other = random_model(other_cfg, seed=0, dtype=args.dtype, device="cuda:0")
+                    e, kv = run_decode(other, 8, args.steps, min(args.warmup, 4))
+                    gb = (weight_bytes_per_step(other) + 8 * kv * kv_bytes_per_token(other_cfg, itemsize)) / 1e9
+                    larger[f"decode_b8_{name}"] = round(8 * args.steps / e, 1)
+                    larger[f"decode_b8_{name}_ms"] = round(e / args.steps * 1e3, 4)
+                    larger[f"decode_b8_{name}_gb"] = round(gb, 4)
+                    larger[f"decode_b8_{name}_hbm_frac"] = round(gb / (e / args.steps) / HBM_GBS, 4)
+                    del other
+                    torch.cuda.empty_cache()
+                except Exception as err:                              # noqa: BLE001
+                    larger[f"decode_b8_{name}_error"] = f"{type(err).__name__}: {err}"[:300]
+            record["larger_sizes"] = larger
     print(json.dumps(record), flush=True)
     return 0
 
