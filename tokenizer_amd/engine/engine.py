@@ -260,6 +260,7 @@ class Engine:
                                                 v_pages=v_pages, state=self.pools.states.get(source),
                                                 writes=entry.cache_of is None))
         self.steps = 0
+        self._landing: dict[int, tuple] = {}     # pinned rows and events of `decode_greedy` / `decode_sampled`, by batch size
         self.steps_replayed = 0      # steps (decode steps and others) that replayed a captured graph
         self.graphs_captured = 0
         # Decode steps (one token per request, its logits wanted) and other steps whose shape recurs replay a
@@ -361,8 +362,12 @@ class Engine:
                 if on_step is not None and on_step(k, picked[-1]) is False:
                     break
             return picked
-        landing = [torch.empty(count, dtype=torch.int32).pin_memory() for _ in range(2)]
-        arrived = [torch.cuda.Event(), torch.cuda.Event()]
+        # (Two pinned rows for the ids on their way to the host and an event for each, kept from run to run: pinning
+        # memory costs as much as several steps of a small model.)
+        if count not in self._landing:
+            self._landing[count] = ([torch.empty(count, dtype=torch.int32).pin_memory() for _ in range(2)],
+                                    [torch.cuda.Event(), torch.cuda.Event()])
+        landing, arrived = self._landing[count]
         picked: list[list[int]] = []
         previous: torch.Tensor | None = None           # where the step before left its ids, on the device
         greedy_rows, greedy_mask = None, None          # which requests keep the greedy pick in a run with draws
